@@ -1,0 +1,180 @@
+/*
+ * slime_amd_wq.h - C ABI of libslime_amd_wq.so: MI355X (gfx950) kernels for slime's
+ * low-precision weight-conversion path (bf16 -> block-FP8, bf16 -> group-INT4 pack,
+ * block-FP8 -> bf16).
+ *
+ * Conventions
+ *   - All data pointers are DEVICE pointers on the current HIP device unless a parameter is
+ *     marked "host".  Sizes and strides are in ELEMENTS.  `stream` is a hipStream_t passed
+ *     as void*; NULL selects the default stream.  Launches are asynchronous and are ordered
+ *     on `stream` only; the library keeps no mutable global state and every entry point may
+ *     be called concurrently from several host threads.
+ *   - Return value: 0 on success, a negative WQ_ERR_* for rejected arguments (nothing was
+ *     launched), or a positive hipError_t reported by the launch.  wq_error_string() names any
+ *     of them.
+ *   - FP8 is OCP float8_e4m3fn (bias 7, max 448, 0x7F/0xFF NaN, no infinities).
+ *   - Outputs are bit-identical to the reference torch path for finite inputs.  A NaN in a
+ *     block makes the block's scale NaN and all its codes NaN (0x7F or 0xFF: the sign of a NaN
+ *     code is unspecified, as it is host-dependent in the reference); +-Inf behaves as IEEE
+ *     division does (finite/Inf = signed zero, Inf/Inf = NaN).
+ *
+ * Reference citations are paths inside the THUDM/slime checkout.
+ */
+#ifndef SLIME_AMD_WQ_H
+#define SLIME_AMD_WQ_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define WQ_ABI_VERSION 1
+
+enum {
+    WQ_OK = 0,
+    WQ_ERR_NULL = -1,        /* a required pointer is NULL */
+    WQ_ERR_SHAPE = -2,       /* negative size, zero block, N not a multiple of the group ... */
+    WQ_ERR_MODE = -3,        /* unknown mode / dtype selector */
+    WQ_ERR_UNSUPPORTED = -4, /* valid in the reference but not provided by this library */
+    WQ_ERR_ALIGN = -5,       /* pointer or stride violates a documented alignment requirement */
+    WQ_ERR_TOO_LARGE = -6    /* a count exceeds the launch limits of the entry point */
+};
+
+/* element type selectors */
+enum { WQ_DTYPE_BF16 = 0, WQ_DTYPE_F32 = 1 };
+
+/* FP8 block quant arithmetic.
+ * WQ_FP8_MODE_TORCH  : amax clamped at bf16(1e-12) in bf16, scale = f32(amax)/448, q = f32(x)/scale
+ *                      (IEEE division), clamp +-448, RNE to e4m3fn.
+ *                      Replaces block_fp8, tools/convert_hf_to_fp8.py:41-75.
+ * WQ_FP8_MODE_TRITON : fp32 amax floored at 1e-10f, scale = amax/448, q = f32(x)*(1.0f/scale).
+ *                      Replaces _blockwise_cast_to_fp8_triton,
+ *                      slime/backends/megatron_utils/kernels/fp8_kernel.py:24-58. */
+enum { WQ_FP8_MODE_TORCH = 0, WQ_FP8_MODE_TRITON = 1 };
+
+/* FP8 block dequant arithmetic.
+ * WQ_DEQ_MODE_F32SCALE  : y = bf16(f32(x) * s).  Replaces weight_dequant, tools/fp8_cast_bf16.py:16-41.
+ * WQ_DEQ_MODE_BF16SCALE : y = bf16(f32(x) * f32(bf16(s))).  Replaces the dequant-on-read of
+ *                         slime/backends/megatron_utils/hf_to_megatron/common.py:42-56. */
+enum { WQ_DEQ_MODE_F32SCALE = 0, WQ_DEQ_MODE_BF16SCALE = 1 };
+
+int wq_abi_version(void);
+const char *wq_error_string(int code);
+
+/* ---------------------------------------------------------------------------------------------
+ * bf16 [M,N] -> e4m3fn [M,N] + fp32 scale [ceil(M/bm), ceil(N/bn)], one (bm x bn) block per scale.
+ * x: bf16, element (i,j) at x[i*sx_m + j*sx_n] (any strides, as the reference kernel accepts,
+ * fp8_kernel.py:51,72-75).  y: bytes, element (i,j) at y[i*sy_m + j].  s: contiguous.
+ * Elements of an edge block outside [M,N] count as +0.0 (F.pad, convert_hf_to_fp8.py:51-56).
+ * The 128x128 contiguous-row case runs the single-pass vector kernel; every other block shape
+ * or layout runs a generic kernel with identical results. */
+int wq_fp8_block_quant(const void *x, int64_t M, int64_t N, int64_t sx_m, int64_t sx_n,
+                       void *y, int64_t sy_m, float *s, int bm, int bn, int mode, void *stream);
+
+/* One launch over many tensors (a weight-sync bucket or a whole state dict; the per-parameter
+ * loop it replaces is slime/backends/megatron_utils/update_weight/hf_weight_iterator_direct.py:50-67
+ * calling quantizer_fp8.py:98-118 once per tensor).  `descs` is a DEVICE array of n_desc
+ * descriptors; `tile_start` is a DEVICE array of n_desc+1 int64: exclusive prefix sum of
+ * ceil(M/bm)*ceil(N/bn) over the descriptors; total_tiles = tile_start[n_desc] (passed by value). */
+typedef struct wq_fp8_quant_desc {
+    const void *x;   /* bf16 */
+    void *y;         /* e4m3fn bytes */
+    float *s;        /* fp32 scales, contiguous [ceil(M/bm), ceil(N/bn)] */
+    int64_t M, N;
+    int64_t sx_m, sx_n;
+    int64_t sy_m;
+} wq_fp8_quant_desc;
+
+int wq_fp8_block_quant_grouped(const wq_fp8_quant_desc *descs, const int64_t *tile_start, int n_desc,
+                               int64_t total_tiles, int bm, int bn, int mode, void *stream);
+
+/* Per-row and per-tensor scaling: channel_fp8 / tensor_fp8, tools/convert_hf_to_fp8.py:78-91, and the
+ * per-tensor branch of _quantize_param, quantizer_fp8.py:112-117.  s has M entries (row) or 1 (tensor).
+ * wq_fp8_tensor_quant needs `workspace`: one zero-initialised uint32 in device memory that the call
+ * may overwrite (the cross-workgroup amax). */
+int wq_fp8_row_quant(const void *x, int64_t M, int64_t N, int64_t sx_m, int64_t sx_n,
+                     void *y, int64_t sy_m, float *s, void *stream);
+int wq_fp8_tensor_quant(const void *x, int64_t M, int64_t N, int64_t sx_m, int64_t sx_n,
+                        void *y, int64_t sy_m, float *s, uint32_t *workspace, void *stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * e4m3fn [M,N] contiguous + fp32 scale [ceil(M/block), ceil(N/block)] contiguous -> y [M,N]
+ * contiguous, of type out_dtype: WQ_DTYPE_BF16 (product rounded once, RNE) or WQ_DTYPE_F32 (the fp32
+ * product itself).  Replaces weight_dequant (tools/fp8_cast_bf16.py:31-41), which asserts the same
+ * contiguity and writes torch's default dtype (bf16 in the tool, :45). */
+int wq_fp8_block_dequant(const void *x, const float *s, void *y, int out_dtype, int64_t M, int64_t N,
+                         int block, int mode, void *stream);
+
+typedef struct wq_fp8_dequant_desc {
+    const void *x;
+    const float *s;
+    void *y;
+    int64_t M, N;
+} wq_fp8_dequant_desc;
+
+/* Grouped form: `descs` DEVICE array, `work_start` DEVICE int64[n_desc+1] exclusive prefix sum of
+ * per-tensor work items, where a tensor has ceil(M/WQ_DEQ_ROWS) * ceil(N/WQ_DEQ_COLS) items. */
+#define WQ_DEQ_ROWS 16
+#define WQ_DEQ_COLS 1024
+int wq_fp8_block_dequant_grouped(const wq_fp8_dequant_desc *descs, const int64_t *work_start, int n_desc,
+                                 int64_t total_work, int out_dtype, int block, int mode, void *stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * "Fake" INT4 quantisation: per (bm x bn) group, q = rintf(x/scale) [+ zero] stored in the input
+ * dtype, plus scale and zero point [ceil(M/bm), ceil(N/bn)] in the input dtype.
+ * Replaces fake_int4_quant_cuda(x, block_size, sym),
+ * slime/backends/megatron_utils/kernels/int4_qat/fake_int4_quant_cuda.cu:327-378 (kernels :37-267).
+ * dtype: WQ_DTYPE_BF16 or WQ_DTYPE_F32.  x has any strides; q/scale/zero are contiguous.
+ * Group shapes: (1, 32k), or bn dividing 32 with bm*bn a multiple of 32 (the shapes for which the
+ * reference kernels are well defined); others return WQ_ERR_UNSUPPORTED. */
+int wq_int4_fake_quant(const void *x, int dtype, int64_t M, int64_t N, int64_t sx_m, int64_t sx_n,
+                       int bm, int bn, int sym, void *q, void *scale, void *zero, void *stream);
+
+/* Fused symmetric group quantise + nibble pack: bf16 [M,N] (row stride sx_m, unit column stride,
+ * N % group == 0, group % 32 == 0) -> packed int32 [M, N/8] + bf16 scale [M, N/group], both contiguous.
+ * Word c of row i holds sum_j (q[i,8c+j]+8) << 4j.  Replaces pack_layer(weight, group_size, sym=True),
+ * tools/convert_hf_to_int4_direct.py:123-153 == quantizer_compressed_tensors.py:235-265. */
+int wq_int4_group_quant_pack(const void *x, int64_t M, int64_t N, int64_t sx_m, int group,
+                             int32_t *packed, void *scale, void *stream);
+
+typedef struct wq_int4_pack_desc {
+    const void *x;   /* bf16, contiguous [M,N] */
+    int32_t *packed; /* [M, N/8] */
+    void *scale;     /* bf16 [M, N/group] */
+    int64_t n_groups; /* M * N / group */
+} wq_int4_pack_desc;
+
+/* Grouped form for contiguous tensors (e.g. all experts of a layer).  `descs` DEVICE array;
+ * `work_start` DEVICE int64[n_desc+1] exclusive prefix sum of ceil(n_groups / WQ_INT4_GROUPS_PER_WG). */
+#define WQ_INT4_GROUPS_PER_WG 64
+int wq_int4_group_quant_pack_grouped(const wq_int4_pack_desc *descs, const int64_t *work_start, int n_desc,
+                                     int64_t total_work, int group, void *stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Self-checks and calibration helpers (used by the test-suite and the benchmark, not by callers).
+ *
+ * wq_selftest_fp8_elem: for every bf16 amax a in [amax_lo, amax_hi) (bit patterns, finite) and every
+ * bf16 x with |x| <= max(a, floor), compares the production element function (reciprocal + two FMA
+ * refinement + hardware e4m3 conversion) with plain IEEE division + software RNE conversion.
+ * Writes {mismatch count, first mismatching (a<<16|x)} to out[0..1] (DEVICE uint64[2], zeroed here).
+ * wq_selftest_int4_elem: same for the INT4 element function q = rintf(x/scale).
+ * wq_selftest_cvt_fp8: compares the hardware fp32->e4m3 conversion with the software one for the
+ * fp32 bit patterns [lo, hi) whose magnitude is <= 464 or NaN. */
+int wq_selftest_fp8_elem(uint32_t amax_lo, uint32_t amax_hi, int mode, uint64_t *out, void *stream);
+int wq_selftest_int4_elem(uint32_t amax_lo, uint32_t amax_hi, uint64_t *out, void *stream);
+int wq_selftest_cvt_fp8(uint64_t lo, uint64_t hi, uint64_t *out, void *stream);
+/* wq_selftest_cvt_bf16: hardware fp32->bf16 conversion vs software RNE for the non-NaN fp32 bit
+ * patterns in [lo, hi).  wq_selftest_decode_fp8: hardware e4m3fn->fp32 vs the format definition for all
+ * 256 codes.  Same out[] convention. */
+int wq_selftest_cvt_bf16(uint64_t lo, uint64_t hi, uint64_t *out, void *stream);
+int wq_selftest_decode_fp8(uint64_t *out, void *stream);
+
+/* Plain 16-byte-per-lane copy of n_bytes (multiple of 16, 16-byte aligned): the known-traffic kernel
+ * that hardware counters are scaled against. */
+int wq_copy_bytes(const void *src, void *dst, int64_t n_bytes, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SLIME_AMD_WQ_H */

@@ -1,0 +1,153 @@
+"""ctypes binding of the scalar C oracle (``wq_oracle.c``).  TEST INFRASTRUCTURE ONLY.
+
+Takes and returns CPU torch tensors; all arithmetic happens inside ``libwq_oracle.so``.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_SO = os.path.join(_HERE, "libwq_oracle.so")
+_lib = None
+
+_i64, _int, _vp = ctypes.c_int64, ctypes.c_int, ctypes.c_void_p
+
+
+def build(force: bool = False) -> str:
+    src = os.path.join(_HERE, "wq_oracle.c")
+    if force or not os.path.exists(_SO) or os.path.getmtime(_SO) < os.path.getmtime(src):
+        subprocess.check_call(["make", "-C", _HERE, "-B" if force else "-s"], stdout=subprocess.DEVNULL)
+    return _SO
+
+
+def lib() -> ctypes.CDLL:
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_SO):
+            build()
+        L = ctypes.CDLL(_SO)
+        L.wqo_fp8_block_quant.argtypes = [_vp, _i64, _i64, _i64, _i64, _i64, _i64, _int, _vp, _vp]
+        L.wqo_fp8_channel_quant.argtypes = [_vp, _i64, _i64, _i64, _i64, _vp, _vp]
+        L.wqo_fp8_tensor_quant.argtypes = [_vp, _i64, _i64, _i64, _i64, _vp, _vp]
+        L.wqo_fp8_block_dequant.argtypes = [_vp, _vp, _i64, _i64, _i64, _int, _vp]
+        L.wqo_int4_fake_quant.argtypes = [_vp, _int, _i64, _i64, _i64, _i64, _i64, _i64, _int, _vp, _vp, _vp]
+        L.wqo_int4_pack_layer.argtypes = [_vp, _i64, _i64, _i64, _int, _vp, _vp, _vp]
+        for n in ("wqo_f32_to_e4m3fn_n", "wqo_e4m3fn_to_f32_n", "wqo_f32_to_bf16_n"):
+            getattr(L, n).argtypes = [_vp, _vp, _i64]
+            getattr(L, n).restype = None
+        L.wqo_num_threads.restype = _int
+        L.wqo_set_num_threads.argtypes = [_int]
+        _lib = L
+    return _lib
+
+
+def _check(rc: int, what: str) -> None:
+    if rc != 0:
+        raise RuntimeError(f"{what}: oracle rejected the arguments (code {rc})")
+
+
+def _cpu(t: torch.Tensor) -> torch.Tensor:
+    assert t.device.type == "cpu"
+    return t
+
+
+def _cdiv(a, b):
+    return -(-a // b)
+
+
+def f32_to_e4m3fn(x: torch.Tensor) -> torch.Tensor:
+    x = _cpu(x).contiguous().to(torch.float32)
+    y = torch.empty(x.shape, dtype=torch.uint8)
+    lib().wqo_f32_to_e4m3fn_n(x.data_ptr(), y.data_ptr(), x.numel())
+    return y
+
+
+def e4m3fn_to_f32(x: torch.Tensor) -> torch.Tensor:
+    x = _cpu(x).contiguous().view(torch.uint8)
+    y = torch.empty(x.shape, dtype=torch.float32)
+    lib().wqo_e4m3fn_to_f32_n(x.data_ptr(), y.data_ptr(), x.numel())
+    return y
+
+
+def f32_to_bf16(x: torch.Tensor) -> torch.Tensor:
+    x = _cpu(x).contiguous().to(torch.float32)
+    y = torch.empty(x.shape, dtype=torch.bfloat16)
+    lib().wqo_f32_to_bf16_n(x.data_ptr(), y.data_ptr(), x.numel())
+    return y
+
+
+def fp8_block_quant(w: torch.Tensor, block_size=(128, 128), mode: int = 0):
+    """-> (uint8 [M,N] holding e4m3fn codes, float32 [cdiv(M,bm), cdiv(N,bn)])."""
+    assert _cpu(w).dtype == torch.bfloat16 and w.dim() == 2
+    M, N = w.shape
+    bm, bn = int(block_size[0]), int(block_size[1])
+    y = torch.empty(M, N, dtype=torch.uint8)
+    s = torch.empty(_cdiv(M, bm), _cdiv(N, bn), dtype=torch.float32)
+    _check(lib().wqo_fp8_block_quant(w.data_ptr(), M, N, w.stride(0), w.stride(1), bm, bn, mode,
+                                     y.data_ptr(), s.data_ptr()), "fp8_block_quant")
+    return y, s
+
+
+def fp8_channel_quant(w: torch.Tensor):
+    assert _cpu(w).dtype == torch.bfloat16 and w.dim() == 2
+    M, N = w.shape
+    y = torch.empty(M, N, dtype=torch.uint8)
+    s = torch.empty(M, 1, dtype=torch.float32)
+    _check(lib().wqo_fp8_channel_quant(w.data_ptr(), M, N, w.stride(0), w.stride(1), y.data_ptr(), s.data_ptr()),
+           "fp8_channel_quant")
+    return y, s
+
+
+def fp8_tensor_quant(w: torch.Tensor):
+    assert _cpu(w).dtype == torch.bfloat16 and w.dim() == 2
+    M, N = w.shape
+    y = torch.empty(M, N, dtype=torch.uint8)
+    s = torch.empty(1, dtype=torch.float32)
+    _check(lib().wqo_fp8_tensor_quant(w.data_ptr(), M, N, w.stride(0), w.stride(1), y.data_ptr(), s.data_ptr()),
+           "fp8_tensor_quant")
+    return y, s
+
+
+def fp8_block_dequant(x: torch.Tensor, s: torch.Tensor, block: int = 128, mode: int = 0) -> torch.Tensor:
+    x = _cpu(x).contiguous().view(torch.uint8)
+    s = _cpu(s).contiguous().to(torch.float32)
+    M, N = x.shape
+    assert tuple(s.shape) == (_cdiv(M, block), _cdiv(N, block))
+    y = torch.empty(M, N, dtype=torch.bfloat16)
+    _check(lib().wqo_fp8_block_dequant(x.data_ptr(), s.data_ptr(), M, N, block, mode, y.data_ptr()),
+           "fp8_block_dequant")
+    return y
+
+
+def int4_fake_quant(x: torch.Tensor, block_size, sym: bool):
+    assert _cpu(x).dim() == 2 and x.dtype in (torch.bfloat16, torch.float32)
+    M, N = x.shape
+    bm, bn = int(block_size[0]), int(block_size[1])
+    q = torch.empty(M, N, dtype=x.dtype)
+    sc = torch.empty(_cdiv(M, bm), _cdiv(N, bn), dtype=x.dtype)
+    zp = torch.empty_like(sc)
+    _check(lib().wqo_int4_fake_quant(x.data_ptr(), 0 if x.dtype == torch.bfloat16 else 1, M, N, x.stride(0),
+                                     x.stride(1), bm, bn, int(sym), q.data_ptr(), sc.data_ptr(), zp.data_ptr()),
+           "int4_fake_quant")
+    return q, sc, zp
+
+
+def int4_pack_layer(w: torch.Tensor, group_size: int, sym: bool = True):
+    w = _cpu(w).contiguous()
+    assert w.dtype == torch.bfloat16 and w.dim() == 2
+    M, N = w.shape
+    packed = torch.empty(M, N // 8, dtype=torch.int32)
+    sc = torch.empty(M, N // group_size, dtype=torch.bfloat16)
+    pzp = None if sym else torch.empty(N // group_size, M // 8, dtype=torch.int32)
+    _check(lib().wqo_int4_pack_layer(w.data_ptr(), M, N, group_size, int(sym), packed.data_ptr(), sc.data_ptr(),
+                                     None if sym else pzp.data_ptr()), "int4_pack_layer")
+    return packed, sc, pzp
+
+
+def num_threads() -> int:
+    return lib().wqo_num_threads()

@@ -1,0 +1,39 @@
+"""slime_amd - MI355X-native low-precision weight conversion for slime.
+
+bf16 -> block-FP8 (e4m3fn, 128x128 blocks, fp32 ``weight_scale_inv``), bf16 -> group-wise INT4
+(``weight_packed`` / ``weight_scale`` / ``weight_shape``) and block-FP8 -> bf16, behind the reference's
+own function names.  Everything computes in hand-written gfx950 HIP kernels reached through the C ABI
+of ``slime_amd/lib/libslime_amd_wq.so``; there is no CPU or pure-torch fallback.
+"""
+
+from . import _lib
+from .fp8 import (
+    Fp8DequantPlan,
+    Fp8QuantPlan,
+    block_fp8,
+    block_fp8_many,
+    blockwise_cast_to_fp8_triton,
+    channel_fp8,
+    quant_fp8,
+    tensor_fp8,
+    weight_dequant,
+    weight_dequant_bf16_scale,
+)
+from .int4 import Int4PackPlan, fake_int4_quant_cuda, pack_layer, pack_to_int32, quantize
+from .processors import (
+    _quantize_param,
+    quantize_params,
+    quantize_params_compressed_tensors,
+    quantize_params_fp8,
+)
+
+# the injectable `quantize_weight(weight, (128, 128)) -> (qweight, scale)` hook of the reference's
+# alignment forwards (slime/backends/megatron_utils/alignment/deepgemm_moe_forward.py:1145) is this function
+quantize_weight = blockwise_cast_to_fp8_triton
+
+__all__ = [
+    "Fp8DequantPlan", "Fp8QuantPlan", "Int4PackPlan", "block_fp8", "block_fp8_many",
+    "blockwise_cast_to_fp8_triton", "channel_fp8", "fake_int4_quant_cuda", "pack_layer", "pack_to_int32",
+    "quant_fp8", "quantize", "quantize_params", "quantize_params_compressed_tensors", "quantize_params_fp8",
+    "quantize_weight", "tensor_fp8", "weight_dequant", "weight_dequant_bf16_scale", "_quantize_param",
+]

@@ -1,0 +1,245 @@
+// Device-side helpers shared by the gfx950 weight-conversion kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/slime_amd_wq.h"
+
+#define WQ_EXPORT extern "C" __attribute__((visibility("default")))
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint16_t u16x2 __attribute__((ext_vector_type(2)));
+
+namespace wq {
+
+constexpr float kFp8Max = 448.0f;
+constexpr uint32_t kBf16Floor1em12 = 0x2B8Du;  // bf16(1e-12): the clamp bound after torch rounds it to bf16
+constexpr uint32_t kBf16Inf = 0x7F80u;
+
+__device__ __forceinline__ float u2f(uint32_t u) { return __builtin_bit_cast(float, u); }
+__device__ __forceinline__ uint32_t f2u(float f) { return __builtin_bit_cast(uint32_t, f); }
+
+// A dword holds two bf16: element 2k in the low half, 2k+1 in the high half.
+__device__ __forceinline__ float bf16lo(uint32_t w) { return u2f(w << 16); }
+__device__ __forceinline__ float bf16hi(uint32_t w) { return u2f(w & 0xFFFF0000u); }
+
+// Magnitude bits of a bf16 order exactly like the values, so the block amax is an integer max;
+// a NaN (> 0x7F80) wins the max and so propagates like torch.max does.
+__device__ __forceinline__ uint32_t pk_absmax(uint32_t acc, uint32_t w)
+{
+    u16x2 a = __builtin_bit_cast(u16x2, acc);
+    u16x2 b = __builtin_bit_cast(u16x2, w & 0x7FFF7FFFu);
+    return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(a, b));
+}
+__device__ __forceinline__ uint32_t pk_fold(uint32_t acc) { return max(acc & 0xFFFFu, acc >> 16); }
+
+// fp32 -> bf16, round to nearest even, NaN -> 0x7FC0 (sign dropped).
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f)
+{
+    uint32_t u = f2u(f);
+    if ((u & 0x7FFFFFFFu) > 0x7F800000u) return 0x7FC0u;
+    return (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
+}
+
+// Software fp32 -> e4m3fn, RNE, non-saturating (|f| > 464, Inf, NaN -> NaN code, sign kept).
+// Used on the slow paths (NaN/Inf blocks, generic layouts) and as the checker of the hardware
+// conversion in the self-tests.
+__device__ __forceinline__ uint32_t f32_to_e4m3fn_sw(float f)
+{
+    uint32_t u = f2u(f);
+    uint32_t sign = (u >> 24) & 0x80u;
+    uint32_t a = u & 0x7FFFFFFFu;
+    uint32_t code;
+    if (a >= 0x43F00000u) {
+        code = 0x7Fu;
+    } else if (a < 0x3C800000u) {
+        // k * 2^-9, k = RNE(|f| * 512) in 0..8; adding 2^23 leaves k in the low mantissa bits
+        float t = u2f(a) * 512.0f + 8388608.0f;
+        code = f2u(t) & 0xFu;
+    } else {
+        uint32_t c = ((a >> 20) & 0x7FFu) - ((127u - 7u) << 3);
+        uint32_t rem = a & 0xFFFFFu;
+        if (rem > 0x80000u || (rem == 0x80000u && (c & 1u))) c += 1u;
+        code = c;
+    }
+    return sign | code;
+}
+
+// Hardware conversion of two fp32 to two e4m3fn bytes in the low 16 bits (v_cvt_pk_fp8_f32;
+// OCP encoding on gfx950).  Inputs must already be within +-448*(1+2^-20): the production
+// paths guarantee it, so saturation behaviour is never relied on.
+__device__ __forceinline__ uint32_t cvt_pk_fp8_lo(float a, float b, uint32_t old)
+{
+    return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(a, b, (int)old, false);
+}
+__device__ __forceinline__ uint32_t cvt_pk_fp8_hi(float a, float b, uint32_t old)
+{
+    return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(a, b, (int)old, true);
+}
+
+// ---- 16-lane (DPP row) all-reduce max.  After it every lane of the row holds the row max.
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_u32(uint32_t v)
+{
+    return (uint32_t)__builtin_amdgcn_update_dpp((int)v, (int)v, CTRL, 0xF, 0xF, false);
+}
+__device__ __forceinline__ uint32_t row16_max_u32(uint32_t v)
+{
+    v = max(v, dpp_u32<0xB1>(v));   // quad_perm [1,0,3,2]
+    v = max(v, dpp_u32<0x4E>(v));   // quad_perm [2,3,0,1]
+    v = max(v, dpp_u32<0x141>(v));  // row_half_mirror
+    v = max(v, dpp_u32<0x140>(v));  // row_mirror
+    return v;
+}
+__device__ __forceinline__ float row16_max_f32(float v)
+{
+    v = fmaxf(v, u2f(dpp_u32<0xB1>(f2u(v))));
+    v = fmaxf(v, u2f(dpp_u32<0x4E>(f2u(v))));
+    v = fmaxf(v, u2f(dpp_u32<0x141>(f2u(v))));
+    v = fmaxf(v, u2f(dpp_u32<0x140>(f2u(v))));
+    return v;
+}
+__device__ __forceinline__ float row16_min_f32(float v)
+{
+    v = fminf(v, u2f(dpp_u32<0xB1>(f2u(v))));
+    v = fminf(v, u2f(dpp_u32<0x4E>(f2u(v))));
+    v = fminf(v, u2f(dpp_u32<0x141>(f2u(v))));
+    v = fminf(v, u2f(dpp_u32<0x140>(f2u(v))));
+    return v;
+}
+__device__ __forceinline__ uint32_t wave64_max_u32(uint32_t v)
+{
+    v = row16_max_u32(v);
+    v = max(v, (uint32_t)__shfl_xor((int)v, 16));
+    v = max(v, (uint32_t)__shfl_xor((int)v, 32));
+    return v;
+}
+
+// ---- scale rules -------------------------------------------------------------------------
+
+// mode TORCH: amax is a bf16 magnitude bit pattern (possibly NaN/Inf).
+__device__ __forceinline__ float fp8_scale_torch(uint32_t amax_bf16_bits)
+{
+    uint32_t a = amax_bf16_bits < kBf16Floor1em12 ? kBf16Floor1em12 : amax_bf16_bits;
+    return u2f(a << 16) / kFp8Max;
+}
+// mode TRITON: fp32 amax floored at 1e-10f.
+__device__ __forceinline__ float fp8_scale_triton(uint32_t amax_bf16_bits)
+{
+    float a = u2f(amax_bf16_bits << 16);
+    a = (a != a) ? a : fmaxf(a, 1e-10f);
+    return a / kFp8Max;
+}
+
+// Per-block constants of the element function.
+struct Fp8BlockParams {
+    float scale;  // value stored to the scale tensor
+    float rcp;    // correctly rounded 1/scale
+    bool fast;    // amax finite: the refinement below reproduces IEEE x/scale exactly
+};
+
+template <int MODE>
+__device__ __forceinline__ Fp8BlockParams fp8_block_params(uint32_t amax_bf16_bits)
+{
+    Fp8BlockParams p;
+    p.scale = MODE == WQ_FP8_MODE_TORCH ? fp8_scale_torch(amax_bf16_bits) : fp8_scale_triton(amax_bf16_bits);
+    p.rcp = 1.0f / p.scale;
+    p.fast = amax_bf16_bits < kBf16Inf;
+    return p;
+}
+
+// q = RN(x / scale) without a per-element division: q0 = RN(x*r), rem = x - q0*scale (exact in an
+// FMA), q = RN(q0 + rem*r).  With r the correctly rounded reciprocal this is the correctly rounded
+// quotient for every (x, scale) pair the block quantiser can produce; wq_selftest_fp8_elem checks the
+// whole domain against the IEEE division.  An exact zero loses its sign here (+0 + -0 = +0); callers
+// restore the sign bit on the fp8 code.
+__device__ __forceinline__ float div_by_scale(float x, float scale, float rcp)
+{
+    float q0 = x * rcp;
+    float rem = __builtin_fmaf(-q0, scale, x);
+    return __builtin_fmaf(rem, rcp, q0);
+}
+
+// mode TORCH slow/reference element function: IEEE division, NaN-propagating clamp, software RNE.
+__device__ __forceinline__ uint32_t fp8_elem_exact_torch(float x, float scale)
+{
+    float q = x / scale;
+    if (q == q) q = fminf(fmaxf(q, -kFp8Max), kFp8Max);
+    return f32_to_e4m3fn_sw(q);
+}
+__device__ __forceinline__ uint32_t fp8_elem_exact_triton(float x, float s_inv)
+{
+    float q = x * s_inv;
+    if (q == q) q = fminf(fmaxf(q, -kFp8Max), kFp8Max);
+    return f32_to_e4m3fn_sw(q);
+}
+
+// Sign bits of the four bf16 in (w0, w1) moved to bits 7, 15, 23, 31.
+__device__ __forceinline__ uint32_t bf16x4_signs_to_bytes(uint32_t w0, uint32_t w1)
+{
+    // bytes picked: w0.b1, w0.b3, w1.b1, w1.b3  (v_perm_b32: selector bytes 0-3 = second operand)
+    return __builtin_amdgcn_perm(w1, w0, 0x07050301u) & 0x80808080u;
+}
+
+// Four bf16 (two dwords) -> four e4m3fn bytes, production path (block amax finite).
+template <int MODE>
+__device__ __forceinline__ uint32_t fp8_quant4_fast(uint32_t w0, uint32_t w1, const Fp8BlockParams& p)
+{
+    float q0, q1, q2, q3;
+    if (MODE == WQ_FP8_MODE_TORCH) {
+        q0 = div_by_scale(bf16lo(w0), p.scale, p.rcp);
+        q1 = div_by_scale(bf16hi(w0), p.scale, p.rcp);
+        q2 = div_by_scale(bf16lo(w1), p.scale, p.rcp);
+        q3 = div_by_scale(bf16hi(w1), p.scale, p.rcp);
+    } else {
+        q0 = bf16lo(w0) * p.rcp;
+        q1 = bf16hi(w0) * p.rcp;
+        q2 = bf16lo(w1) * p.rcp;
+        q3 = bf16hi(w1) * p.rcp;
+    }
+    // |q| <= 448*(1+2^-22): clamping to +-448 cannot change the RNE result (next boundary is 464),
+    // so the clamp of the reference is a no-op here and is skipped.
+    uint32_t r = cvt_pk_fp8_lo(q0, q1, 0u);
+    r = cvt_pk_fp8_hi(q2, q3, r);
+    if (MODE == WQ_FP8_MODE_TORCH) r |= bf16x4_signs_to_bytes(w0, w1);
+    return r;
+}
+
+template <int MODE>
+__device__ __forceinline__ uint32_t fp8_quant1_exact(float x, const Fp8BlockParams& p)
+{
+    return MODE == WQ_FP8_MODE_TORCH ? fp8_elem_exact_torch(x, p.scale) : fp8_elem_exact_triton(x, p.rcp);
+}
+
+template <int MODE>
+__device__ __forceinline__ uint32_t fp8_quant4_exact(uint32_t w0, uint32_t w1, const Fp8BlockParams& p)
+{
+    return fp8_quant1_exact<MODE>(bf16lo(w0), p) | (fp8_quant1_exact<MODE>(bf16hi(w0), p) << 8) |
+           (fp8_quant1_exact<MODE>(bf16lo(w1), p) << 16) | (fp8_quant1_exact<MODE>(bf16hi(w1), p) << 24);
+}
+
+// ---- INT4 ---------------------------------------------------------------------------------
+
+__device__ __forceinline__ float int4_scale_sym(float amax) { return fmaxf(amax * (1.0f / 7.0f), 1e-5f); }
+
+// Host-side launch helpers.
+inline int64_t cdiv64(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// Grid for n workgroups of 256 threads, addressed in the kernels as blockIdx.x + blockIdx.y * gridDim.x.
+// x stays at or below 2^22 workgroups so that gridDim.x * blockDim.x fits 32 bits.
+inline dim3 grid_for_items(int64_t n)
+{
+    const int64_t lim = 1 << 22;
+    if (n <= lim) return dim3((unsigned)(n > 0 ? n : 1), 1, 1);
+    return dim3((unsigned)lim, (unsigned)cdiv64(n, lim), 1);
+}
+
+}  // namespace wq
+
+#define WQ_LAUNCH_CHECK()                              \
+    do {                                               \
+        hipError_t e_ = hipGetLastError();             \
+        if (e_ != hipSuccess) return (int)e_;          \
+    } while (0)

@@ -1,0 +1,315 @@
+// bf16 -> block-FP8 (e4m3fn) quantisation for gfx950.
+//
+// Vector kernel (128x128 blocks, unit column stride, 16-byte aligned rows): one 256-thread
+// workgroup owns one block.  Each lane issues eight 16-byte loads (8 bf16 each, rows rb+16*i), so a
+// wavefront load covers four 256-byte row segments and the whole 32 KiB block is in flight before
+// the first use.  The block lives in registers from then on: amax is an integer max over the bf16
+// magnitude bits (packed 16-bit max), reduced over 16 lanes with DPP and across the workgroup
+// through 64 bytes of LDS; the scale is computed once; every element is divided with a
+// reciprocal + two FMA refinement that equals the IEEE quotient, converted with v_cvt_pk_fp8_f32
+// and stored as 8-byte pieces.  HBM traffic is exactly one read of x, one write of y and 4 bytes of
+// scale per block.
+//
+// Generic kernel: any block shape / strides / alignment, one workgroup per block, two passes over
+// the block (the second one hits L2), exact IEEE division and software conversion.
+
+#include "wq_common.h"
+
+namespace wq {
+
+struct Fp8QuantArgs {
+    wq_fp8_quant_desc d;  // single-tensor launch: descriptor travels in the kernel arguments
+    const wq_fp8_quant_desc* descs;
+    const int64_t* tile_start;
+    int32_t n_desc;
+    int32_t bm, bn;
+};
+
+__device__ __forceinline__ bool desc_vector_ok(const wq_fp8_quant_desc& d)
+{
+    // 128 rows of either operand must span fewer than 2^31 bytes: lane offsets are 32-bit
+    return d.sx_n == 1 && (d.sx_m & 7) == 0 && (d.N & 7) == 0 && (d.sy_m & 7) == 0 &&
+           ((uintptr_t)d.x & 15) == 0 && ((uintptr_t)d.y & 7) == 0 && d.sx_m >= 0 && d.sx_m < (1 << 22) &&
+           d.sy_m >= 0 && d.sy_m < (1 << 22);
+}
+
+// Finds the descriptor that owns flat tile `t`: largest i with tile_start[i] <= t.
+__device__ __forceinline__ int find_desc(const int64_t* __restrict__ start, int n, int64_t t)
+{
+    int lo = 0, hi = n;  // invariant: start[lo] <= t < start[hi]
+    while (hi - lo > 1) {
+        int mid = (lo + hi) >> 1;
+        if (start[mid] <= t) lo = mid; else hi = mid;
+    }
+    return lo;
+}
+
+template <int MODE>
+__device__ __forceinline__ void quant_tile_vec128(const wq_fp8_quant_desc& d, int64_t tm, int64_t tn, int kt,
+                                                  uint32_t* lds)
+{
+    const int t = threadIdx.x;
+    const int cc = t & 15;  // which 8-element piece of the 128 columns
+    const int rb = t >> 4;  // 0..15
+    // Workgroup-uniform tile origin (scalar registers) + 32-bit per-lane byte offsets.
+    const char* xt = (const char*)d.x + (tm * 128 * d.sx_m + tn * 128) * 2;
+    char* yt = (char*)d.y + (tm * 128 * d.sy_m + tn * 128);
+    const uint32_t xstep = (uint32_t)d.sx_m * 32u, ystep = (uint32_t)d.sy_m * 16u;  // 16 rows, in bytes
+    const uint32_t xoff = (uint32_t)rb * (uint32_t)d.sx_m * 2u + (uint32_t)cc * 16u;
+    const uint32_t yoff = (uint32_t)rb * (uint32_t)d.sy_m + (uint32_t)cc * 8u;
+    const int rows_left = (int)min((int64_t)128, d.M - tm * 128) - rb;  // row rb+16*i is valid iff 16*i < rows_left
+    const bool col_ok = tn * 128 + cc * 8 < d.N;
+    const bool full = (tm * 128 + 128 <= d.M) && (tn * 128 + 128 <= d.N);
+
+    u32x4 v[8];
+    if (full) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = __builtin_nontemporal_load((const u32x4*)(xt + (xoff + i * xstep)));
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            v[i] = (u32x4){0u, 0u, 0u, 0u};
+            if (col_ok && 16 * i < rows_left) v[i] = __builtin_nontemporal_load((const u32x4*)(xt + (xoff + i * xstep)));
+        }
+    }
+
+    uint32_t m = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        m = pk_absmax(m, v[i].x);
+        m = pk_absmax(m, v[i].y);
+        m = pk_absmax(m, v[i].z);
+        m = pk_absmax(m, v[i].w);
+    }
+    m = row16_max_u32(pk_fold(m));
+    if (cc == 0) lds[rb] = m;
+    __syncthreads();
+    {
+        const u32x4* l4 = (const u32x4*)lds;
+        u32x4 a = l4[0], b = l4[1], c = l4[2], e = l4[3];
+        uint32_t m0 = max(max(a.x, a.y), max(a.z, a.w));
+        uint32_t m1 = max(max(b.x, b.y), max(b.z, b.w));
+        uint32_t m2 = max(max(c.x, c.y), max(c.z, c.w));
+        uint32_t m3 = max(max(e.x, e.y), max(e.z, e.w));
+        m = max(max(m0, m1), max(m2, m3));
+    }
+
+    const Fp8BlockParams p = fp8_block_params<MODE>(m);
+    if (t == 0) d.s[tm * kt + tn] = p.scale;
+
+    if (p.fast) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            u32x2 o;
+            o.x = fp8_quant4_fast<MODE>(v[i].x, v[i].y, p);
+            o.y = fp8_quant4_fast<MODE>(v[i].z, v[i].w, p);
+            if (full || (col_ok && 16 * i < rows_left)) __builtin_nontemporal_store(o, (u32x2*)(yt + (yoff + i * ystep)));
+        }
+    } else {
+        // NaN/Inf block (rare): literal arithmetic.  The rows are re-read so that the register copy of
+        // the block is never indexed dynamically.
+#pragma nounroll
+        for (int i = 0; i < 8; ++i) {
+            if (!(full || (col_ok && 16 * i < rows_left))) continue;
+            const u32x4 w = *(const u32x4*)(xt + (xoff + i * xstep));
+            u32x2 o;
+            o.x = fp8_quant4_exact<MODE>(w.x, w.y, p);
+            o.y = fp8_quant4_exact<MODE>(w.z, w.w, p);
+            *(u32x2*)(yt + (yoff + i * ystep)) = o;
+        }
+    }
+}
+
+template <int MODE>
+__device__ __forceinline__ void quant_tile_generic(const wq_fp8_quant_desc& d, int64_t tm, int64_t tn, int kt,
+                                                   int bm, int bn, uint32_t* lds)
+{
+    const int64_t r0 = tm * bm, c0 = tn * bn;
+    const int rows = (int)min((int64_t)bm, d.M - r0), cols = (int)min((int64_t)bn, d.N - c0);
+    const int n = rows * cols;
+    const uint16_t* x = (const uint16_t*)d.x;
+    uint32_t m = 0;
+    for (int e = threadIdx.x; e < n; e += blockDim.x) {
+        int i = e / cols, j = e - i * cols;
+        m = max(m, (uint32_t)x[(r0 + i) * d.sx_m + (c0 + j) * d.sx_n] & 0x7FFFu);
+    }
+    m = wave64_max_u32(m);
+    if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6] = m;
+    __syncthreads();
+    m = max(max(lds[0], lds[1]), max(lds[2], lds[3]));
+    const Fp8BlockParams p = fp8_block_params<MODE>(m);
+    if (threadIdx.x == 0) d.s[tm * kt + tn] = p.scale;
+    uint8_t* y = (uint8_t*)d.y;
+    for (int e = threadIdx.x; e < n; e += blockDim.x) {
+        int i = e / cols, j = e - i * cols;
+        float xv = u2f((uint32_t)x[(r0 + i) * d.sx_m + (c0 + j) * d.sx_n] << 16);
+        y[(r0 + i) * d.sy_m + (c0 + j)] = (uint8_t)fp8_quant1_exact<MODE>(xv, p);
+    }
+}
+
+template <int MODE, bool GROUPED>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 8))) void fp8_block_quant_kernel(const Fp8QuantArgs a, const int64_t total_tiles)
+{
+    __shared__ __attribute__((aligned(16))) uint32_t lds[16];
+    const int64_t tile = (int64_t)blockIdx.x + (int64_t)blockIdx.y * gridDim.x;
+    if (tile >= total_tiles) return;  // uniform per workgroup
+
+    wq_fp8_quant_desc d;
+    int64_t local = tile;
+    if (GROUPED) {
+        const int di = find_desc(a.tile_start, a.n_desc, tile);
+        d = a.descs[di];
+        local = tile - a.tile_start[di];
+    } else {
+        d = a.d;
+    }
+    const int kt = (int)((d.N + a.bn - 1) / a.bn);
+    const int64_t tm = local / kt, tn = local - tm * kt;
+    if (a.bm == 128 && a.bn == 128 && desc_vector_ok(d))
+        quant_tile_vec128<MODE>(d, tm, tn, kt, lds);
+    else
+        quant_tile_generic<MODE>(d, tm, tn, kt, a.bm, a.bn, lds);
+}
+
+// ---- per-row (channel) and per-tensor scaling -------------------------------------------------
+
+// One workgroup per row: amax over the row, then quantise.  Second pass re-reads the row (L2).
+__global__ __launch_bounds__(256) void fp8_row_quant_kernel(const uint16_t* __restrict__ x, int64_t M, int64_t N,
+                                                           int64_t sx_m, int64_t sx_n, uint8_t* __restrict__ y,
+                                                           int64_t sy_m, float* __restrict__ s)
+{
+    __shared__ uint32_t lds[4];
+    const int64_t row = (int64_t)blockIdx.x + (int64_t)blockIdx.y * gridDim.x;
+    if (row >= M) return;
+    const uint16_t* xr = x + row * sx_m;
+    uint32_t m = 0;
+    for (int64_t j = threadIdx.x; j < N; j += 256) m = max(m, (uint32_t)xr[j * sx_n] & 0x7FFFu);
+    m = wave64_max_u32(m);
+    if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6] = m;
+    __syncthreads();
+    m = max(max(lds[0], lds[1]), max(lds[2], lds[3]));
+    const Fp8BlockParams p = fp8_block_params<WQ_FP8_MODE_TORCH>(m);
+    if (threadIdx.x == 0) s[row] = p.scale;
+    uint8_t* yr = y + row * sy_m;
+    for (int64_t j = threadIdx.x; j < N; j += 256)
+        yr[j] = (uint8_t)fp8_elem_exact_torch(u2f((uint32_t)xr[j * sx_n] << 16), p.scale);
+}
+
+__global__ __launch_bounds__(256) void fp8_tensor_amax_kernel(const uint16_t* __restrict__ x, int64_t M, int64_t N,
+                                                             int64_t sx_m, int64_t sx_n, uint32_t* __restrict__ ws)
+{
+    __shared__ uint32_t lds[4];
+    const int64_t total = M * N;
+    uint32_t m = 0;
+    for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < total; e += (int64_t)gridDim.x * 256) {
+        int64_t i = e / N, j = e - i * N;
+        m = max(m, (uint32_t)x[i * sx_m + j * sx_n] & 0x7FFFu);
+    }
+    m = wave64_max_u32(m);
+    if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6] = m;
+    __syncthreads();
+    if (threadIdx.x == 0) atomicMax(ws, max(max(lds[0], lds[1]), max(lds[2], lds[3])));
+}
+
+__global__ __launch_bounds__(256) void fp8_tensor_apply_kernel(const uint16_t* __restrict__ x, int64_t M, int64_t N,
+                                                              int64_t sx_m, int64_t sx_n, uint8_t* __restrict__ y,
+                                                              int64_t sy_m, float* __restrict__ s,
+                                                              const uint32_t* __restrict__ ws)
+{
+    const Fp8BlockParams p = fp8_block_params<WQ_FP8_MODE_TORCH>(*ws);
+    if (blockIdx.x == 0 && threadIdx.x == 0) s[0] = p.scale;
+    const int64_t total = M * N;
+    for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < total; e += (int64_t)gridDim.x * 256) {
+        int64_t i = e / N, j = e - i * N;
+        // The reference divides a bf16 tensor by a 0-dim fp32 tensor, which torch evaluates as a bf16
+        // result: the fp32 quotient is rounded to bf16 before the clamp and the e4m3 cast.
+        float q = u2f((uint32_t)x[i * sx_m + j * sx_n] << 16) / p.scale;
+        q = u2f(f32_to_bf16_bits(q) << 16);
+        if (q == q) q = fminf(fmaxf(q, -kFp8Max), kFp8Max);
+        y[i * sy_m + j] = (uint8_t)f32_to_e4m3fn_sw(q);
+    }
+}
+
+static int check_desc_host(const void* x, int64_t M, int64_t N, const void* y, const float* s, int bm, int bn, int mode)
+{
+    if (M < 0 || N < 0 || bm <= 0 || bn <= 0) return WQ_ERR_SHAPE;
+    if (mode != WQ_FP8_MODE_TORCH && mode != WQ_FP8_MODE_TRITON) return WQ_ERR_MODE;
+    if (M > 0 && N > 0 && (!x || !y || !s)) return WQ_ERR_NULL;
+    if ((int64_t)bm * bn > (1 << 30)) return WQ_ERR_TOO_LARGE;
+    return WQ_OK;
+}
+
+}  // namespace wq
+
+using namespace wq;
+
+WQ_EXPORT int wq_fp8_block_quant(const void* x, int64_t M, int64_t N, int64_t sx_m, int64_t sx_n, void* y,
+                                 int64_t sy_m, float* s, int bm, int bn, int mode, void* stream)
+{
+    int rc = check_desc_host(x, M, N, y, s, bm, bn, mode);
+    if (rc) return rc;
+    if (M == 0 || N == 0) return WQ_OK;
+    Fp8QuantArgs a{};
+    a.d = wq_fp8_quant_desc{x, y, s, M, N, sx_m, sx_n, sy_m};
+    a.bm = bm;
+    a.bn = bn;
+    const int64_t tiles = cdiv64(M, bm) * cdiv64(N, bn);
+    hipStream_t st = (hipStream_t)stream;
+    if (mode == WQ_FP8_MODE_TORCH)
+        fp8_block_quant_kernel<WQ_FP8_MODE_TORCH, false><<<grid_for_items(tiles), 256, 0, st>>>(a, tiles);
+    else
+        fp8_block_quant_kernel<WQ_FP8_MODE_TRITON, false><<<grid_for_items(tiles), 256, 0, st>>>(a, tiles);
+    WQ_LAUNCH_CHECK();
+    return WQ_OK;
+}
+
+WQ_EXPORT int wq_fp8_block_quant_grouped(const wq_fp8_quant_desc* descs, const int64_t* tile_start, int n_desc,
+                                         int64_t total_tiles, int bm, int bn, int mode, void* stream)
+{
+    if (n_desc < 0 || total_tiles < 0 || bm <= 0 || bn <= 0) return WQ_ERR_SHAPE;
+    if (mode != WQ_FP8_MODE_TORCH && mode != WQ_FP8_MODE_TRITON) return WQ_ERR_MODE;
+    if (n_desc == 0 || total_tiles == 0) return WQ_OK;
+    if (!descs || !tile_start) return WQ_ERR_NULL;
+    if ((int64_t)bm * bn > (1 << 30)) return WQ_ERR_TOO_LARGE;
+    Fp8QuantArgs a{};
+    a.descs = descs;
+    a.tile_start = tile_start;
+    a.n_desc = n_desc;
+    a.bm = bm;
+    a.bn = bn;
+    hipStream_t st = (hipStream_t)stream;
+    if (mode == WQ_FP8_MODE_TORCH)
+        fp8_block_quant_kernel<WQ_FP8_MODE_TORCH, true><<<grid_for_items(total_tiles), 256, 0, st>>>(a, total_tiles);
+    else
+        fp8_block_quant_kernel<WQ_FP8_MODE_TRITON, true><<<grid_for_items(total_tiles), 256, 0, st>>>(a, total_tiles);
+    WQ_LAUNCH_CHECK();
+    return WQ_OK;
+}
+
+WQ_EXPORT int wq_fp8_row_quant(const void* x, int64_t M, int64_t N, int64_t sx_m, int64_t sx_n, void* y,
+                               int64_t sy_m, float* s, void* stream)
+{
+    if (M < 0 || N < 0) return WQ_ERR_SHAPE;
+    if (M == 0) return WQ_OK;
+    if (!s || (N > 0 && (!x || !y))) return WQ_ERR_NULL;
+    fp8_row_quant_kernel<<<grid_for_items(M), 256, 0, (hipStream_t)stream>>>((const uint16_t*)x, M, N, sx_m, sx_n,
+                                                                      (uint8_t*)y, sy_m, s);
+    WQ_LAUNCH_CHECK();
+    return WQ_OK;
+}
+
+WQ_EXPORT int wq_fp8_tensor_quant(const void* x, int64_t M, int64_t N, int64_t sx_m, int64_t sx_n, void* y,
+                                  int64_t sy_m, float* s, uint32_t* workspace, void* stream)
+{
+    if (M < 0 || N < 0) return WQ_ERR_SHAPE;
+    if (!s || !workspace || (M * N > 0 && (!x || !y))) return WQ_ERR_NULL;
+    const int64_t total = M * N;
+    int blocks = (int)min((int64_t)(256 * 16), max((int64_t)1, cdiv64(total, 256 * 8)));
+    hipStream_t st = (hipStream_t)stream;
+    fp8_tensor_amax_kernel<<<blocks, 256, 0, st>>>((const uint16_t*)x, M, N, sx_m, sx_n, workspace);
+    WQ_LAUNCH_CHECK();
+    fp8_tensor_apply_kernel<<<blocks, 256, 0, st>>>((const uint16_t*)x, M, N, sx_m, sx_n, (uint8_t*)y, sy_m, s,
+                                                   workspace);
+    WQ_LAUNCH_CHECK();
+    return WQ_OK;
+}

@@ -1,0 +1,285 @@
+// Group-wise INT4 quantisation for gfx950.
+//
+// int4_pack_kernel: fused symmetric quantise + nibble pack for bf16 rows.  A group of G = 8*L
+// elements (L = 4, 8 or 16 lanes; G = 32, 64, 128) is owned by L adjacent lanes: one 16-byte load
+// per lane brings the whole group into registers, the amax is an integer max over bf16 magnitude
+// bits reduced with DPP inside the 16-lane row, the scale is max(amax * (1/7), 1e-5) in fp32, every
+// element is divided exactly (reciprocal + two FMA), rounded half-to-even by a magic-constant add
+// and the eight 4-bit codes of the lane are assembled into the one int32 the lane stores.  One HBM
+// read of x, one write of the packed words, one bf16 scale per group.  The dequantise /
+// re-quantise chain that the reference runs between its fake-quant kernel and the packing is the
+// identity on the integer codes for every reachable (code, bf16 scale) pair, so it is not executed.
+//
+// int4_fake_quant_kernel: the general "fake quant" form (codes, scale and zero point written in the
+// input dtype) for any supported group shape, strides, bf16 or fp32, symmetric or asymmetric.
+
+#include "wq_common.h"
+
+namespace wq {
+
+constexpr int kGroupsPerWg = WQ_INT4_GROUPS_PER_WG;
+
+struct Int4PackArgs {
+    wq_int4_pack_desc d;
+    const wq_int4_pack_desc* descs;
+    const int64_t* work_start;
+    int32_t n_desc;
+};
+
+__device__ __forceinline__ int find_desc_i4(const int64_t* __restrict__ start, int n, int64_t t)
+{
+    int lo = 0, hi = n;
+    while (hi - lo > 1) {
+        int mid = (lo + hi) >> 1;
+        if (start[mid] <= t) lo = mid; else hi = mid;
+    }
+    return lo;
+}
+
+template <int L>
+__device__ __forceinline__ uint32_t lanes_max_u32(uint32_t v)
+{
+    v = max(v, dpp_u32<0xB1>(v));
+    v = max(v, dpp_u32<0x4E>(v));
+    if (L >= 8) v = max(v, dpp_u32<0x141>(v));
+    if (L >= 16) v = max(v, dpp_u32<0x140>(v));
+    return v;
+}
+
+// rintf(q) + 8 in the low four bits: 12582912 = 1.5 * 2^23 makes the add round q to an integer
+// (half to even) and leaves it, offset by 8, in the low mantissa bits.
+__device__ __forceinline__ uint32_t nibble_of(float q) { return f2u(q + 12582920.0f) & 0xFu; }
+
+__device__ __forceinline__ uint32_t pack8_sym(const u32x4& v, float scale, float rcp)
+{
+    uint32_t w = nibble_of(div_by_scale(bf16lo(v.x), scale, rcp));
+    w |= nibble_of(div_by_scale(bf16hi(v.x), scale, rcp)) << 4;
+    w |= nibble_of(div_by_scale(bf16lo(v.y), scale, rcp)) << 8;
+    w |= nibble_of(div_by_scale(bf16hi(v.y), scale, rcp)) << 12;
+    w |= nibble_of(div_by_scale(bf16lo(v.z), scale, rcp)) << 16;
+    w |= nibble_of(div_by_scale(bf16hi(v.z), scale, rcp)) << 20;
+    w |= nibble_of(div_by_scale(bf16lo(v.w), scale, rcp)) << 24;
+    w |= nibble_of(div_by_scale(bf16hi(v.w), scale, rcp)) << 28;
+    return w;
+}
+
+// Contiguous tensors only: group g of the tensor starts at x + g*G, its packed words at
+// packed + g*L, its scale at scale[g].
+template <int L, bool GROUPED>
+__global__ __launch_bounds__(256) void int4_pack_kernel(const Int4PackArgs a, const int64_t total_work)
+{
+    constexpr int CL = 256 / L;              // groups per step of the workgroup
+    constexpr int STEPS = kGroupsPerWg / CL; // 1 (L=4), 2 (L=8), 4 (L=16)
+    const int64_t item = (int64_t)blockIdx.x + (int64_t)blockIdx.y * gridDim.x;
+    if (item >= total_work) return;
+    wq_int4_pack_desc d;
+    int64_t local = item;
+    if (GROUPED) {
+        const int di = find_desc_i4(a.work_start, a.n_desc, item);
+        d = a.descs[di];
+        local = item - a.work_start[di];
+    } else {
+        d = a.d;
+    }
+    const int cl = threadIdx.x / L, ll = threadIdx.x % L;
+    const int64_t g0 = local * kGroupsPerWg + cl;
+    const uint16_t* x = (const uint16_t*)d.x;
+
+    u32x4 v[STEPS];
+#pragma unroll
+    for (int i = 0; i < STEPS; ++i) {
+        const int64_t g = g0 + i * CL;
+        v[i] = (u32x4){0u, 0u, 0u, 0u};
+        if (g < d.n_groups) v[i] = __builtin_nontemporal_load((const u32x4*)(x + g * (8 * L) + ll * 8));
+    }
+#pragma unroll
+    for (int i = 0; i < STEPS; ++i) {
+        const int64_t g = g0 + i * CL;
+        uint32_t m = pk_absmax(pk_absmax(pk_absmax(pk_absmax(0u, v[i].x), v[i].y), v[i].z), v[i].w);
+        m = lanes_max_u32<L>(pk_fold(m));
+        const float scale = int4_scale_sym(u2f(m << 16));
+        const float rcp = 1.0f / scale;
+        const uint32_t w = pack8_sym(v[i], scale, rcp);
+        if (g < d.n_groups) {
+            __builtin_nontemporal_store(w, (uint32_t*)d.packed + g * L + ll);
+            if (ll == 0) ((uint16_t*)d.scale)[g] = (uint16_t)f32_to_bf16_bits(scale);
+        }
+    }
+}
+
+// Any group size that is a multiple of 32, strided rows, unaligned pointers.  One 16-lane row per
+// group, two passes over the group.
+__global__ __launch_bounds__(256) void int4_pack_generic_kernel(const uint16_t* __restrict__ x, int64_t M, int64_t N,
+                                                               int64_t sx_m, int group, uint32_t* __restrict__ packed,
+                                                               uint16_t* __restrict__ scale_out)
+{
+    const int64_t G = N / group;
+    const int64_t total = M * G;
+    const int64_t g = ((int64_t)blockIdx.x + (int64_t)blockIdx.y * gridDim.x) * 16 + (threadIdx.x >> 4);
+    const int ll = threadIdx.x & 15;
+    const bool live = g < total;
+    const int64_t row = live ? g / G : 0, gi = live ? g - row * G : 0;
+    const uint16_t* xg = x + row * sx_m + gi * group;
+    uint32_t m = 0;
+    if (live)
+        for (int e = ll; e < group; e += 16) m = max(m, (uint32_t)xg[e] & 0x7FFFu);
+    m = lanes_max_u32<16>(m);
+    const float scale = int4_scale_sym(u2f(m << 16));
+    if (!live) return;
+    if (ll == 0) scale_out[g] = (uint16_t)f32_to_bf16_bits(scale);
+    uint32_t* pg = packed + row * (N / 8) + gi * (group / 8);
+    for (int wi = ll; wi < group / 8; wi += 16) {
+        uint32_t w = 0;
+        for (int j = 0; j < 8; ++j) {
+            float q = u2f((uint32_t)xg[wi * 8 + j] << 16) / scale;
+            w |= nibble_of(q) << (4 * j);
+        }
+        pg[wi] = w;
+    }
+}
+
+// ---- fake quant (codes in the input dtype) -------------------------------------------------------
+
+template <typename T> __device__ __forceinline__ float ld_as_f32(const T* p, int64_t off);
+template <> __device__ __forceinline__ float ld_as_f32<uint16_t>(const uint16_t* p, int64_t off)
+{ return u2f((uint32_t)p[off] << 16); }
+template <> __device__ __forceinline__ float ld_as_f32<float>(const float* p, int64_t off) { return p[off]; }
+template <typename T> __device__ __forceinline__ void st_from_f32(T* p, int64_t off, float v);
+template <> __device__ __forceinline__ void st_from_f32<uint16_t>(uint16_t* p, int64_t off, float v)
+{ p[off] = (uint16_t)f32_to_bf16_bits(v); }
+template <> __device__ __forceinline__ void st_from_f32<float>(float* p, int64_t off, float v) { p[off] = v; }
+
+__device__ __forceinline__ float wave64_max_f32(float v)
+{
+    v = row16_max_f32(v);
+    v = fmaxf(v, __shfl_xor(v, 16));
+    v = fmaxf(v, __shfl_xor(v, 32));
+    return v;
+}
+__device__ __forceinline__ float wave64_min_f32(float v)
+{
+    v = row16_min_f32(v);
+    v = fminf(v, __shfl_xor(v, 16));
+    v = fminf(v, __shfl_xor(v, 32));
+    return v;
+}
+
+// One wavefront per (bm x bn) group.
+template <typename T>
+__global__ __launch_bounds__(256) void int4_fake_quant_kernel(const T* __restrict__ x, int64_t M, int64_t N,
+                                                             int64_t sx_m, int64_t sx_n, int bm, int bn, int sym,
+                                                             T* __restrict__ q, T* __restrict__ scale_out,
+                                                             T* __restrict__ zero_out)
+{
+    const int64_t gn = (N + bn - 1) / bn, gm = (M + bm - 1) / bm;
+    const int64_t grp = ((int64_t)blockIdx.x + (int64_t)blockIdx.y * gridDim.x) * 4 + (threadIdx.x >> 6);
+    if (grp >= gm * gn) return;  // uniform per wavefront
+    const int lane = threadIdx.x & 63;
+    const int64_t bi = grp / gn, bj = grp - bi * gn;
+    const int64_t r0 = bi * bm, c0 = bj * bn;
+    const int n = bm * bn;
+    float vmax = -INFINITY, vmin = INFINITY;
+    for (int e = lane; e < n; e += 64) {
+        const int di = e / bn, dj = e - di * bn;
+        const int64_t i = r0 + di, j = c0 + dj;
+        const float v = (i < M && j < N) ? ld_as_f32<T>(x, i * sx_m + j * sx_n) : 0.0f;
+        if (sym) vmax = fmaxf(vmax, fabsf(v));
+        else { vmax = fmaxf(vmax, v); vmin = fminf(vmin, v); }
+    }
+    vmax = wave64_max_f32(vmax);
+    float scale, zero = 0.0f;
+    if (sym) {
+        scale = fmaxf(vmax * (1.0f / 7.0f), 1e-5f);
+    } else {
+        vmin = wave64_min_f32(vmin);
+        scale = fmaxf((vmax - vmin) * (1.0f / 15.0f), 1e-5f);
+        // "+ 0.0f": a zero result is +0 whatever operand order the max instruction prefers for -0 vs +0
+        zero = fminf(fmaxf(-__builtin_rintf(vmin / scale), 0.0f), 15.0f) + 0.0f;
+    }
+    if (lane == 0) {
+        st_from_f32<T>(scale_out, grp, scale);
+        st_from_f32<T>(zero_out, grp, zero);
+    }
+    for (int e = lane; e < n; e += 64) {
+        const int di = e / bn, dj = e - di * bn;
+        const int64_t i = r0 + di, j = c0 + dj;
+        if (i < M && j < N) {
+            float v = __builtin_rintf(ld_as_f32<T>(x, i * sx_m + j * sx_n) / scale);
+            if (!sym) v += zero;  // the symmetric branch must not add: -0.0f + 0.0f would lose the sign
+            st_from_f32<T>(q, i * N + j, v);
+        }
+    }
+}
+
+template <bool GROUPED>
+static int launch_pack(const Int4PackArgs& a, int64_t work, int group, hipStream_t st)
+{
+    switch (group) {
+    case 32: int4_pack_kernel<4, GROUPED><<<grid_for_items(work), 256, 0, st>>>(a, work); break;
+    case 64: int4_pack_kernel<8, GROUPED><<<grid_for_items(work), 256, 0, st>>>(a, work); break;
+    case 128: int4_pack_kernel<16, GROUPED><<<grid_for_items(work), 256, 0, st>>>(a, work); break;
+    default: return WQ_ERR_UNSUPPORTED;
+    }
+    WQ_LAUNCH_CHECK();
+    return WQ_OK;
+}
+
+}  // namespace wq
+
+using namespace wq;
+
+WQ_EXPORT int wq_int4_group_quant_pack(const void* x, int64_t M, int64_t N, int64_t sx_m, int group, int32_t* packed,
+                                       void* scale, void* stream)
+{
+    if (M < 0 || N < 0 || group <= 0 || group % 32 != 0 || N % group != 0) return WQ_ERR_SHAPE;
+    if (M == 0 || N == 0) return WQ_OK;
+    if (!x || !packed || !scale) return WQ_ERR_NULL;
+    hipStream_t st = (hipStream_t)stream;
+    const int64_t n_groups = M * (N / group);
+    const bool fast = (group == 32 || group == 64 || group == 128) && sx_m == N && ((uintptr_t)x & 15) == 0;
+    if (fast) {
+        Int4PackArgs a{};
+        a.d = wq_int4_pack_desc{x, packed, scale, n_groups};
+        return launch_pack<false>(a, cdiv64(n_groups, kGroupsPerWg), group, st);
+    }
+    int4_pack_generic_kernel<<<grid_for_items(cdiv64(n_groups, 16)), 256, 0, st>>>(
+        (const uint16_t*)x, M, N, sx_m, group, (uint32_t*)packed, (uint16_t*)scale);
+    WQ_LAUNCH_CHECK();
+    return WQ_OK;
+}
+
+WQ_EXPORT int wq_int4_group_quant_pack_grouped(const wq_int4_pack_desc* descs, const int64_t* work_start, int n_desc,
+                                               int64_t total_work, int group, void* stream)
+{
+    if (n_desc < 0 || total_work < 0) return WQ_ERR_SHAPE;
+    if (group != 32 && group != 64 && group != 128) return WQ_ERR_UNSUPPORTED;
+    if (n_desc == 0 || total_work == 0) return WQ_OK;
+    if (!descs || !work_start) return WQ_ERR_NULL;
+    Int4PackArgs a{};
+    a.descs = descs;
+    a.work_start = work_start;
+    a.n_desc = n_desc;
+    return launch_pack<true>(a, total_work, group, (hipStream_t)stream);
+}
+
+WQ_EXPORT int wq_int4_fake_quant(const void* x, int dtype, int64_t M, int64_t N, int64_t sx_m, int64_t sx_n, int bm,
+                                 int bn, int sym, void* q, void* scale, void* zero, void* stream)
+{
+    if (M < 0 || N < 0 || bm <= 0 || bn <= 0) return WQ_ERR_SHAPE;
+    if (dtype != WQ_DTYPE_BF16 && dtype != WQ_DTYPE_F32) return WQ_ERR_MODE;
+    if (((int64_t)bm * bn) % 32 != 0) return WQ_ERR_SHAPE;
+    if (!((bm == 1 && bn % 32 == 0) || (32 % bn == 0))) return WQ_ERR_UNSUPPORTED;
+    if ((int64_t)bm * bn > (1 << 30)) return WQ_ERR_TOO_LARGE;
+    if (M == 0 || N == 0) return WQ_OK;
+    if (!x || !q || !scale || !zero) return WQ_ERR_NULL;
+    const int64_t groups = cdiv64(M, bm) * cdiv64(N, bn);
+    hipStream_t st = (hipStream_t)stream;
+    if (dtype == WQ_DTYPE_BF16)
+        int4_fake_quant_kernel<uint16_t><<<grid_for_items(cdiv64(groups, 4)), 256, 0, st>>>(
+            (const uint16_t*)x, M, N, sx_m, sx_n, bm, bn, sym, (uint16_t*)q, (uint16_t*)scale, (uint16_t*)zero);
+    else
+        int4_fake_quant_kernel<float><<<grid_for_items(cdiv64(groups, 4)), 256, 0, st>>>(
+            (const float*)x, M, N, sx_m, sx_n, bm, bn, sym, (float*)q, (float*)scale, (float*)zero);
+    WQ_LAUNCH_CHECK();
+    return WQ_OK;
+}

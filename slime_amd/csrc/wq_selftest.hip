@@ -1,0 +1,230 @@
+// On-device self-checks of the element functions and of the hardware number-format conversions the
+// production kernels rely on, plus the plain copy kernel used to calibrate hardware counters.
+//
+// The production element functions replace the reference's per-element IEEE division by a
+// reciprocal-and-refine sequence and its software casts by gfx950 conversion instructions.  These
+// kernels compare them, over the complete input domain, with the literal arithmetic (IEEE "/",
+// software round-to-nearest-even), so that the shortcut is licensed by exhaustion, not by argument.
+
+#include "wq_common.h"
+
+namespace wq {
+
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+__global__ void selftest_init_kernel(uint64_t* out)
+{
+    out[0] = 0;
+    out[1] = ~0ull;
+}
+
+__device__ __forceinline__ void report(uint64_t* out, uint64_t key)
+{
+    atomicAdd((unsigned long long*)&out[0], 1ull);
+    atomicMin((unsigned long long*)&out[1], (unsigned long long)key);
+}
+
+// grid.x = 16384 threads' worth of x quadruples per amax, grid.y = amax index
+template <int MODE>
+__global__ __launch_bounds__(256) void selftest_fp8_elem_kernel(uint32_t amax_lo, uint32_t amax_hi, uint64_t* out)
+{
+    const uint32_t a = amax_lo + blockIdx.y;
+    if (a >= amax_hi || a >= kBf16Inf) return;
+    const uint32_t x0 = (blockIdx.x * 256u + threadIdx.x) * 4u;
+    if (x0 >= 65536u) return;
+    const Fp8BlockParams p = fp8_block_params<MODE>(a);
+    const uint32_t w0 = x0 | ((x0 + 1u) << 16), w1 = (x0 + 2u) | ((x0 + 3u) << 16);
+    const uint32_t fast = fp8_quant4_fast<MODE>(w0, w1, p);
+    const uint32_t exact = fp8_quant4_exact<MODE>(w0, w1, p);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const uint32_t xb = x0 + k;
+        if ((xb & 0x7FFFu) > a) continue;  // not reachable: |x| <= block amax
+        if (((fast >> (8 * k)) & 0xFFu) != ((exact >> (8 * k)) & 0xFFu)) report(out, ((uint64_t)a << 16) | xb);
+    }
+}
+
+__global__ __launch_bounds__(256) void selftest_int4_elem_kernel(uint32_t amax_lo, uint32_t amax_hi, uint64_t* out)
+{
+    const uint32_t a = amax_lo + blockIdx.y;
+    if (a >= amax_hi || a >= kBf16Inf) return;
+    const uint32_t xb = blockIdx.x * 256u + threadIdx.x;
+    if (xb >= 65536u || (xb & 0x7FFFu) > a) return;
+    const float scale = int4_scale_sym(u2f(a << 16));
+    const float rcp = 1.0f / scale;
+    const float x = u2f(xb << 16);
+    const float qf = __builtin_rintf(x / scale);
+    const int qi = (int)qf;
+    const uint32_t want = (uint32_t)(qi + 8) & 0xFu;
+    const uint32_t got = f2u(div_by_scale(x, scale, rcp) + 12582920.0f) & 0xFu;
+    if (got != want || qi < -7 || qi > 7) report(out, ((uint64_t)a << 16) | xb);
+}
+
+// hardware fp32 -> e4m3fn vs software, both word positions of the packed conversion
+__global__ __launch_bounds__(256) void selftest_cvt_fp8_kernel(uint64_t lo, uint64_t hi, uint64_t* out)
+{
+    for (uint64_t b = lo + (uint64_t)blockIdx.x * 256u + threadIdx.x; b < hi; b += (uint64_t)gridDim.x * 256u) {
+        const uint32_t u = (uint32_t)b;
+        const uint32_t mag = u & 0x7FFFFFFFu;
+        const bool is_nan = mag > 0x7F800000u;
+        if (!is_nan && mag > 0x43E80000u) continue;  // |v| > 464: overflow behaviour is never relied on
+        const float f = u2f(u);
+        const uint32_t sw = f32_to_e4m3fn_sw(f);
+        const uint32_t h0 = cvt_pk_fp8_lo(f, 0.0f, 0u);
+        const uint32_t h1 = cvt_pk_fp8_hi(0.0f, f, 0u);
+        uint32_t g0 = h0 & 0xFFu, g1 = (h1 >> 24) & 0xFFu;
+        bool bad;
+        if (is_nan) bad = ((g0 & 0x7Fu) != 0x7Fu) || ((g1 & 0x7Fu) != 0x7Fu);
+        else bad = (g0 != sw) || (g1 != sw);
+        if (bad) report(out, b);
+    }
+}
+
+// hardware fp32 -> bf16 (v_cvt_pk_bf16_f32) vs software RNE, non-NaN inputs
+__global__ __launch_bounds__(256) void selftest_cvt_bf16_kernel(uint64_t lo, uint64_t hi, uint64_t* out)
+{
+    for (uint64_t b = lo + (uint64_t)blockIdx.x * 256u + threadIdx.x; b < hi; b += (uint64_t)gridDim.x * 256u) {
+        const uint32_t u = (uint32_t)b;
+        if ((u & 0x7FFFFFFFu) > 0x7F800000u) continue;
+        f32x2 v = {u2f(u), u2f(u ^ 0x80000000u)};
+        const uint32_t hw = __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+        const uint32_t sw = f32_to_bf16_bits(v.x) | (f32_to_bf16_bits(v.y) << 16);
+        if (hw != sw) report(out, b);
+    }
+}
+
+// hardware e4m3fn -> fp32 (v_cvt_pk_f32_fp8) vs the definition, all 256 codes in all 4 byte lanes
+__global__ void selftest_decode_fp8_kernel(uint64_t* out)
+{
+    const uint32_t c = threadIdx.x;  // 256 threads
+    const uint32_t e = (c >> 3) & 0xFu, m = c & 7u;
+    uint32_t want;
+    if (e == 0xFu && m == 7u) want = 0x7FC00000u;
+    else if (e == 0) want = f2u((float)m * 0.001953125f);
+    else want = ((e - 7u + 127u) << 23) | (m << 20);
+    want |= (c & 0x80u) << 24;
+    const uint32_t packed = c | ((c ^ 0xFFu) << 8) | (c << 16) | ((c ^ 0xFFu) << 24);
+    f32x2 lo = __builtin_amdgcn_cvt_pk_f32_fp8((int)packed, false);
+    f32x2 hi = __builtin_amdgcn_cvt_pk_f32_fp8((int)packed, true);
+    const bool nan = (e == 0xFu && m == 7u);
+    bool bad = nan ? !(lo.x != lo.x && hi.x != hi.x) : (f2u(lo.x) != want || f2u(hi.x) != want);
+    if (bad) report(out, c);
+}
+
+__global__ __launch_bounds__(256) void copy_kernel(const u32x4* __restrict__ src, u32x4* __restrict__ dst, int64_t n16)
+{
+    const int64_t base = ((int64_t)blockIdx.x + (int64_t)blockIdx.y * gridDim.x) * 1024 + threadIdx.x;
+    u32x4 v[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int64_t k = base + i * 256;
+        v[i] = (u32x4){0u, 0u, 0u, 0u};
+        if (k < n16) v[i] = __builtin_nontemporal_load(src + k);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int64_t k = base + i * 256;
+        if (k < n16) __builtin_nontemporal_store(v[i], dst + k);
+    }
+}
+
+}  // namespace wq
+
+using namespace wq;
+
+WQ_EXPORT int wq_abi_version(void) { return WQ_ABI_VERSION; }
+
+WQ_EXPORT const char* wq_error_string(int code)
+{
+    switch (code) {
+    case WQ_OK: return "success";
+    case WQ_ERR_NULL: return "a required pointer is NULL";
+    case WQ_ERR_SHAPE: return "invalid shape, block or group size";
+    case WQ_ERR_MODE: return "unknown mode or dtype selector";
+    case WQ_ERR_UNSUPPORTED: return "configuration not supported by this library";
+    case WQ_ERR_ALIGN: return "pointer or stride alignment requirement violated";
+    case WQ_ERR_TOO_LARGE: return "count exceeds the limits of this entry point";
+    default: break;
+    }
+    if (code > 0) return hipGetErrorString((hipError_t)code);
+    return "unknown error";
+}
+
+WQ_EXPORT int wq_selftest_fp8_elem(uint32_t amax_lo, uint32_t amax_hi, int mode, uint64_t* out, void* stream)
+{
+    if (!out) return WQ_ERR_NULL;
+    if (amax_hi < amax_lo || amax_hi > 0x8000u) return WQ_ERR_SHAPE;
+    if (mode != WQ_FP8_MODE_TORCH && mode != WQ_FP8_MODE_TRITON) return WQ_ERR_MODE;
+    hipStream_t st = (hipStream_t)stream;
+    selftest_init_kernel<<<1, 1, 0, st>>>(out);
+    WQ_LAUNCH_CHECK();
+    if (amax_hi == amax_lo) return WQ_OK;
+    dim3 grid(64, amax_hi - amax_lo, 1);
+    if (mode == WQ_FP8_MODE_TORCH) selftest_fp8_elem_kernel<WQ_FP8_MODE_TORCH><<<grid, 256, 0, st>>>(amax_lo, amax_hi, out);
+    else selftest_fp8_elem_kernel<WQ_FP8_MODE_TRITON><<<grid, 256, 0, st>>>(amax_lo, amax_hi, out);
+    WQ_LAUNCH_CHECK();
+    return WQ_OK;
+}
+
+WQ_EXPORT int wq_selftest_int4_elem(uint32_t amax_lo, uint32_t amax_hi, uint64_t* out, void* stream)
+{
+    if (!out) return WQ_ERR_NULL;
+    if (amax_hi < amax_lo || amax_hi > 0x8000u) return WQ_ERR_SHAPE;
+    hipStream_t st = (hipStream_t)stream;
+    selftest_init_kernel<<<1, 1, 0, st>>>(out);
+    WQ_LAUNCH_CHECK();
+    if (amax_hi == amax_lo) return WQ_OK;
+    dim3 grid(256, amax_hi - amax_lo, 1);
+    selftest_int4_elem_kernel<<<grid, 256, 0, st>>>(amax_lo, amax_hi, out);
+    WQ_LAUNCH_CHECK();
+    return WQ_OK;
+}
+
+static int launch_range(void (*k)(uint64_t, uint64_t, uint64_t*), uint64_t lo, uint64_t hi, uint64_t* out, void* stream)
+{
+    if (!out) return WQ_ERR_NULL;
+    if (hi < lo || hi > (1ull << 32)) return WQ_ERR_SHAPE;
+    hipStream_t st = (hipStream_t)stream;
+    selftest_init_kernel<<<1, 1, 0, st>>>(out);
+    WQ_LAUNCH_CHECK();
+    if (hi == lo) return WQ_OK;
+    uint64_t blocks = (hi - lo + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    k<<<(unsigned)blocks, 256, 0, st>>>(lo, hi, out);
+    WQ_LAUNCH_CHECK();
+    return WQ_OK;
+}
+
+WQ_EXPORT int wq_selftest_cvt_fp8(uint64_t lo, uint64_t hi, uint64_t* out, void* stream)
+{
+    return launch_range(selftest_cvt_fp8_kernel, lo, hi, out, stream);
+}
+
+WQ_EXPORT int wq_selftest_cvt_bf16(uint64_t lo, uint64_t hi, uint64_t* out, void* stream)
+{
+    return launch_range(selftest_cvt_bf16_kernel, lo, hi, out, stream);
+}
+
+WQ_EXPORT int wq_selftest_decode_fp8(uint64_t* out, void* stream)
+{
+    if (!out) return WQ_ERR_NULL;
+    hipStream_t st = (hipStream_t)stream;
+    selftest_init_kernel<<<1, 1, 0, st>>>(out);
+    WQ_LAUNCH_CHECK();
+    selftest_decode_fp8_kernel<<<1, 256, 0, st>>>(out);
+    WQ_LAUNCH_CHECK();
+    return WQ_OK;
+}
+
+WQ_EXPORT int wq_copy_bytes(const void* src, void* dst, int64_t n_bytes, void* stream)
+{
+    if (n_bytes < 0 || (n_bytes & 15)) return WQ_ERR_SHAPE;
+    if (n_bytes == 0) return WQ_OK;
+    if (!src || !dst) return WQ_ERR_NULL;
+    if (((uintptr_t)src & 15) || ((uintptr_t)dst & 15)) return WQ_ERR_ALIGN;
+    const int64_t n16 = n_bytes / 16;
+    copy_kernel<<<grid_for_items(cdiv64(n16, 1024)), 256, 0, (hipStream_t)stream>>>((const u32x4*)src, (u32x4*)dst, n16);
+    WQ_LAUNCH_CHECK();
+    return WQ_OK;
+}

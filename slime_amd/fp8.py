@@ -1,0 +1,259 @@
+"""Block-FP8 weight quantisation and dequantisation on MI355X.
+
+Function names, argument meaning, return layouts and error behaviour follow the reference:
+
+* ``block_fp8`` / ``channel_fp8`` / ``tensor_fp8`` / ``quant_fp8``  - tools/convert_hf_to_fp8.py:41-100
+* ``blockwise_cast_to_fp8_triton``                                  - slime/backends/megatron_utils/kernels/fp8_kernel.py:61-79
+  (the name is kept for call-site compatibility; nothing here uses Triton)
+* ``weight_dequant``                                                - tools/fp8_cast_bf16.py:31-41
+* ``weight_dequant_bf16_scale``                                     - slime/backends/megatron_utils/hf_to_megatron/common.py:42-56
+
+All arithmetic runs in the HIP kernels of ``libslime_amd_wq.so``; inputs must live on the GPU.
+``Fp8QuantPlan`` / ``Fp8DequantPlan`` quantise many tensors with ONE kernel launch and write into
+one flat output buffer - the shape a weight-sync bucket wants.
+"""
+
+from __future__ import annotations
+
+from typing import Sequence
+
+import torch
+
+from . import _lib
+
+FP8_DTYPE = torch.float8_e4m3fn
+FP8_INFO = torch.finfo(FP8_DTYPE)
+FP8_MAX, FP8_MIN = FP8_INFO.max, FP8_INFO.min
+
+
+def ceildiv(a: int, b: int) -> int:
+    return -(-a // b)
+
+
+def _check_weight(w: torch.Tensor, what: str) -> None:
+    _lib.require_gpu(w, what)
+    if w.dim() != 2:
+        raise ValueError(f"{what}: expected a 2-D weight, got shape {tuple(w.shape)}")
+    if w.dtype != torch.bfloat16:
+        raise TypeError(f"{what}: only bfloat16 weights are supported (got {w.dtype})")
+
+
+def _block_quant(w: torch.Tensor, bm: int, bn: int, mode: int, what: str):
+    _check_weight(w, what)
+    if bm <= 0 or bn <= 0:
+        raise ValueError(f"{what}: block size must be positive, got {(bm, bn)}")
+    M, N = w.shape
+    q = torch.empty((M, N), dtype=FP8_DTYPE, device=w.device)
+    s = torch.empty((ceildiv(M, bm), ceildiv(N, bn)), dtype=torch.float32, device=w.device)
+    if M and N:
+        with torch.cuda.device(w.device):
+            rc = _lib.load().wq_fp8_block_quant(w.data_ptr(), M, N, w.stride(0), w.stride(1), q.data_ptr(), N,
+                                                s.data_ptr(), bm, bn, mode, _lib.stream_ptr(w.device))
+        _lib.check(rc, what)
+    return q, s
+
+
+def block_fp8(weight: torch.Tensor, block_size) -> tuple[torch.Tensor, torch.Tensor]:
+    """-> (qweight float8_e4m3fn [M,N] contiguous, scale float32 [ceil(M/bn), ceil(N/bk)]).
+
+    Arithmetic of tools/convert_hf_to_fp8.py:41-75: zero padding of edge blocks, amax clamped at
+    1e-12 in the weight dtype, scale = f32(amax)/448, q = clamp(f32(w)/scale), RNE to e4m3fn."""
+    return _block_quant(weight, int(block_size[0]), int(block_size[1]), _lib.FP8_MODE_TORCH, "block_fp8")
+
+
+def channel_fp8(weight: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """Per-row scaling, tools/convert_hf_to_fp8.py:78-83 -> (qweight [M,N], scale float32 [M,1])."""
+    _check_weight(weight, "channel_fp8")
+    M, N = weight.shape
+    q = torch.empty((M, N), dtype=FP8_DTYPE, device=weight.device)
+    s = torch.empty((M, 1), dtype=torch.float32, device=weight.device)
+    if M:
+        with torch.cuda.device(weight.device):
+            rc = _lib.load().wq_fp8_row_quant(weight.data_ptr(), M, N, weight.stride(0), weight.stride(1),
+                                              q.data_ptr(), N, s.data_ptr(), _lib.stream_ptr(weight.device))
+        _lib.check(rc, "channel_fp8")
+    return q, s
+
+
+def tensor_fp8(weight: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """Per-tensor scaling, tools/convert_hf_to_fp8.py:86-91 -> (qweight [M,N], scale float32 [1])."""
+    _check_weight(weight, "tensor_fp8")
+    M, N = weight.shape
+    q = torch.empty((M, N), dtype=FP8_DTYPE, device=weight.device)
+    s = torch.empty((1,), dtype=torch.float32, device=weight.device)
+    ws = torch.zeros((1,), dtype=torch.int32, device=weight.device)
+    with torch.cuda.device(weight.device):
+        rc = _lib.load().wq_fp8_tensor_quant(weight.data_ptr(), M, N, weight.stride(0), weight.stride(1),
+                                             q.data_ptr(), N, s.data_ptr(), ws.data_ptr(),
+                                             _lib.stream_ptr(weight.device))
+    _lib.check(rc, "tensor_fp8")
+    return q, s
+
+
+def quant_fp8(weight: torch.Tensor, strategy: str, block_size=None):
+    """Dispatcher of tools/convert_hf_to_fp8.py:94-100 ("tensor", "channel", anything else = block)."""
+    if strategy == "tensor":
+        return tensor_fp8(weight)
+    if strategy == "channel":
+        return channel_fp8(weight)
+    return block_fp8(weight, block_size)
+
+
+def blockwise_cast_to_fp8_triton(x: torch.Tensor, block_size=None) -> tuple[torch.Tensor, torch.Tensor]:
+    """Weight-sync variant (fp8_kernel.py:61-79): fp32 amax floored at 1e-10, y = x * (1/scale).
+    Accepts any strides, like the kernel it replaces; block size defaults to 128x128."""
+    bm, bn = (128, 128) if not block_size else (int(block_size[0]), int(block_size[1]))
+    return _block_quant(x, bm, bn, _lib.FP8_MODE_TRITON, "blockwise_cast_to_fp8_triton")
+
+
+def _dequant(x: torch.Tensor, s: torch.Tensor, block_size: int, mode: int, out_dtype: torch.dtype, what: str):
+    _lib.require_gpu(x, what)
+    assert x.is_contiguous() and s.is_contiguous()
+    assert x.dim() == 2 and s.dim() == 2
+    if x.element_size() != 1:
+        raise TypeError(f"{what}: x must hold one-byte e4m3fn codes, got {x.dtype}")
+    if s.dtype != torch.float32:
+        raise TypeError(f"{what}: scale must be float32, got {s.dtype}")
+    if out_dtype not in (torch.bfloat16, torch.float32):
+        raise TypeError(f"{what}: output dtype {out_dtype} is not supported (bfloat16 or float32)")
+    M, N = x.shape
+    if tuple(s.shape) != (ceildiv(M, block_size), ceildiv(N, block_size)):
+        raise ValueError(f"{what}: scale shape {tuple(s.shape)} does not match x {tuple(x.shape)} / {block_size}")
+    y = torch.empty((M, N), dtype=out_dtype, device=x.device)
+    if M and N:
+        with torch.cuda.device(x.device):
+            rc = _lib.load().wq_fp8_block_dequant(
+                x.data_ptr(), s.data_ptr(), y.data_ptr(),
+                _lib.DTYPE_BF16 if out_dtype == torch.bfloat16 else _lib.DTYPE_F32,
+                M, N, int(block_size), mode, _lib.stream_ptr(x.device))
+        _lib.check(rc, what)
+    return y
+
+
+def weight_dequant(x: torch.Tensor, s: torch.Tensor, block_size: int = 128) -> torch.Tensor:
+    """y = (f32(x) * s[block]) in torch's default dtype (tools/fp8_cast_bf16.py:31-41; the tool sets the
+    default dtype to bfloat16 at :45, callers that have not get float32, as with the reference)."""
+    return _dequant(x, s, block_size, _lib.DEQ_MODE_F32SCALE, torch.get_default_dtype(), "weight_dequant")
+
+
+def weight_dequant_bf16_scale(x: torch.Tensor, s: torch.Tensor, block_size: int = 128) -> torch.Tensor:
+    """Dequant-on-read of the HF->Megatron loader (hf_to_megatron/common.py:42-56): the scale is
+    rounded to bf16 before the multiply; result bf16."""
+    return _dequant(x, s, block_size, _lib.DEQ_MODE_BF16SCALE, torch.bfloat16, "weight_dequant_bf16_scale")
+
+
+# ------------------------------------------------------------------------------------ grouped launches
+
+
+def _align(n: int, a: int = 256) -> int:
+    return (n + a - 1) // a * a
+
+
+def _to_device_i64(rows, device) -> torch.Tensor:
+    return torch.tensor(rows, dtype=torch.int64).to(device)
+
+
+class Fp8QuantPlan:
+    """Quantise a fixed list of bf16 weights with one kernel launch per ``run()``.
+
+    Outputs live in two flat buffers owned by the plan (``flat_q`` bytes, ``flat_s`` fp32); ``outputs``
+    holds per-tensor views ``(qweight [M,N] e4m3fn, scale [tm,tn])`` in input order.  The plan reads
+    the weights' current contents on every run, so it can be reused across weight-sync steps as long
+    as the input tensors stay at the same addresses.  mode: 0 = ``block_fp8`` arithmetic,
+    1 = ``blockwise_cast_to_fp8_triton`` arithmetic.
+    """
+
+    def __init__(self, weights: Sequence[torch.Tensor], block_size=(128, 128), mode: int = 0):
+        if not weights:
+            raise ValueError("Fp8QuantPlan: empty weight list")
+        self.bm, self.bn = int(block_size[0]), int(block_size[1])
+        self.mode = int(mode)
+        self.device = weights[0].device
+        self.weights = list(weights)
+        q_off, s_off, q_total, s_total = [], [], 0, 0
+        for w in self.weights:
+            _check_weight(w, "Fp8QuantPlan")
+            if w.device != self.device:
+                raise ValueError("Fp8QuantPlan: all weights must be on one device")
+            M, N = w.shape
+            q_off.append(q_total)
+            s_off.append(s_total)
+            q_total += _align(M * N)
+            s_total += _align(ceildiv(M, self.bm) * ceildiv(N, self.bn) * 4) // 4
+        self.flat_q = torch.empty(max(q_total, 1), dtype=torch.uint8, device=self.device)
+        self.flat_s = torch.empty(max(s_total, 1), dtype=torch.float32, device=self.device)
+        rows, starts, tiles = [], [0], 0
+        self.outputs = []
+        for w, qo, so in zip(self.weights, q_off, s_off):
+            M, N = w.shape
+            tm, tn = ceildiv(M, self.bm), ceildiv(N, self.bn)
+            q = self.flat_q[qo:qo + M * N].view(FP8_DTYPE).view(M, N)
+            s = self.flat_s[so:so + tm * tn].view(tm, tn)
+            self.outputs.append((q, s))
+            rows.append([w.data_ptr(), q.data_ptr(), s.data_ptr(), M, N, w.stride(0), w.stride(1), N])
+            tiles += tm * tn
+            starts.append(tiles)
+        self.total_tiles = tiles
+        self.bf16_bytes = sum(2 * w.numel() for w in self.weights)
+        self._descs = _to_device_i64(rows, self.device)
+        self._starts = _to_device_i64(starts, self.device)
+
+    def run(self):
+        with torch.cuda.device(self.device):
+            rc = _lib.load().wq_fp8_block_quant_grouped(self._descs.data_ptr(), self._starts.data_ptr(),
+                                                        len(self.weights), self.total_tiles, self.bm, self.bn,
+                                                        self.mode, _lib.stream_ptr(self.device))
+        _lib.check(rc, "Fp8QuantPlan.run")
+        return self.outputs
+
+
+def block_fp8_many(weights: Sequence[torch.Tensor], block_size=(128, 128), mode: int = 0):
+    """One-launch ``block_fp8`` over a list of weights -> list of (qweight, scale)."""
+    return Fp8QuantPlan(weights, block_size, mode).run() if weights else []
+
+
+class Fp8DequantPlan:
+    """One-launch block-FP8 -> bf16 over a fixed list of (codes, scale_inv) pairs; see Fp8QuantPlan."""
+
+    def __init__(self, xs: Sequence[torch.Tensor], ss: Sequence[torch.Tensor], block_size: int = 128,
+                 mode: int = 0, out_dtype: torch.dtype = torch.bfloat16):
+        if not xs or len(xs) != len(ss):
+            raise ValueError("Fp8DequantPlan: need equally many code and scale tensors")
+        if out_dtype not in (torch.bfloat16, torch.float32):
+            raise TypeError(f"Fp8DequantPlan: output dtype {out_dtype} is not supported")
+        self.block, self.mode, self.out_dtype = int(block_size), int(mode), out_dtype
+        self.device = xs[0].device
+        self.xs, self.ss = list(xs), list(ss)
+        esz = 2 if out_dtype == torch.bfloat16 else 4
+        offs, total = [], 0
+        for x, s in zip(self.xs, self.ss):
+            _lib.require_gpu(x, "Fp8DequantPlan")
+            assert x.is_contiguous() and s.is_contiguous() and x.dim() == 2 and s.dim() == 2
+            assert x.element_size() == 1 and s.dtype == torch.float32
+            M, N = x.shape
+            assert tuple(s.shape) == (ceildiv(M, self.block), ceildiv(N, self.block))
+            offs.append(total)
+            total += _align(M * N * esz) // esz
+        self.flat_y = torch.empty(max(total, 1), dtype=out_dtype, device=self.device)
+        rows, starts, work = [], [0], 0
+        self.outputs = []
+        for x, s, o in zip(self.xs, self.ss, offs):
+            M, N = x.shape
+            y = self.flat_y[o:o + M * N].view(M, N)
+            self.outputs.append(y)
+            rows.append([x.data_ptr(), s.data_ptr(), y.data_ptr(), M, N])
+            work += ceildiv(M, _lib.DEQ_ROWS) * ceildiv(N, _lib.DEQ_COLS)
+            starts.append(work)
+        self.total_work = work
+        self.out_bytes = sum(x.numel() * esz for x in self.xs)
+        self._descs = _to_device_i64(rows, self.device)
+        self._starts = _to_device_i64(starts, self.device)
+
+    def run(self):
+        with torch.cuda.device(self.device):
+            rc = _lib.load().wq_fp8_block_dequant_grouped(
+                self._descs.data_ptr(), self._starts.data_ptr(), len(self.xs), self.total_work,
+                _lib.DTYPE_BF16 if self.out_dtype == torch.bfloat16 else _lib.DTYPE_F32,
+                self.block, self.mode, _lib.stream_ptr(self.device))
+        _lib.check(rc, "Fp8DequantPlan.run")
+        return self.outputs

@@ -1,0 +1,193 @@
+"""Group-wise INT4 weight quantisation and packing on MI355X.
+
+Mirrors, name for name, the functions of tools/convert_hf_to_int4_direct.py:32-153 (identical copies live
+in slime/backends/megatron_utils/megatron_to_hf/processors/quantizer_compressed_tensors.py:137-265) and
+the extension entry point fake_int4_quant_cuda(x, block_size, sym) of
+slime/backends/megatron_utils/kernels/int4_qat/fake_int4_quant_cuda.cu:327-378.
+
+``pack_layer`` with ``sym=True`` on a bf16 weight runs ONE fused HIP kernel (amax, scale, divide,
+round, nibble pack).  The reference's intermediate dequantise / re-quantise steps map every integer
+code back to itself for all reachable (code, bf16 scale) pairs - the test-suite re-proves this by
+exhaustion - so they are not executed.  The asymmetric branch runs the HIP fake-quant kernel and then
+the reference's own chain of tensor ops on the GPU.
+"""
+
+from __future__ import annotations
+
+import math
+from typing import Sequence
+
+import torch
+
+from . import _lib
+
+
+def _dtype_sel(t: torch.Tensor, what: str) -> int:
+    if t.dtype == torch.bfloat16:
+        return _lib.DTYPE_BF16
+    if t.dtype == torch.float32:
+        return _lib.DTYPE_F32
+    raise TypeError(f"{what}: dtype {t.dtype} is not supported (bfloat16 or float32)")
+
+
+def fake_int4_quant_cuda(x: torch.Tensor, block_size: Sequence[int], sym: bool):
+    """-> (q, scale, zero): q has x's shape and dtype and holds the integer codes as floats; scale and
+    zero are [ceil(M/bm), ceil(N/bn)] in x's dtype.  Errors are RuntimeError, as TORCH_CHECK raises
+    (fake_int4_quant_cuda.cu:333-344)."""
+    if x.dim() != 2:
+        raise RuntimeError("Input must be 2D")
+    if not x.is_cuda:
+        raise RuntimeError("Input must be on the GPU")
+    bm, bn = int(block_size[0]), int(block_size[1])
+    if bm <= 0 or bn <= 0:
+        raise RuntimeError(f"Block sizes must be positive, got block_m={bm}, block_n={bn}")
+    if (bm * bn) % 32 != 0:
+        raise RuntimeError(f"block_m * block_n ({bm * bn}) must be divisible by 32. But got a {bm}x{bn} block.")
+    sel = _dtype_sel(x, "fake_int4_quant_cuda")
+    M, N = x.shape
+    q = torch.empty((M, N), dtype=x.dtype, device=x.device)
+    scale = torch.empty((-(-M // bm), -(-N // bn)), dtype=x.dtype, device=x.device)
+    zero = torch.empty_like(scale)
+    with torch.cuda.device(x.device):
+        rc = _lib.load().wq_int4_fake_quant(x.data_ptr(), sel, M, N, x.stride(0), x.stride(1), bm, bn, int(bool(sym)),
+                                            q.data_ptr(), scale.data_ptr(), zero.data_ptr(), _lib.stream_ptr(x.device))
+    _lib.check(rc, "fake_int4_quant_cuda")
+    return q, scale, zero
+
+
+def pack_to_int32(value: torch.Tensor, num_bits: int, packed_dim: int = 1, sym: bool = False) -> torch.Tensor:
+    """Pack ``32 // num_bits`` integers per int32 along ``packed_dim``; element j of a word sits at bits
+    [j*num_bits, (j+1)*num_bits).  ``sym`` adds the offset 2**(num_bits-1) first.
+    (tools/convert_hf_to_int4_direct.py:32-75; pure integer tensor ops on value's device.)"""
+    if num_bits > 8:
+        raise ValueError("Packing is only supported for less than 8 bits")
+    if num_bits < 1:
+        raise ValueError(f"num_bits must be at least 1, got {num_bits}")
+    if sym:
+        value = (value + (1 << (num_bits - 1))).to(torch.uint8)
+    per_word = 32 // num_bits
+    if packed_dim == 0:
+        value = value.transpose(0, 1)
+    rows, cols = value.shape
+    n_words = math.ceil(cols / per_word)
+    if n_words * per_word != cols:
+        value = torch.nn.functional.pad(value, (0, n_words * per_word - cols))
+    shifts = torch.arange(per_word, device=value.device, dtype=torch.int32) * num_bits
+    words = (value.view(rows, n_words, per_word).to(torch.int32) << shifts).sum(dim=2, dtype=torch.int32)
+    return words.transpose(0, 1) if packed_dim == 0 else words
+
+
+def round_to_quantized_type_dtype(tensor: torch.Tensor, dtype: torch.dtype, cast_to_original_dtype: bool = False):
+    """clamp to dtype's integer range, round half to even, cast (convert_hf_to_int4_direct.py:78-88)."""
+    lim = torch.iinfo(dtype)
+    out = torch.round(torch.clamp(tensor, lim.min, lim.max)).to(dtype)
+    return out.to(tensor.dtype) if cast_to_original_dtype else out
+
+
+@torch.no_grad()
+def quantize(x: torch.Tensor, scale: torch.Tensor, zero_point, dtype: torch.dtype = torch.int8) -> torch.Tensor:
+    """x / scale (+ zero_point) per group of x.shape[-1] // scale.shape[-1] columns, clamped, rounded and
+    cast to ``dtype`` (convert_hf_to_int4_direct.py:91-120)."""
+    group = x.shape[-1] // scale.shape[-1]
+    scaled = x.unflatten(-1, (math.ceil(x.shape[-1] / group), group)) / scale.unsqueeze(-1)
+    if zero_point is not None:
+        scaled += zero_point.unsqueeze(-1).to(x.dtype)
+    return round_to_quantized_type_dtype(scaled, dtype).flatten(start_dim=-2).to(dtype)
+
+
+def _check_pack_input(weight: torch.Tensor, group_size: int, what: str) -> None:
+    if weight.dim() != 2:
+        raise RuntimeError(f"{what}: expected a 2-D weight")
+    _lib.require_gpu(weight, what)
+    if group_size <= 0 or weight.shape[1] % group_size != 0:
+        # the reference fails in .view(M, 1, N // group_size, group_size)
+        raise RuntimeError(f"{what}: shape '{[weight.shape[0], 1, weight.shape[1] // max(group_size, 1), group_size]}' "
+                           f"is invalid for input of size {weight.numel()}")
+    if group_size % 32 != 0:
+        raise RuntimeError(f"block_m * block_n ({group_size}) must be divisible by 32. But got a 1x{group_size} block.")
+
+
+def pack_layer(weight: torch.Tensor, group_size: int, sym: bool = True):
+    """-> (weight_packed int32 [M, N/8], weight_scale [M, N/group_size] in weight dtype,
+    packed_zero_point int32 [N/group_size, M/8] or None).  convert_hf_to_int4_direct.py:123-153."""
+    _check_pack_input(weight, group_size, "pack_layer")
+    M, N = weight.shape
+    if sym and weight.dtype == torch.bfloat16 and weight.stride(1) == 1:
+        packed = torch.empty((M, N // 8), dtype=torch.int32, device=weight.device)
+        scale = torch.empty((M, N // group_size), dtype=torch.bfloat16, device=weight.device)
+        if M and N:
+            with torch.cuda.device(weight.device):
+                rc = _lib.load().wq_int4_group_quant_pack(weight.data_ptr(), M, N, weight.stride(0), int(group_size),
+                                                          packed.data_ptr(), scale.data_ptr(),
+                                                          _lib.stream_ptr(weight.device))
+            _lib.check(rc, "pack_layer")
+        return packed, scale, None
+
+    # general form: HIP fake-quant kernel, then the reference's tensor-op chain on the GPU
+    G = N // group_size
+    q, scale, zp = fake_int4_quant_cuda(weight, (1, group_size), sym)
+    q = q.view(M, 1, G, group_size)
+    scale = scale.view(M, 1, G, 1)
+    zp = zp.view(M, 1, G, 1)
+    deq = (q * scale if sym else (q - zp) * scale).view(M, N)
+    scale = scale.view(M, -1).contiguous()
+    if sym:
+        zp = packed_zp = None
+    else:
+        zp = zp.view(M, -1)
+        z = zp.t().contiguous().to(torch.float32).to(torch.int32)
+        awq_order = torch.tensor([0, 4, 1, 5, 2, 6, 3, 7], device=z.device) * 4
+        packed_zp = (z.reshape(-1, z.shape[1] // 8, 8) << awq_order).sum(dim=-1).to(torch.int32)
+    codes = quantize(deq, scale, zp, torch.int8 if sym else torch.uint8)
+    return pack_to_int32(codes, 4, sym=sym), scale, packed_zp
+
+
+class Int4PackPlan:
+    """Symmetric quantise+pack of a fixed list of contiguous bf16 weights with one launch per ``run()``.
+
+    ``outputs`` holds ``(weight_packed int32 [M,N/8], weight_scale bf16 [M,N/group])`` views into the
+    plan's flat buffers, in input order."""
+
+    def __init__(self, weights: Sequence[torch.Tensor], group_size: int = 128):
+        if not weights:
+            raise ValueError("Int4PackPlan: empty weight list")
+        if group_size not in (32, 64, 128):
+            raise ValueError("Int4PackPlan: group_size must be 32, 64 or 128")
+        self.group = int(group_size)
+        self.device = weights[0].device
+        self.weights = list(weights)
+        p_off, s_off, p_total, s_total = [], [], 0, 0
+        for w in self.weights:
+            _check_pack_input(w, self.group, "Int4PackPlan")
+            if w.dtype != torch.bfloat16 or not w.is_contiguous() or w.data_ptr() % 16:
+                raise ValueError("Int4PackPlan: weights must be contiguous, 16-byte aligned bfloat16")
+            M, N = w.shape
+            p_off.append(p_total)
+            s_off.append(s_total)
+            p_total += (M * N // 8 + 63) // 64 * 64
+            s_total += (M * N // self.group + 127) // 128 * 128
+        self.flat_packed = torch.empty(max(p_total, 1), dtype=torch.int32, device=self.device)
+        self.flat_scale = torch.empty(max(s_total, 1), dtype=torch.bfloat16, device=self.device)
+        rows, starts, work = [], [0], 0
+        self.outputs = []
+        for w, po, so in zip(self.weights, p_off, s_off):
+            M, N = w.shape
+            n_groups = M * N // self.group
+            packed = self.flat_packed[po:po + M * N // 8].view(M, N // 8)
+            scale = self.flat_scale[so:so + n_groups].view(M, N // self.group)
+            self.outputs.append((packed, scale))
+            rows.append([w.data_ptr(), packed.data_ptr(), scale.data_ptr(), n_groups])
+            work += -(-n_groups // _lib.INT4_GROUPS_PER_WG)
+            starts.append(work)
+        self.total_work = work
+        self.bf16_bytes = sum(2 * w.numel() for w in self.weights)
+        self._descs = torch.tensor(rows, dtype=torch.int64).to(self.device)
+        self._starts = torch.tensor(starts, dtype=torch.int64).to(self.device)
+
+    def run(self):
+        with torch.cuda.device(self.device):
+            rc = _lib.load().wq_int4_group_quant_pack_grouped(self._descs.data_ptr(), self._starts.data_ptr(),
+                                                              len(self.weights), self.total_work, self.group,
+                                                              _lib.stream_ptr(self.device))
+        _lib.check(rc, "Int4PackPlan.run")
+        return self.outputs

@@ -1,0 +1,89 @@
+"""The C-ABI library loads without a GPU, exports every symbol the header declares, and rejects bad
+arguments before launching anything (no compute calls here)."""
+
+import ctypes
+import os
+import re
+
+import pytest
+
+from slime_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "slime_amd_wq.h")
+
+
+def _declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(wq_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_symbols_are_exported_and_bound():
+    lib = _lib.load()
+    names = _declared_symbols()
+    assert len(names) >= 15
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in the header but not exported"
+        assert n in _lib.SIGNATURES, f"{n} has no ctypes signature"
+    assert sorted(_lib.SIGNATURES) == names
+
+
+def test_abi_version_and_error_strings():
+    lib = _lib.load()
+    assert lib.wq_abi_version() == _lib.ABI_VERSION
+    for code in (0, -1, -2, -3, -4, -5, -6):
+        assert lib.wq_error_string(code)
+    assert lib.wq_error_string(-99) == b"unknown error"
+
+
+def test_argument_validation_without_launch():
+    lib = _lib.load()
+    S, M_, U, N_ = -2, -3, -4, -1
+    assert lib.wq_fp8_block_quant(None, -1, 4, 4, 1, None, 4, None, 128, 128, 0, None) == S
+    assert lib.wq_fp8_block_quant(None, 4, 4, 4, 1, None, 4, None, 0, 128, 0, None) == S
+    assert lib.wq_fp8_block_quant(None, 4, 4, 4, 1, None, 4, None, 128, 128, 7, None) == M_
+    assert lib.wq_fp8_block_quant(None, 4, 4, 4, 1, None, 4, None, 128, 128, 0, None) == N_
+    assert lib.wq_fp8_block_quant(None, 0, 4, 4, 1, None, 4, None, 128, 128, 0, None) == 0      # empty: no-op
+    assert lib.wq_fp8_block_quant_grouped(None, None, 3, 10, 128, 128, 0, None) == N_
+    assert lib.wq_fp8_block_quant_grouped(None, None, 0, 0, 128, 128, 0, None) == 0
+    assert lib.wq_fp8_row_quant(None, -1, 4, 4, 1, None, 4, None, None) == S
+    assert lib.wq_fp8_tensor_quant(None, 4, 4, 4, 1, None, 4, None, None, None) == N_
+    assert lib.wq_fp8_block_dequant(None, None, None, 0, 4, 4, 0, 0, None) == S
+    assert lib.wq_fp8_block_dequant(None, None, None, 5, 4, 4, 128, 0, None) == M_
+    assert lib.wq_fp8_block_dequant(None, None, None, 0, 4, 4, 128, 0, None) == N_
+    assert lib.wq_fp8_block_dequant_grouped(None, None, 1, 1, 0, 128, 3, None) == M_
+    assert lib.wq_int4_fake_quant(None, 0, 4, 64, 64, 1, 1, 48, 1, None, None, None, None) == S
+    assert lib.wq_int4_fake_quant(None, 0, 4, 64, 64, 1, 2, 64, 1, None, None, None, None) == U
+    assert lib.wq_int4_fake_quant(None, 9, 4, 64, 64, 1, 1, 32, 1, None, None, None, None) == M_
+    assert lib.wq_int4_group_quant_pack(None, 4, 100, 100, 128, None, None, None) == S
+    assert lib.wq_int4_group_quant_pack(None, 4, 128, 128, 128, None, None, None) == N_
+    assert lib.wq_int4_group_quant_pack_grouped(None, None, 1, 1, 96, None) == U
+    assert lib.wq_copy_bytes(None, None, 24, None) == S
+    assert lib.wq_selftest_fp8_elem(0, 0x9000, 0, ctypes.c_void_p(8), None) == S
+
+
+def test_check_raises_runtime_error():
+    with pytest.raises(RuntimeError, match="invalid shape"):
+        _lib.check(-2, "probe")
+
+
+def test_cpu_tensors_are_refused():
+    import torch
+
+    import slime_amd
+
+    w = torch.zeros(128, 128, dtype=torch.bfloat16)
+    for fn in (lambda: slime_amd.block_fp8(w, (128, 128)), lambda: slime_amd.channel_fp8(w),
+               lambda: slime_amd.tensor_fp8(w), lambda: slime_amd.blockwise_cast_to_fp8_triton(w),
+               lambda: slime_amd.pack_layer(w, 128), lambda: slime_amd.fake_int4_quant_cuda(w, (1, 128), True),
+               lambda: slime_amd.weight_dequant(w.view(torch.uint8)[:, :128].contiguous(), torch.ones(1, 1))):
+        with pytest.raises(RuntimeError, match="GPU"):
+            fn()
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "nope.so"))
+    with pytest.raises(_lib.WqLibraryError, match="no CPU or pure-torch fallback"):
+        _lib.load()

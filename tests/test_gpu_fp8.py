@@ -1,0 +1,265 @@
+"""HIP FP8 kernels (through the C ABI) against the CPU oracle: bit-exact codes and scales."""
+
+import os
+
+import pytest
+import torch
+
+import slime_amd
+from oracle import c_oracle as C
+from oracle import torch_ref as T
+from tests import wq_inputs as I
+
+pytestmark = pytest.mark.gpu
+E4M3 = torch.float8_e4m3fn
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def _codes(t):
+    return t.cpu().view(torch.uint8)
+
+
+def _bits32(t):
+    return t.cpu().contiguous().view(torch.int32)
+
+
+def _check_block(w_cpu, w_gpu, block=(128, 128), mode=0):
+    fn = slime_amd.block_fp8 if mode == 0 else slime_amd.blockwise_cast_to_fp8_triton
+    q, s = fn(w_gpu, block)
+    assert q.dtype == E4M3 and q.is_contiguous() and s.dtype == torch.float32
+    qo, so = C.fp8_block_quant(w_cpu, block, mode)
+    assert q.shape == qo.shape and s.shape == so.shape
+    nbad = int((_codes(q) != qo).sum())
+    assert nbad == 0, f"{nbad} code mismatches"
+    assert torch.equal(_bits32(s), _bits32(so))
+    return q, s
+
+
+SHAPES = [(128, 128), (256, 384), (300, 200), (7, 7168), (1, 1), (1, 8), (129, 127), (4100, 3000), (4096, 4096),
+          (1024, 2560), (2560, 9728)]
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+@pytest.mark.parametrize("mode", [0, 1])
+def test_block_quant_shapes(cuda, shape, mode):
+    w = I.zero_blocks(I.weights(*shape, seed=sum(shape)), 0.2, seed=1)
+    _check_block(w, w.to(cuda), mode=mode)
+
+
+def test_block_quant_config1_roundtrip(cuda):
+    # [4096,4096] N(0,0.02), 0.1% of entries x20, seed 0: quant then dequant of its own output
+    w = I.weights(4096, 4096, seed=0)
+    q, s = _check_block(w, w.to(cuda))
+    torch.set_default_dtype(torch.bfloat16)
+    try:
+        d = slime_amd.weight_dequant(q, s)
+    finally:
+        torch.set_default_dtype(torch.float32)
+    assert d.dtype == torch.bfloat16
+    assert I.same_bits(d.cpu(), C.fp8_block_dequant(_codes(q), s.cpu(), 128, 0))
+    step = s.cpu().repeat_interleave(128, 0).repeat_interleave(128, 1) * 32
+    assert ((d.cpu().float() - w.float()).abs() <= step / 2 * 1.01).all()
+
+
+def test_block_quant_tall_ragged(cuda):
+    # [151937, 2560]: vocabulary-sized, 1-row remainder block row
+    w = I.weights(151937, 2560, seed=5, outlier_p=0)
+    _check_block(w, w.to(cuda))
+
+
+@pytest.mark.parametrize("block", [(32, 32), (64, 128), (128, 64), (1, 128), (16, 48), (256, 256)])
+def test_block_quant_other_block_sizes(cuda, block):
+    w = I.weights(200, 330, seed=2)
+    for mode in (0, 1):
+        _check_block(w, w.to(cuda), block, mode)
+
+
+def test_block_quant_strided_and_unaligned(cuda):
+    base = I.weights(512, 776, seed=4)
+    bg = base.to(cuda)
+    views = [lambda t: t[:, 128:640], lambda t: t.t(), lambda t: t[::2, ::3], lambda t: t[100:357, 5:700],
+             lambda t: t[:, 8:], lambda t: t[:, 1:769], lambda t: t[3:, :768]]
+    for v in views:
+        for mode in (0, 1):
+            _check_block(v(base), v(bg), mode=mode)
+
+
+def test_block_quant_special_blocks(cuda):
+    blocks = [I.subnormal_block(seed=1), I.near_max_block(seed=2), I.near_max_block(seed=3, amax=3.0e38),
+              I.near_max_block(seed=4, amax=1.2e-38), torch.zeros(128, 128, dtype=torch.bfloat16),
+              -torch.zeros(128, 128, dtype=torch.bfloat16)]
+    w = torch.cat(blocks, dim=1)
+    for mode in (0, 1):
+        q, s = _check_block(w, w.to(cuda), mode=mode)
+    assert _bits32(s)[0, 4].item() != 0
+    q, s = slime_amd.block_fp8(w.to(cuda), (128, 128))
+    assert _bits32(s)[0, 4].item() == 0x27212492 and (_codes(q)[:, 640:] == 0x80).all()
+
+
+def test_block_quant_every_bf16_value(cuda):
+    g = I.gen(9)
+    amax_bits = torch.cat([torch.randint(1, 0x7F80, (40,), generator=g),
+                           torch.tensor([1, 0x2B8C, 0x2B8D, 0x2B8E, 0x7F7F, 0x0080, 0x007F])]).tolist()
+    vals = I.finite_bf16_values()
+    for ab in amax_bits:
+        amax = torch.tensor([ab], dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+        x = vals[vals.abs() <= amax]
+        x = torch.cat([x, torch.zeros((-x.numel()) % (128 * 128), dtype=torch.bfloat16)]).view(-1, 128)
+        x[::128, 0] = amax
+        for mode in (0, 1):
+            _check_block(x, x.to(cuda), mode=mode)
+
+
+def test_block_quant_nan_inf(cuda):
+    w = I.weights(128, 384, seed=6)
+    w[5, 5] = float("nan")
+    w[9, 130] = float("inf")
+    w[10, 131] = -float("inf")
+    q, s = slime_amd.block_fp8(w.to(cuda), (128, 128))
+    q, s = _codes(q), s.cpu()
+    qo, so = C.fp8_block_quant(w, (128, 128), 0)
+    assert s[0, 0].isnan() and ((q[:, :128] & 0x7F) == 0x7F).all()
+    assert s[0, 1].isinf()
+    nan_o = (qo & 0x7F) == 0x7F
+    assert torch.equal((q & 0x7F) == 0x7F, nan_o)
+    assert torch.equal(q[~nan_o], qo[~nan_o])
+    assert torch.equal(_bits32(s[:, 2]), _bits32(so[:, 2]))
+
+
+def test_reference_suite_invariants_on_gpu(cuda):
+    # the three cases of the reference's tests/test_block_fp8_zero_block.py:38-75
+    w = torch.zeros(256, 256, dtype=torch.bfloat16)
+    w[0, 0] = 1.0
+    q, s = slime_amd.block_fp8(w.to(cuda), (128, 128))
+    assert not torch.isnan(q.float()).any() and not torch.isinf(q.float()).any() and (s > 0).all()
+    q, s = slime_amd.block_fp8(torch.zeros(128, 128, dtype=torch.bfloat16, device=cuda), (128, 128))
+    assert ((q.float() * s.float()) == 0).all()
+    torch.manual_seed(0)
+    w = torch.randn(256, 256, dtype=torch.float32).to(torch.bfloat16)
+    q, s = slime_amd.block_fp8(w.to(cuda), (128, 128))
+    deq = q.float().cpu() * s.cpu().repeat_interleave(128, 0).repeat_interleave(128, 1)
+    assert not torch.isnan(q.float()).any() and (deq - w.float()).abs().max() < 0.5
+
+
+@pytest.mark.parametrize("shape", [(64, 256), (3, 1000), (257, 129), (1024, 2560)])
+def test_channel_and_tensor_quant(cuda, shape):
+    w = I.weights(*shape, seed=8)
+    w[1] = 0
+    for gpu_fn, ora, sshape in ((slime_amd.channel_fp8, C.fp8_channel_quant, (shape[0], 1)),
+                                (slime_amd.tensor_fp8, C.fp8_tensor_quant, (1,))):
+        q, s = gpu_fn(w.to(cuda))
+        qo, so = ora(w)
+        assert tuple(s.shape) == sshape
+        assert torch.equal(_codes(q), qo) and torch.equal(_bits32(s), _bits32(so))
+    q, s = slime_amd.quant_fp8(w.to(cuda), "channel")
+    assert tuple(s.shape) == (shape[0], 1)
+    q, s = slime_amd.quant_fp8(w.to(cuda), "block", (128, 128))
+    assert tuple(s.shape) == (-(-shape[0] // 128), -(-shape[1] // 128))
+
+
+# ------------------------------------------------------------------ dequant
+
+def test_dequant_all_codes(cuda):
+    codes = torch.arange(256, dtype=torch.int32).to(torch.uint8).repeat(128, 1)
+    s = I.log_uniform_scales(1, 2, seed=3)
+    for mode, fn in ((0, lambda x, sc: slime_amd.fp8._dequant(x, sc, 128, 0, torch.bfloat16, "t")),
+                     (1, slime_amd.weight_dequant_bf16_scale)):
+        got = fn(codes.to(cuda).view(E4M3), s.to(cuda)).cpu()
+        want = C.fp8_block_dequant(codes, s, 128, mode)
+        ok = ~want.isnan()
+        assert torch.equal(got.isnan(), want.isnan())
+        assert torch.equal(got[ok].view(torch.int16), want[ok].view(torch.int16))
+
+
+@pytest.mark.parametrize("shape", [(256, 256), (300, 200), (7, 7168), (129, 1), (2048, 7168), (7168, 2048), (16, 1024),
+                                   (17, 1040), (5, 1000)])
+def test_dequant_shapes(cuda, shape):
+    x = I.fp8_codes(*shape, seed=shape[0])
+    s = I.log_uniform_scales(-(-shape[0] // 128), -(-shape[1] // 128), seed=shape[1])
+    xg, sg = x.to(cuda).view(E4M3), s.to(cuda)
+    y0 = slime_amd.fp8._dequant(xg, sg, 128, 0, torch.bfloat16, "t")
+    assert I.same_bits(y0.cpu(), C.fp8_block_dequant(x, s, 128, 0))
+    y1 = slime_amd.weight_dequant_bf16_scale(xg, sg)
+    assert I.same_bits(y1.cpu(), C.fp8_block_dequant(x, s, 128, 1))
+    # default dtype float32 (torch's default): the un-rounded fp32 product, as the reference would give
+    y32 = slime_amd.weight_dequant(xg, sg)
+    assert y32.dtype == torch.float32
+    assert I.same_bits(y32.cpu(), x.view(E4M3).float() * T._expand_scale(s, shape[0], shape[1], 128))
+
+
+def test_dequant_reference_kat(cuda):
+    # tests/test_hf_to_megatron.py:345-358 of the reference
+    w = torch.linspace(-2, 2, 128 * 128).view(128, 128).to(E4M3)
+    s = torch.tensor([[2.0]])
+    got = slime_amd.weight_dequant_bf16_scale(w.to(cuda), s.to(cuda))
+    assert got.dtype == torch.bfloat16 and torch.equal(got.cpu(), w.to(torch.bfloat16) * 2)
+
+
+def test_dequant_asserts_like_reference(cuda):
+    x = I.fp8_codes(128, 256).to(cuda).view(E4M3)
+    s = torch.ones(1, 2, device=cuda)
+    with pytest.raises(AssertionError):
+        slime_amd.weight_dequant(x.t(), s)
+    with pytest.raises(AssertionError):
+        slime_amd.weight_dequant(x.view(-1), s)
+
+
+# ------------------------------------------------------------------ grouped launches
+
+def test_quant_plan_equals_single_calls(cuda):
+    shapes = [(4096, 2560), (1024, 2560), (1024, 2560), (2560, 4096), (300, 200), (7, 7168), (129, 127), (128, 128)]
+    ws = [I.zero_blocks(I.weights(*sh, seed=i), 0.1, seed=i) for i, sh in enumerate(shapes)]
+    wg = [w.to(cuda) for w in ws]
+    wg[2] = wg[2].t().contiguous().t()      # a strided member: generic path inside the grouped launch
+    ws[2] = ws[2]
+    for mode in (0, 1):
+        plan = slime_amd.Fp8QuantPlan(wg, (128, 128), mode)
+        outs = plan.run()
+        for w, (q, s) in zip(ws, outs):
+            qo, so = C.fp8_block_quant(w, (128, 128), mode)
+            assert torch.equal(_codes(q), qo) and torch.equal(_bits32(s), _bits32(so))
+        # second run after the inputs changed in place: the plan reads current contents
+        wg[0].mul_(2)
+        outs = plan.run()
+        qo, so = C.fp8_block_quant((ws[0].float() * 2).to(torch.bfloat16), (128, 128), mode)
+        assert torch.equal(_codes(outs[0][0]), qo) and torch.equal(_bits32(outs[0][1]), _bits32(so))
+        wg[0].div_(2)
+
+
+def test_dequant_plan_equals_single_calls(cuda):
+    shapes = [(2048, 7168), (7168, 2048), (300, 200), (16, 1024), (5, 1000)]
+    xs = [I.fp8_codes(*sh, seed=i) for i, sh in enumerate(shapes)]
+    ss = [I.log_uniform_scales(-(-sh[0] // 128), -(-sh[1] // 128), seed=i) for i, sh in enumerate(shapes)]
+    plan = slime_amd.Fp8DequantPlan([x.to(cuda).view(E4M3) for x in xs], [s.to(cuda) for s in ss])
+    for x, s, y in zip(xs, ss, plan.run()):
+        assert I.same_bits(y.cpu(), C.fp8_block_dequant(x, s, 128, 0))
+
+
+# ------------------------------------------------------------------ full-size configurations
+
+def test_qwen3_4b_layer_all_linears(cuda):
+    # one decoder layer of the Qwen3-4B-shaped state dict (q, k, v, o, gate, up, down), grouped launch
+    shapes = {"q": (4096, 2560), "k": (1024, 2560), "v": (1024, 2560), "o": (2560, 4096),
+              "gate": (9728, 2560), "up": (9728, 2560), "down": (2560, 9728)}
+    ws = {n: I.weights(*sh, seed=100 + i, outlier_p=0) for i, (n, sh) in enumerate(shapes.items())}
+    outs = slime_amd.block_fp8_many([w.to(cuda) for w in ws.values()], (128, 128))
+    for (n, w), (q, s) in zip(ws.items(), outs):
+        qo, so = C.fp8_block_quant(w, (128, 128), 0)
+        assert torch.equal(_codes(q), qo) and torch.equal(_bits32(s), _bits32(so)), n
+
+
+def test_golden_fixtures(cuda):
+    from safetensors.torch import load_file
+
+    f = load_file(os.path.join(GOLDEN, "fp8_golden.safetensors"))
+    for case in sorted({k.split("/")[0] for k in f}):
+        w = f[f"{case}/w"]
+        q, s = slime_amd.block_fp8(w.to(cuda), (128, 128))
+        assert torch.equal(_codes(q), f[f"{case}/q_block"].view(torch.uint8)), case
+        assert torch.equal(_bits32(s), _bits32(f[f"{case}/s_block"])), case
+        q, s = slime_amd.blockwise_cast_to_fp8_triton(w.to(cuda), (128, 128))
+        assert torch.equal(_codes(q), f[f"{case}/q_cast"].view(torch.uint8)), case
+        assert torch.equal(_bits32(s), _bits32(f[f"{case}/s_cast"])), case
+        d = slime_amd.fp8._dequant(f[f"{case}/q_block"].to(cuda), f[f"{case}/s_block"].to(cuda), 128, 0,
+                                   torch.bfloat16, "golden")
+        assert I.same_bits(d.cpu(), f[f"{case}/deq"]), case

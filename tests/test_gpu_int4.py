@@ -1,0 +1,155 @@
+"""HIP INT4 kernels (through the C ABI) against the CPU oracle: bit-exact words, codes and scales."""
+
+import os
+
+import pytest
+import torch
+
+import slime_amd
+from oracle import c_oracle as C
+from tests import wq_inputs as I
+
+pytestmark = pytest.mark.gpu
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def _check_pack(w, cuda, gs=128):
+    p, s, z = slime_amd.pack_layer(w.to(cuda), gs, True)
+    assert z is None and p.dtype == torch.int32 and s.dtype == torch.bfloat16
+    assert p.is_contiguous() and s.is_contiguous()
+    po, so, _ = C.int4_pack_layer(w, gs, True)
+    assert p.shape == po.shape and s.shape == so.shape
+    nbad = int((p.cpu() != po).sum())
+    assert nbad == 0, f"{nbad} packed-word mismatches"
+    assert I.same_bits(s.cpu(), so)
+
+
+@pytest.mark.parametrize("shape", [(768, 2048), (2048, 768), (16, 256), (33, 768), (1, 128), (7, 7168), (1000, 2560)])
+def test_pack_layer_g128(cuda, shape):
+    w = I.weights(*shape, seed=shape[1])
+    w[0, :128] = 0
+    _check_pack(w, cuda)
+
+
+@pytest.mark.parametrize("gs,shape", [(32, (24, 96)), (32, (768, 2048)), (64, (8, 512)), (64, (333, 1024)),
+                                      (256, (16, 1024)), (96, (8, 480)), (512, (4, 2048))])
+def test_pack_layer_other_groups(cuda, gs, shape):
+    _check_pack(I.weights(*shape, seed=gs), cuda, gs)
+
+
+def test_pack_layer_special_values(cuda):
+    rows = [I.subnormal_block(4, 1024, seed=1), I.near_max_block(4, 1024, seed=2, amax=7e-5),
+            I.near_max_block(4, 1024, seed=3, amax=3.0e38), torch.zeros(4, 1024, dtype=torch.bfloat16),
+            -torch.zeros(4, 1024, dtype=torch.bfloat16), I.weights(4, 1024, seed=4, std=1e-6)]
+    _check_pack(torch.cat(rows), cuda)
+
+
+def test_pack_layer_every_bf16_value(cuda):
+    vals = I.finite_bf16_values()
+    g = I.gen(3)
+    for ab in torch.randint(1, 0x7F80, (24,), generator=g).tolist() + [0x3728, 0x3727, 0x3880, 0x7F7F]:
+        amax = torch.tensor([ab], dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+        x = vals[vals.abs() <= amax]
+        x = torch.cat([x, torch.zeros((-x.numel()) % 128, dtype=torch.bfloat16)]).view(-1, 128)
+        x[:, 0] = amax
+        _check_pack(x, cuda)
+
+
+def test_pack_layer_strided_rows(cuda):
+    base = I.weights(64, 1536, seed=9)
+    bg = base.to(cuda)
+    for v in (lambda t: t[:, 256:1280], lambda t: t[::2], lambda t: t[:, 8:1032]):
+        w, wg = v(base), v(bg)
+        p, s, _ = slime_amd.pack_layer(wg, 128, True)
+        po, so, _ = C.int4_pack_layer(w.contiguous(), 128, True)
+        assert torch.equal(p.cpu(), po) and I.same_bits(s.cpu(), so)
+
+
+def test_pack_layer_ragged_n_fails_like_reference(cuda):
+    w = I.weights(4100, 3000, seed=1).to(cuda)
+    with pytest.raises(RuntimeError):
+        slime_amd.pack_layer(w, 128, True)      # the reference fails in .view(M, 1, N // 128, 128)
+
+
+@pytest.mark.parametrize("block", [(1, 32), (1, 128), (1, 64), (32, 1), (4, 8), (2, 16), (1, 256)])
+@pytest.mark.parametrize("sym", [True, False])
+def test_fake_quant(cuda, block, sym):
+    w = I.weights(70, 300, seed=block[0] * 100 + block[1])
+    for x in (w, w.float(), w.t()):
+        q, s, z = slime_amd.fake_int4_quant_cuda(x.to(cuda), block, sym)
+        assert q.dtype == x.dtype and s.dtype == x.dtype and z.dtype == x.dtype
+        qo, so, zo = C.int4_fake_quant(x, block, sym)
+        assert I.same_bits(q.cpu(), qo) and I.same_bits(s.cpu(), so) and I.same_bits(z.cpu(), zo)
+
+
+def test_fake_quant_ragged_big(cuda):
+    w = I.weights(4100, 3000, seed=2)
+    q, s, z = slime_amd.fake_int4_quant_cuda(w.to(cuda), (1, 128), True)
+    qo, so, zo = C.int4_fake_quant(w, (1, 128), True)
+    assert s.shape == (4100, 24)
+    assert I.same_bits(q.cpu(), qo) and I.same_bits(s.cpu(), so) and I.same_bits(z.cpu(), zo)
+
+
+def test_fake_quant_errors(cuda):
+    w = torch.zeros(64, 64, dtype=torch.bfloat16, device=cuda)
+    with pytest.raises(RuntimeError, match="divisible by 32"):
+        slime_amd.fake_int4_quant_cuda(w, (1, 48), True)
+    with pytest.raises(RuntimeError, match="2D"):
+        slime_amd.fake_int4_quant_cuda(w.view(-1), (1, 32), True)
+    with pytest.raises(RuntimeError, match="not supported"):
+        slime_amd.fake_int4_quant_cuda(w, (2, 64), True)
+    with pytest.raises(RuntimeError, match="positive"):
+        slime_amd.fake_int4_quant_cuda(w, (0, 32), True)
+
+
+@pytest.mark.parametrize("shape,gs", [((16, 256), 128), ((8, 2048), 128), ((24, 96), 32)])
+def test_pack_layer_asym(cuda, shape, gs):
+    w = I.weights(*shape, seed=shape[1])
+    p, s, z = slime_amd.pack_layer(w.to(cuda), gs, False)
+    po, so, zo = C.int4_pack_layer(w, gs, False)
+    assert torch.equal(p.cpu(), po) and I.same_bits(s.cpu(), so) and torch.equal(z.cpu(), zo)
+
+
+def test_pack_plan_moe_experts(cuda):
+    # Qwen3-30B-A3B expert shapes: 8 experts x {gate, up [768,2048], down [2048,768]} in one launch
+    ws = []
+    for e in range(8):
+        ws += [I.weights(768, 2048, seed=3 * e), I.weights(768, 2048, seed=3 * e + 1), I.weights(2048, 768, seed=3 * e + 2)]
+    plan = slime_amd.Int4PackPlan([w.to(cuda) for w in ws], 128)
+    for w, (p, s) in zip(ws, plan.run()):
+        po, so, _ = C.int4_pack_layer(w, 128, True)
+        assert torch.equal(p.cpu(), po) and I.same_bits(s.cpu(), so)
+    # reconstruction error bound: |w - (nib-8)*scale| <= scale/2 (+ bf16 rounding of the scale)
+    p, s = plan.outputs[0]
+    nib = torch.stack([(p >> (4 * j)) & 0xF for j in range(8)], dim=-1).view(768, 2048).float() - 8
+    sf = s.float().repeat_interleave(128, dim=1)
+    assert ((nib * sf - ws[0].to(cuda).float()).abs() <= sf * (0.5 + 7 * 2 ** -8)).all()
+
+
+def test_int4_golden(cuda):
+    from safetensors.torch import load_file
+
+    f = load_file(os.path.join(GOLDEN, "int4_golden.safetensors"))
+    for case in sorted({k.split("/")[0] for k in f}):
+        w = f[f"{case}/w"].to(cuda)
+        gs = int(case.split("_")[0][1:])
+        q, s, _ = slime_amd.fake_int4_quant_cuda(w, (1, gs), True)
+        assert I.same_bits(q.cpu(), f[f"{case}/q"]) and I.same_bits(s.cpu(), f[f"{case}/scale"]), case
+        p, s2, _ = slime_amd.pack_layer(w, gs, True)
+        assert torch.equal(p.cpu(), f[f"{case}/packed"]) and I.same_bits(s2.cpu(), f[f"{case}/pack_scale"]), case
+        if f"{case}/packed_asym" in f:
+            pa, _, pz = slime_amd.pack_layer(w, gs, False)
+            assert torch.equal(pa.cpu(), f[f"{case}/packed_asym"]) and torch.equal(pz.cpu(), f[f"{case}/packed_zp"])
+
+
+def test_pack_helpers_on_gpu(cuda):
+    g = I.gen(0)
+    q = torch.randint(-8, 8, (9, 37), generator=g, dtype=torch.int32).to(torch.int8)
+    from oracle import torch_ref as T
+
+    assert torch.equal(slime_amd.pack_to_int32(q.to(cuda), 4, sym=True).cpu(), T.pack_to_int32_ref(q, 4, sym=True))
+    with pytest.raises(ValueError):
+        slime_amd.pack_to_int32(q.to(cuda), 9)
+    x = I.weights(8, 256, seed=1)
+    sc = (x.float().abs().view(8, 2, 128).amax(-1) / 7).to(torch.bfloat16)
+    assert torch.equal(slime_amd.quantize(x.to(cuda), sc.to(cuda), None).cpu(), T.quantize_ref(x, sc, None))

@@ -1,0 +1,57 @@
+"""Exhaustive on-device checks of the shortcuts the production kernels take (GPU only).
+
+The kernels replace the reference's per-element IEEE division by a reciprocal + two-FMA refinement and
+its software casts by gfx950 conversion instructions.  Each shortcut is compared with the literal
+arithmetic over its complete input domain."""
+
+import pytest
+import torch
+
+from slime_amd import _lib
+
+pytestmark = pytest.mark.gpu
+
+
+def _run(fn, *args):
+    out = torch.zeros(2, dtype=torch.int64, device="cuda")
+    rc = fn(*args, out.data_ptr(), torch.cuda.current_stream().cuda_stream)
+    _lib.check(rc, "selftest")
+    torch.cuda.synchronize()
+    count, first = out.tolist()
+    return count, first & 0xFFFFFFFFFFFFFFFF
+
+
+@pytest.mark.parametrize("mode", [0, 1])
+def test_fp8_element_function_whole_domain(cuda, mode):
+    # every finite bf16 amax x every bf16 x with |x| <= amax: 2^31 pairs
+    count, first = _run(_lib.load().wq_selftest_fp8_elem, 0, 0x7F80, mode)
+    assert count == 0, f"{count} mismatches, first at amax=0x{first >> 16:04x} x=0x{first & 0xFFFF:04x}"
+
+
+def test_int4_element_function_whole_domain(cuda):
+    count, first = _run(_lib.load().wq_selftest_int4_elem, 0, 0x7F80)
+    assert count == 0, f"{count} mismatches, first at amax=0x{first >> 16:04x} x=0x{first & 0xFFFF:04x}"
+
+
+def test_hw_fp32_to_e4m3_all_inputs(cuda):
+    count, first = _run(_lib.load().wq_selftest_cvt_fp8, 0, 1 << 32)
+    assert count == 0, f"{count} mismatches, first at fp32 bits 0x{first:08x}"
+
+
+def test_hw_fp32_to_bf16_all_inputs(cuda):
+    count, first = _run(_lib.load().wq_selftest_cvt_bf16, 0, 1 << 32)
+    assert count == 0, f"{count} mismatches, first at fp32 bits 0x{first:08x}"
+
+
+def test_hw_e4m3_to_fp32_all_codes(cuda):
+    count, first = _run(_lib.load().wq_selftest_decode_fp8)
+    assert count == 0, f"{count} mismatches, first code 0x{first:02x}"
+
+
+def test_copy_kernel(cuda):
+    g = torch.Generator().manual_seed(0)
+    src = torch.randint(0, 256, (1 << 20,), generator=g, dtype=torch.int32).to(torch.uint8).cuda()
+    dst = torch.zeros_like(src)
+    _lib.check(_lib.load().wq_copy_bytes(src.data_ptr(), dst.data_ptr(), src.numel(),
+                                         torch.cuda.current_stream().cuda_stream), "copy")
+    assert torch.equal(src, dst)
