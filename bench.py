@@ -178,6 +178,26 @@ def bench_fp8_dequant(dev, steps, warmup, experts):
     return out
 
 
+def bench_copy(dev, steps, warmup, nbytes=4 << 30):
+    """Plain 16-byte-per-lane copy of 4 GiB: known HBM traffic (nbytes read + nbytes written) for scaling the
+    FETCH_SIZE / WRITE_SIZE counters, and the practical bandwidth ceiling of this box."""
+    import torch
+
+    from slime_amd import _lib
+
+    src = torch.empty(nbytes, dtype=torch.uint8, device=dev).random_(0, 256)
+    dst = torch.empty_like(src)
+
+    def run():
+        _lib.check(_lib.load().wq_copy_bytes(src.data_ptr(), dst.data_ptr(), nbytes, _lib.stream_ptr(dev)), "copy")
+
+    wall_ms, ev_ms, ev_min = _time_launches(run, steps, warmup)
+    assert torch.equal(src[:1 << 20], dst[:1 << 20]) and torch.equal(src[-(1 << 20):], dst[-(1 << 20):])
+    return {"workload": "copy_kernel 4 GiB", "bytes_read": nbytes, "bytes_written": nbytes, "kernel_ms": ev_ms,
+            "kernel_ms_min": ev_min, "GBps_read_plus_write": 2 * nbytes / ev_ms / 1e6,
+            "hbm_frac": 2 * nbytes / ev_ms / 1e6 / HBM_PEAK_GBS}
+
+
 def cpu_baseline(sample, budget_s: float):
     """The CPU restatement of the reference torch path (block_fp8 op sequence) on one layer's tensors."""
     import torch
@@ -196,7 +216,7 @@ def cpu_baseline(sample, budget_s: float):
             torch_ref.block_fp8_ref(w, (128, 128))
         reps += 1
         dt = time.perf_counter() - t0
-        if dt >= budget_s or reps >= 50:
+        if dt >= budget_s or reps >= 500:
             break
     return {"value": nbytes * reps / dt / 1e9, "unit": "GB/s of bf16 weights", "cores": torch.get_num_threads(),
             "kind": "port",
@@ -214,6 +234,9 @@ def main():
     ap.add_argument("--dequant-experts", type=int, default=256)
     ap.add_argument("--no-extras", action="store_true", help="headline workload only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--only", choices=["int4", "dequant", "copy"], default=None,
+                    help="profiling aid: run just one of the other kernels (or the plain copy kernel that hardware "
+                         "counters are calibrated against) and print its record")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures ONE GPU: the path has no cross-GPU exchange and this build has no multi-GPU "
@@ -227,6 +250,16 @@ def main():
         sys.exit(2)
     dev = torch.device("cuda:0")
     torch.manual_seed(0)
+
+    if args.only == "int4":
+        print(json.dumps(bench_int4_pack(dev, args.steps, args.warmup, args.int4_layers)))
+        return
+    if args.only == "dequant":
+        print(json.dumps(bench_fp8_dequant(dev, args.steps, args.warmup, args.dequant_experts)))
+        return
+    if args.only == "copy":
+        print(json.dumps(bench_copy(dev, args.steps, args.warmup)))
+        return
 
     r = bench_fp8_quant(dev, args.steps, args.warmup)
     achieved = r["algo_bytes"] / r["kernel_ms"] / 1e6      # GB/s

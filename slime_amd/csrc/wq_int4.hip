@@ -63,6 +63,36 @@ __device__ __forceinline__ uint32_t pack8_sym(const u32x4& v, float scale, float
     return w;
 }
 
+// Scales at or above 2^121 (bf16 bits 0x7C00): the reference's dequantise / re-quantise chain is no
+// longer the identity there - bf16(7 * scale) can overflow to infinity, which its clamp turns into the
+// code 127 and its packing sum then carries into the neighbouring nibbles.  Such groups (weights of
+// magnitude ~1e37) take the literal chain so that even this corner packs the words the reference packs.
+constexpr uint32_t kLiteralChainScaleBits = 0x7C00u;
+
+__device__ __forceinline__ float bf16_round(float f) { return u2f(f32_to_bf16_bits(f) << 16); }
+
+__device__ __forceinline__ uint32_t code_literal(float x, float scale, float sb)
+{
+    const float q = __builtin_rintf(x / scale);
+    const float d = bf16_round(q * sb);
+    float r = bf16_round(d / sb);
+    if (r == r) r = fminf(fmaxf(r, -128.0f), 127.0f);
+    return (uint32_t)((int)__builtin_rintf(r) + 8) & 0xFFu;  // int8 + 8, reinterpreted as uint8
+}
+
+__device__ __forceinline__ uint32_t pack8_literal(const u32x4& v, float scale, float sb)
+{
+    uint32_t w = code_literal(bf16lo(v.x), scale, sb);
+    w += code_literal(bf16hi(v.x), scale, sb) << 4;
+    w += code_literal(bf16lo(v.y), scale, sb) << 8;
+    w += code_literal(bf16hi(v.y), scale, sb) << 12;
+    w += code_literal(bf16lo(v.z), scale, sb) << 16;
+    w += code_literal(bf16hi(v.z), scale, sb) << 20;
+    w += code_literal(bf16lo(v.w), scale, sb) << 24;
+    w += code_literal(bf16hi(v.w), scale, sb) << 28;
+    return w;
+}
+
 // Contiguous tensors only: group g of the tensor starts at x + g*G, its packed words at
 // packed + g*L, its scale at scale[g].
 template <int L, bool GROUPED>
@@ -99,10 +129,12 @@ __global__ __launch_bounds__(256) void int4_pack_kernel(const Int4PackArgs a, co
         m = lanes_max_u32<L>(pk_fold(m));
         const float scale = int4_scale_sym(u2f(m << 16));
         const float rcp = 1.0f / scale;
-        const uint32_t w = pack8_sym(v[i], scale, rcp);
+        uint32_t w = pack8_sym(v[i], scale, rcp);
+        const uint32_t sb_bits = f32_to_bf16_bits(scale);
+        if (sb_bits >= kLiteralChainScaleBits) w = pack8_literal(v[i], scale, u2f(sb_bits << 16));
         if (g < d.n_groups) {
             __builtin_nontemporal_store(w, (uint32_t*)d.packed + g * L + ll);
-            if (ll == 0) ((uint16_t*)d.scale)[g] = (uint16_t)f32_to_bf16_bits(scale);
+            if (ll == 0) ((uint16_t*)d.scale)[g] = (uint16_t)sb_bits;
         }
     }
 }
@@ -126,13 +158,16 @@ __global__ __launch_bounds__(256) void int4_pack_generic_kernel(const uint16_t* 
     m = lanes_max_u32<16>(m);
     const float scale = int4_scale_sym(u2f(m << 16));
     if (!live) return;
-    if (ll == 0) scale_out[g] = (uint16_t)f32_to_bf16_bits(scale);
+    const uint32_t sb_bits = f32_to_bf16_bits(scale);
+    if (ll == 0) scale_out[g] = (uint16_t)sb_bits;
+    const bool literal = sb_bits >= kLiteralChainScaleBits;
+    const float sb = u2f(sb_bits << 16);
     uint32_t* pg = packed + row * (N / 8) + gi * (group / 8);
     for (int wi = ll; wi < group / 8; wi += 16) {
         uint32_t w = 0;
         for (int j = 0; j < 8; ++j) {
-            float q = u2f((uint32_t)xg[wi * 8 + j] << 16) / scale;
-            w |= nibble_of(q) << (4 * j);
+            const float xv = u2f((uint32_t)xg[wi * 8 + j] << 16);
+            w += (literal ? code_literal(xv, scale, sb) : nibble_of(xv / scale)) << (4 * j);
         }
         pg[wi] = w;
     }

@@ -58,7 +58,8 @@ def test_block_quant_config1_roundtrip(cuda):
     assert d.dtype == torch.bfloat16
     assert I.same_bits(d.cpu(), C.fp8_block_dequant(_codes(q), s.cpu(), 128, 0))
     step = s.cpu().repeat_interleave(128, 0).repeat_interleave(128, 1) * 32
-    assert ((d.cpu().float() - w.float()).abs() <= step / 2 * 1.01).all()
+    # half an e4m3 step of the block, plus the bf16 rounding of the dequantised value
+    assert ((d.cpu().float() - w.float()).abs() <= step / 2 * 1.01 + w.float().abs() * 2.0 ** -7).all()
 
 
 def test_block_quant_tall_ragged(cuda):

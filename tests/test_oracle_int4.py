@@ -185,3 +185,19 @@ def test_pack_layer_sym_equals_direct_formula():
         want += (q[:, j::8].to(torch.int64) + 8) << (4 * j)
     want = torch.where(want >= 2 ** 31, want - 2 ** 32, want).to(torch.int32)
     assert torch.equal(p, want) and I.same_bits(s, s2)
+
+
+def test_pack_layer_extreme_scales_where_the_chain_is_not_the_identity():
+    # bf16(7 * scale) overflows to infinity for scales near 2^125: the chain then yields code 127 and the
+    # packing sum carries into neighbouring nibbles.  Both oracles must agree on that corner too.
+    w = I.near_max_block(8, 256, seed=3, amax=3.0e38)
+    w[1] = I.near_max_block(1, 256, seed=4, amax=3.3895e38)[0]
+    p, s, _ = C.int4_pack_layer(w, 128, True)
+    pr, sr, _ = T.pack_layer_ref(w, 128, True)
+    assert torch.equal(p, pr) and I.same_bits(s, sr)
+    q, _, _ = C.int4_fake_quant(w, (1, 128), True)
+    direct = torch.zeros(8, 32, dtype=torch.int64)
+    for j in range(8):
+        direct += (q[:, j::8].to(torch.int64) + 8) << (4 * j)
+    direct = torch.where(direct >= 2 ** 31, direct - 2 ** 32, direct).to(torch.int32)
+    assert not torch.equal(p, direct)      # the corner is real: the literal chain differs from the direct formula
