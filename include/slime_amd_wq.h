@@ -114,9 +114,10 @@ typedef struct wq_fp8_dequant_desc {
 } wq_fp8_dequant_desc;
 
 /* Grouped form: `descs` DEVICE array, `work_start` DEVICE int64[n_desc+1] exclusive prefix sum of
- * per-tensor work items, where a tensor has ceil(M/WQ_DEQ_ROWS) * ceil(N/WQ_DEQ_COLS) items. */
-#define WQ_DEQ_ROWS 16
-#define WQ_DEQ_COLS 1024
+ * per-tensor work items, where a tensor has ceil(M * ceil(N/WQ_DEQ_SEG) / WQ_DEQ_SEGS_PER_WG) items
+ * (rows are cut into segments of WQ_DEQ_SEG codes; a work item is WQ_DEQ_SEGS_PER_WG consecutive segments). */
+#define WQ_DEQ_SEG 512
+#define WQ_DEQ_SEGS_PER_WG 32
 int wq_fp8_block_dequant_grouped(const wq_fp8_dequant_desc *descs, const int64_t *work_start, int n_desc,
                                  int64_t total_work, int out_dtype, int block, int mode, void *stream);
 

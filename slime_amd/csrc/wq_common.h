@@ -79,6 +79,23 @@ __device__ __forceinline__ uint32_t cvt_pk_fp8_hi(float a, float b, uint32_t old
     return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(a, b, (int)old, true);
 }
 
+// ---- work-item order ------------------------------------------------------------------------
+// Workgroups are dealt to the eight XCDs round-robin in dispatch order, and every XCD has its own L2
+// and address-translation cache.  A streaming kernel is measurably faster (about +10 points of HBM
+// utilisation on the block quantiser) when each XCD walks a contiguous run of work items instead of
+// every eighth one.  Within each span of 8*C dispatch slots, XCD k therefore takes items
+// [k*C, (k+1)*C) of the span; slots past the last full span keep the identity order.  The map is a
+// bijection on [0, total).
+constexpr int kXcds = 8;
+__device__ __forceinline__ int64_t xcd_chunked_item(int64_t slot, int64_t total, int C)
+{
+    const int64_t span = (int64_t)kXcds * C;
+    const int64_t blk = slot / span;
+    if ((blk + 1) * span > total) return slot;
+    const int r = (int)(slot - blk * span);
+    return blk * span + (int64_t)(r % kXcds) * C + r / kXcds;
+}
+
 // ---- 16-lane (DPP row) all-reduce max.  After it every lane of the row holds the row max.
 template <int CTRL>
 __device__ __forceinline__ uint32_t dpp_u32(uint32_t v)

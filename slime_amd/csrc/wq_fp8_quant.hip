@@ -17,6 +17,13 @@
 
 namespace wq {
 
+// Measured on MI355X (7.3 GB of 128x128 tiles, row widths 2560 / 4096 / 9728): runs of 32 consecutive tiles
+// per XCD and at most four resident workgroups per CU (enforced with unused dynamic LDS) reach 76-81 % of
+// the HBM peak against 69-71 % for plain dispatch order at full occupancy; neighbouring settings (runs of
+// 24-64 tiles, 3-6 workgroups) are within two points.
+constexpr int kTilesPerXcdRun = 32;
+constexpr unsigned kOccupancyPadBytes = 36 * 1024;
+
 struct Fp8QuantArgs {
     wq_fp8_quant_desc d;  // single-tensor launch: descriptor travels in the kernel arguments
     const wq_fp8_quant_desc* descs;
@@ -151,8 +158,9 @@ template <int MODE, bool GROUPED>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 8))) void fp8_block_quant_kernel(const Fp8QuantArgs a, const int64_t total_tiles)
 {
     __shared__ __attribute__((aligned(16))) uint32_t lds[16];
-    const int64_t tile = (int64_t)blockIdx.x + (int64_t)blockIdx.y * gridDim.x;
-    if (tile >= total_tiles) return;  // uniform per workgroup
+    const int64_t slot = (int64_t)blockIdx.x + (int64_t)blockIdx.y * gridDim.x;
+    if (slot >= total_tiles) return;  // uniform per workgroup
+    const int64_t tile = xcd_chunked_item(slot, total_tiles, kTilesPerXcdRun);
 
     wq_fp8_quant_desc d;
     int64_t local = tile;
@@ -256,9 +264,9 @@ WQ_EXPORT int wq_fp8_block_quant(const void* x, int64_t M, int64_t N, int64_t sx
     const int64_t tiles = cdiv64(M, bm) * cdiv64(N, bn);
     hipStream_t st = (hipStream_t)stream;
     if (mode == WQ_FP8_MODE_TORCH)
-        fp8_block_quant_kernel<WQ_FP8_MODE_TORCH, false><<<grid_for_items(tiles), 256, 0, st>>>(a, tiles);
+        fp8_block_quant_kernel<WQ_FP8_MODE_TORCH, false><<<grid_for_items(tiles), 256, kOccupancyPadBytes, st>>>(a, tiles);
     else
-        fp8_block_quant_kernel<WQ_FP8_MODE_TRITON, false><<<grid_for_items(tiles), 256, 0, st>>>(a, tiles);
+        fp8_block_quant_kernel<WQ_FP8_MODE_TRITON, false><<<grid_for_items(tiles), 256, kOccupancyPadBytes, st>>>(a, tiles);
     WQ_LAUNCH_CHECK();
     return WQ_OK;
 }
@@ -279,9 +287,9 @@ WQ_EXPORT int wq_fp8_block_quant_grouped(const wq_fp8_quant_desc* descs, const i
     a.bn = bn;
     hipStream_t st = (hipStream_t)stream;
     if (mode == WQ_FP8_MODE_TORCH)
-        fp8_block_quant_kernel<WQ_FP8_MODE_TORCH, true><<<grid_for_items(total_tiles), 256, 0, st>>>(a, total_tiles);
+        fp8_block_quant_kernel<WQ_FP8_MODE_TORCH, true><<<grid_for_items(total_tiles), 256, kOccupancyPadBytes, st>>>(a, total_tiles);
     else
-        fp8_block_quant_kernel<WQ_FP8_MODE_TRITON, true><<<grid_for_items(total_tiles), 256, 0, st>>>(a, total_tiles);
+        fp8_block_quant_kernel<WQ_FP8_MODE_TRITON, true><<<grid_for_items(total_tiles), 256, kOccupancyPadBytes, st>>>(a, total_tiles);
     WQ_LAUNCH_CHECK();
     return WQ_OK;
 }

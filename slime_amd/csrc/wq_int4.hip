@@ -18,6 +18,7 @@
 namespace wq {
 
 constexpr int kGroupsPerWg = WQ_INT4_GROUPS_PER_WG;
+constexpr int kPackItemsPerXcdRun = 32;  // 32 work items = 512 KiB of contiguous input per XCD run
 
 struct Int4PackArgs {
     wq_int4_pack_desc d;
@@ -100,8 +101,9 @@ __global__ __launch_bounds__(256) void int4_pack_kernel(const Int4PackArgs a, co
 {
     constexpr int CL = 256 / L;              // groups per step of the workgroup
     constexpr int STEPS = kGroupsPerWg / CL; // 1 (L=4), 2 (L=8), 4 (L=16)
-    const int64_t item = (int64_t)blockIdx.x + (int64_t)blockIdx.y * gridDim.x;
-    if (item >= total_work) return;
+    const int64_t slot = (int64_t)blockIdx.x + (int64_t)blockIdx.y * gridDim.x;
+    if (slot >= total_work) return;
+    const int64_t item = xcd_chunked_item(slot, total_work, kPackItemsPerXcdRun);
     wq_int4_pack_desc d;
     int64_t local = item;
     if (GROUPED) {

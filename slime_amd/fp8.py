@@ -242,7 +242,7 @@ class Fp8DequantPlan:
             y = self.flat_y[o:o + M * N].view(M, N)
             self.outputs.append(y)
             rows.append([x.data_ptr(), s.data_ptr(), y.data_ptr(), M, N])
-            work += ceildiv(M, _lib.DEQ_ROWS) * ceildiv(N, _lib.DEQ_COLS)
+            work += ceildiv(M * ceildiv(N, _lib.DEQ_SEG), _lib.DEQ_SEGS_PER_WG)
             starts.append(work)
         self.total_work = work
         self.out_bytes = sum(x.numel() * esz for x in self.xs)
