@@ -115,7 +115,9 @@ typedef struct wq_fp8_dequant_desc {
 
 /* Grouped form: `descs` DEVICE array, `work_start` DEVICE int64[n_desc+1] exclusive prefix sum of
  * per-tensor work items, where a tensor has ceil(M * ceil(N/WQ_DEQ_SEG) / WQ_DEQ_SEGS_PER_WG) items
- * (rows are cut into segments of WQ_DEQ_SEG codes; a work item is WQ_DEQ_SEGS_PER_WG consecutive segments). */
+ * (rows are cut into segments of WQ_DEQ_SEG codes; a work item is WQ_DEQ_SEGS_PER_WG consecutive segments).
+ * Per tensor, N and M * ceil(N/WQ_DEQ_SEG) must be below 2^31 (the single-tensor entry point checks this and
+ * returns WQ_ERR_TOO_LARGE; for the grouped form it is the caller's obligation). */
 #define WQ_DEQ_SEG 512
 #define WQ_DEQ_SEGS_PER_WG 32
 int wq_fp8_block_dequant_grouped(const wq_fp8_dequant_desc *descs, const int64_t *work_start, int n_desc,

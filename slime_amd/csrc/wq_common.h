@@ -96,6 +96,29 @@ __device__ __forceinline__ int64_t xcd_chunked_item(int64_t slot, int64_t total,
     return blk * span + (int64_t)(r % kXcds) * C + r / kXcds;
 }
 
+// Owner of flat work item t in a grouped launch: the largest i with start[i] <= t, where start[] is the
+// exclusive prefix sum of per-tensor item counts (n + 1 entries, start[n] = total > t).  The first probe
+// is the proportional guess - exact when all tensors have equally many items (the experts of a layer) -
+// and the binary search only runs on the side of the guess that holds t.  All values are
+// workgroup-uniform, so this is scalar code.
+__device__ __forceinline__ int find_owner(const int64_t* __restrict__ start, int n, int64_t t, int64_t total)
+{
+    int g = (int)((float)t * ((float)n / (float)total));
+    g = g < 0 ? 0 : (g > n - 1 ? n - 1 : g);
+    int lo = 0, hi = n;
+    if (start[g] <= t) {
+        if (t < start[g + 1]) return g;
+        lo = g + 1;
+    } else {
+        hi = g;
+    }
+    while (hi - lo > 1) {  // invariant: start[lo] <= t < start[hi]
+        const int mid = (lo + hi) >> 1;
+        if (start[mid] <= t) lo = mid; else hi = mid;
+    }
+    return lo;
+}
+
 // ---- 16-lane (DPP row) all-reduce max.  After it every lane of the row holds the row max.
 template <int CTRL>
 __device__ __forceinline__ uint32_t dpp_u32(uint32_t v)
@@ -240,6 +263,41 @@ __device__ __forceinline__ uint32_t fp8_quant4_exact(uint32_t w0, uint32_t w1, c
 // ---- INT4 ---------------------------------------------------------------------------------
 
 __device__ __forceinline__ float int4_scale_sym(float amax) { return fmaxf(amax * (1.0f / 7.0f), 1e-5f); }
+
+// rintf(q) + 8 in the low four bits: 12582912 = 1.5 * 2^23 makes the add round q to an integer
+// (half to even) and leaves it, offset by 8, in the low mantissa bits.
+constexpr float kRoundMagic = 12582920.0f;        // 1.5 * 2^23 + 8
+constexpr uint32_t kRoundMagicBits = 0x4B400000u;  // bits of (kRoundMagic + n) are kRoundMagicBits + n for n in 0..15
+__device__ __forceinline__ uint32_t nibble_of(float q) { return f2u(q + kRoundMagic) & 0xFu; }
+
+// Sum over j of (kRoundMagicBits << 4j) modulo 2^32: what the un-masked accumulation of pack8_sym
+// carries on top of the packed nibbles.
+constexpr uint32_t magic_carry()
+{
+    uint32_t s = 0;
+    for (int j = 0; j < 8; ++j) s += (uint32_t)((uint64_t)kRoundMagicBits << (4 * j));
+    return s;
+}
+
+// Correctly rounded 1/scale from the hardware approximation and one Newton step; equal to the IEEE
+// reciprocal for every scale the symmetric rule can produce from a bf16 amax (wq_selftest_int4_elem
+// checks it together with the quotients).
+__device__ __forceinline__ float rcp_refined(float s)
+{
+    const float r0 = __builtin_amdgcn_rcpf(s);
+    return __builtin_fmaf(__builtin_fmaf(-s, r0, 1.0f), r0, r0);
+}
+
+// Eight exact quotients -> one packed word.  For |rintf(q)| <= 7 the float q + kRoundMagic has the bit
+// pattern kRoundMagicBits + (rintf(q) + 8), so the words can be shifted and added without masking and the
+// constant part removed once at the end: one add and one shift-add per element.
+__device__ __forceinline__ uint32_t pack8_sym(const float (&x)[8], float scale, float rcp)
+{
+    uint32_t acc = f2u(div_by_scale(x[0], scale, rcp) + kRoundMagic);
+#pragma unroll
+    for (int j = 1; j < 8; ++j) acc += f2u(div_by_scale(x[j], scale, rcp) + kRoundMagic) << (4 * j);
+    return acc - magic_carry();
+}
 
 // Host-side launch helpers.
 inline int64_t cdiv64(int64_t a, int64_t b) { return (a + b - 1) / b; }

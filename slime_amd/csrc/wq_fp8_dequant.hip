@@ -18,9 +18,11 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 
 constexpr int kSeg = WQ_DEQ_SEG;                 // codes per segment: 64 lanes x 8
-constexpr int kSegsPerWg = WQ_DEQ_SEGS_PER_WG;   // 4 waves x 8 steps
+constexpr int kSegsPerWg = WQ_DEQ_SEGS_PER_WG;   // 4 waves x kSteps
+constexpr int kSteps = kSegsPerWg / 4;           // loads in flight per lane
 constexpr int kDeqItemsPerXcdRun = 32;
-static_assert(kSeg == 512 && kSegsPerWg == 32, "kernel geometry is written for 512 x 32");
+constexpr unsigned kDeqOccupancyPadBytes = 0;
+static_assert(kSeg == 512 && kSegsPerWg % 4 == 0, "a segment is 64 lanes x 8 codes; four waves per workgroup");
 
 struct DeqArgs {
     wq_fp8_dequant_desc d;
@@ -29,16 +31,6 @@ struct DeqArgs {
     int32_t n_desc;
     int32_t block;
 };
-
-__device__ __forceinline__ int find_desc_deq(const int64_t* __restrict__ start, int n, int64_t t)
-{
-    int lo = 0, hi = n;
-    while (hi - lo > 1) {
-        int mid = (lo + hi) >> 1;
-        if (start[mid] <= t) lo = mid; else hi = mid;
-    }
-    return lo;
-}
 
 // RNE fp32 -> bf16 for two values packed in a dword (v_cvt_pk_bf16_f32).
 __device__ __forceinline__ uint32_t pack_bf16x2(float a, float b)
@@ -83,41 +75,48 @@ __global__ __launch_bounds__(256) void fp8_block_dequant_kernel(const DeqArgs a,
     wq_fp8_dequant_desc d;
     int64_t local = item;
     if (GROUPED) {
-        const int di = find_desc_deq(a.work_start, a.n_desc, item);
+        const int di = find_owner(a.work_start, a.n_desc, item, total_work);
         d = a.descs[di];
         local = item - a.work_start[di];
     } else {
         d = a.d;
     }
-    const int block = a.block;
-    const int64_t spr = (d.N + kSeg - 1) / kSeg;          // segments per row
-    const int64_t n_segs = d.M * spr;
-    const int64_t kt = (d.N + block - 1) / block;
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    // 32-bit index arithmetic: N and the tensor's segment count are below 2^31 (checked on the host)
+    const uint32_t block = (uint32_t)a.block;
+    const int bshift = (block & (block - 1)) == 0 ? __builtin_ctz(block) : -1;   // power-of-two blocks shift
+    const uint32_t N = (uint32_t)d.N;
+    const uint32_t spr = (N + kSeg - 1) / kSeg;          // segments per row
+    const uint32_t n_segs = (uint32_t)d.M * spr;
+    const uint32_t kt = (N + block - 1) / block;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
     const uint8_t* x = (const uint8_t*)d.x;
-    const bool vec = (d.N & 7) == 0 && ((uintptr_t)d.x & 7) == 0 && ((uintptr_t)d.y & 15) == 0 && (block & 7) == 0;
-    // segment of step i: consecutive segments go to consecutive waves, so one step of the workgroup
-    // covers four consecutive segments
-    const int64_t seg0 = local * kSegsPerWg + wave;
+    const bool vec = (N & 7) == 0 && ((uintptr_t)d.x & 7) == 0 && ((uintptr_t)d.y & 15) == 0 && (block & 7) == 0;
+    // segment of step i is seg0 + 4i: consecutive segments go to consecutive waves, so one step of the
+    // workgroup covers four consecutive segments.  (row, segment-in-row) advance incrementally.
+    const uint32_t seg0 = (uint32_t)local * kSegsPerWg + wave;
+    uint32_t r = seg0 / spr, c = seg0 - r * spr;
 
     if (vec) {
-        u32x2 v[8];
-        int64_t row[8];
-        int col[8];
+        u32x2 v[kSteps];
+        uint32_t row[kSteps], col[kSteps];
+        bool ok[kSteps];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const int64_t seg = seg0 + 4 * i;
-            row[i] = seg / spr;
-            col[i] = (int)(seg - row[i] * spr) * kSeg + lane * 8;
+        for (int i = 0; i < kSteps; ++i) {
+            row[i] = r;
+            col[i] = c * kSeg + lane * 8;
+            ok[i] = seg0 + 4 * i < n_segs && col[i] < N;
             v[i] = (u32x2){0u, 0u};
-            if (seg < n_segs && col[i] < d.N) v[i] = __builtin_nontemporal_load((const u32x2*)(x + row[i] * d.N + col[i]));
-            else row[i] = -1;
+            if (ok[i]) v[i] = __builtin_nontemporal_load((const u32x2*)(x + (uint64_t)row[i] * N + col[i]));
+            c += 4;
+            while (c >= spr) { c -= spr; ++r; }
         }
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            if (row[i] < 0) continue;
-            const float sc = load_scale<MODE>(d.s, (row[i] / block) * kt + col[i] / block);
-            const int64_t off = row[i] * d.N + col[i];
+        for (int i = 0; i < kSteps; ++i) {
+            if (!ok[i]) continue;
+            const uint32_t sr = bshift >= 0 ? row[i] >> bshift : row[i] / block;
+            const uint32_t sc_col = bshift >= 0 ? col[i] >> bshift : col[i] / block;
+            const float sc = load_scale<MODE>(d.s, sr * kt + sc_col);
+            const uint64_t off = (uint64_t)row[i] * N + col[i];
             if (OUT == WQ_DTYPE_BF16) {
                 const u32x2 a0 = dequant4(v[i].x, sc), a1 = dequant4(v[i].y, sc);
                 const u32x4 o = {a0.x, a0.y, a1.x, a1.y};
@@ -130,20 +129,20 @@ __global__ __launch_bounds__(256) void fp8_block_dequant_kernel(const DeqArgs a,
         }
     } else {
         // element-wise path: any N, alignment and block size
-        for (int i = 0; i < 8; ++i) {
-            const int64_t seg = seg0 + 4 * i;
-            if (seg >= n_segs) break;
-            const int64_t r = seg / spr;
-            const int64_t c0 = (seg - r * spr) * kSeg;
+        for (int i = 0; i < kSteps; ++i) {
+            if (seg0 + 4 * i >= n_segs) break;
             for (int k = 0; k < 8; ++k) {
-                const int64_t c = c0 + k * 64 + lane;
-                if (c >= d.N) break;
-                const float sc = load_scale<MODE>(d.s, (r / block) * kt + c / block);
-                const uint32_t code = x[r * d.N + c];
+                const uint32_t cc = c * kSeg + k * 64 + lane;
+                if (cc >= N) break;
+                const float sc = load_scale<MODE>(d.s, (r / block) * kt + cc / block);
+                const uint64_t off = (uint64_t)r * N + cc;
+                const uint32_t code = x[off];
                 const f32x2 f = __builtin_amdgcn_cvt_pk_f32_fp8((int)code, false);
-                if (OUT == WQ_DTYPE_BF16) ((uint16_t*)d.y)[r * d.N + c] = (uint16_t)(pack_bf16x2(f.x * sc, 0.0f) & 0xFFFFu);
-                else ((float*)d.y)[r * d.N + c] = f.x * sc;
+                if (OUT == WQ_DTYPE_BF16) ((uint16_t*)d.y)[off] = (uint16_t)(pack_bf16x2(f.x * sc, 0.0f) & 0xFFFFu);
+                else ((float*)d.y)[off] = f.x * sc;
             }
+            c += 4;
+            while (c >= spr) { c -= spr; ++r; }
         }
     }
 }
@@ -162,11 +161,11 @@ static int launch_deq(const DeqArgs& a, int64_t work, int mode, int out_dtype, h
 {
     const dim3 g = grid_for_items(work);
     if (mode == WQ_DEQ_MODE_F32SCALE) {
-        if (out_dtype == WQ_DTYPE_BF16) fp8_block_dequant_kernel<WQ_DEQ_MODE_F32SCALE, GROUPED, WQ_DTYPE_BF16><<<g, 256, 0, st>>>(a, work);
-        else fp8_block_dequant_kernel<WQ_DEQ_MODE_F32SCALE, GROUPED, WQ_DTYPE_F32><<<g, 256, 0, st>>>(a, work);
+        if (out_dtype == WQ_DTYPE_BF16) fp8_block_dequant_kernel<WQ_DEQ_MODE_F32SCALE, GROUPED, WQ_DTYPE_BF16><<<g, 256, kDeqOccupancyPadBytes, st>>>(a, work);
+        else fp8_block_dequant_kernel<WQ_DEQ_MODE_F32SCALE, GROUPED, WQ_DTYPE_F32><<<g, 256, kDeqOccupancyPadBytes, st>>>(a, work);
     } else {
-        if (out_dtype == WQ_DTYPE_BF16) fp8_block_dequant_kernel<WQ_DEQ_MODE_BF16SCALE, GROUPED, WQ_DTYPE_BF16><<<g, 256, 0, st>>>(a, work);
-        else fp8_block_dequant_kernel<WQ_DEQ_MODE_BF16SCALE, GROUPED, WQ_DTYPE_F32><<<g, 256, 0, st>>>(a, work);
+        if (out_dtype == WQ_DTYPE_BF16) fp8_block_dequant_kernel<WQ_DEQ_MODE_BF16SCALE, GROUPED, WQ_DTYPE_BF16><<<g, 256, kDeqOccupancyPadBytes, st>>>(a, work);
+        else fp8_block_dequant_kernel<WQ_DEQ_MODE_BF16SCALE, GROUPED, WQ_DTYPE_F32><<<g, 256, kDeqOccupancyPadBytes, st>>>(a, work);
     }
     WQ_LAUNCH_CHECK();
     return WQ_OK;
@@ -188,7 +187,8 @@ WQ_EXPORT int wq_fp8_block_dequant(const void* x, const float* s, void* y, int o
     if (rc) return rc;
     if (M == 0 || N == 0) return WQ_OK;
     if (!x || !s || !y) return WQ_ERR_NULL;
-    if (N >= (1ll << 31)) return WQ_ERR_TOO_LARGE;
+    // the kernel indexes rows, columns and segments with 32-bit integers
+    if (N >= (1ll << 31) || M >= (1ll << 31) || M * cdiv64(N, kSeg) >= (1ll << 31)) return WQ_ERR_TOO_LARGE;
     DeqArgs a{};
     a.d = wq_fp8_dequant_desc{x, s, y, M, N};
     a.block = block;

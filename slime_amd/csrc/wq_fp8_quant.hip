@@ -40,17 +40,6 @@ __device__ __forceinline__ bool desc_vector_ok(const wq_fp8_quant_desc& d)
            d.sy_m >= 0 && d.sy_m < (1 << 22);
 }
 
-// Finds the descriptor that owns flat tile `t`: largest i with tile_start[i] <= t.
-__device__ __forceinline__ int find_desc(const int64_t* __restrict__ start, int n, int64_t t)
-{
-    int lo = 0, hi = n;  // invariant: start[lo] <= t < start[hi]
-    while (hi - lo > 1) {
-        int mid = (lo + hi) >> 1;
-        if (start[mid] <= t) lo = mid; else hi = mid;
-    }
-    return lo;
-}
-
 template <int MODE>
 __device__ __forceinline__ void quant_tile_vec128(const wq_fp8_quant_desc& d, int64_t tm, int64_t tn, int kt,
                                                   uint32_t* lds)
@@ -165,7 +154,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 8))) voi
     wq_fp8_quant_desc d;
     int64_t local = tile;
     if (GROUPED) {
-        const int di = find_desc(a.tile_start, a.n_desc, tile);
+        const int di = find_owner(a.tile_start, a.n_desc, tile, total_tiles);
         d = a.descs[di];
         local = tile - a.tile_start[di];
     } else {

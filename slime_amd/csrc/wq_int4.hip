@@ -19,6 +19,7 @@ namespace wq {
 
 constexpr int kGroupsPerWg = WQ_INT4_GROUPS_PER_WG;
 constexpr int kPackItemsPerXcdRun = 32;  // 32 work items = 512 KiB of contiguous input per XCD run
+constexpr unsigned kPackOccupancyPadBytes = 0;
 
 struct Int4PackArgs {
     wq_int4_pack_desc d;
@@ -26,16 +27,6 @@ struct Int4PackArgs {
     const int64_t* work_start;
     int32_t n_desc;
 };
-
-__device__ __forceinline__ int find_desc_i4(const int64_t* __restrict__ start, int n, int64_t t)
-{
-    int lo = 0, hi = n;
-    while (hi - lo > 1) {
-        int mid = (lo + hi) >> 1;
-        if (start[mid] <= t) lo = mid; else hi = mid;
-    }
-    return lo;
-}
 
 template <int L>
 __device__ __forceinline__ uint32_t lanes_max_u32(uint32_t v)
@@ -47,21 +38,39 @@ __device__ __forceinline__ uint32_t lanes_max_u32(uint32_t v)
     return v;
 }
 
-// rintf(q) + 8 in the low four bits: 12582912 = 1.5 * 2^23 makes the add round q to an integer
-// (half to even) and leaves it, offset by 8, in the low mantissa bits.
-__device__ __forceinline__ uint32_t nibble_of(float q) { return f2u(q + 12582920.0f) & 0xFu; }
-
-__device__ __forceinline__ uint32_t pack8_sym(const u32x4& v, float scale, float rcp)
+__device__ __forceinline__ void unpack8(const u32x4& v, float (&x)[8])
 {
-    uint32_t w = nibble_of(div_by_scale(bf16lo(v.x), scale, rcp));
-    w |= nibble_of(div_by_scale(bf16hi(v.x), scale, rcp)) << 4;
-    w |= nibble_of(div_by_scale(bf16lo(v.y), scale, rcp)) << 8;
-    w |= nibble_of(div_by_scale(bf16hi(v.y), scale, rcp)) << 12;
-    w |= nibble_of(div_by_scale(bf16lo(v.z), scale, rcp)) << 16;
-    w |= nibble_of(div_by_scale(bf16hi(v.z), scale, rcp)) << 20;
-    w |= nibble_of(div_by_scale(bf16lo(v.w), scale, rcp)) << 24;
-    w |= nibble_of(div_by_scale(bf16hi(v.w), scale, rcp)) << 28;
-    return w;
+    x[0] = bf16lo(v.x); x[1] = bf16hi(v.x); x[2] = bf16lo(v.y); x[3] = bf16hi(v.y);
+    x[4] = bf16lo(v.z); x[5] = bf16hi(v.z); x[6] = bf16lo(v.w); x[7] = bf16hi(v.w);
+}
+
+// max |x| over the lane's eight values; fmaxf drops NaN operands exactly as the reference kernel's does
+__device__ __forceinline__ float absmax8(const float (&x)[8])
+{
+    float m = fmaxf(fabsf(x[0]), fabsf(x[1]));
+    m = fmaxf(fmaxf(m, fabsf(x[2])), fabsf(x[3]));
+    m = fmaxf(fmaxf(m, fabsf(x[4])), fabsf(x[5]));
+    m = fmaxf(fmaxf(m, fabsf(x[6])), fabsf(x[7]));
+    return m;
+}
+
+template <int L>
+__device__ __forceinline__ float lanes_max_f32(float v)
+{
+    v = fmaxf(v, u2f(dpp_u32<0xB1>(f2u(v))));
+    v = fmaxf(v, u2f(dpp_u32<0x4E>(f2u(v))));
+    if (L >= 8) v = fmaxf(v, u2f(dpp_u32<0x141>(f2u(v))));
+    if (L >= 16) v = fmaxf(v, u2f(dpp_u32<0x140>(f2u(v))));
+    return v;
+}
+
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+// fp32 -> bf16 bits, RNE, by v_cvt_pk_bf16_f32 (identical to the software rounding for all non-NaN inputs)
+__device__ __forceinline__ uint32_t bf16_bits_hw(float f)
+{
+    f32x2_t v = {f, 0.0f};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t)) & 0xFFFFu;
 }
 
 // Scales at or above 2^121 (bf16 bits 0x7C00): the reference's dequantise / re-quantise chain is no
@@ -81,16 +90,11 @@ __device__ __forceinline__ uint32_t code_literal(float x, float scale, float sb)
     return (uint32_t)((int)__builtin_rintf(r) + 8) & 0xFFu;  // int8 + 8, reinterpreted as uint8
 }
 
-__device__ __forceinline__ uint32_t pack8_literal(const u32x4& v, float scale, float sb)
+__device__ __forceinline__ uint32_t pack8_literal(const float (&x)[8], float scale, float sb)
 {
-    uint32_t w = code_literal(bf16lo(v.x), scale, sb);
-    w += code_literal(bf16hi(v.x), scale, sb) << 4;
-    w += code_literal(bf16lo(v.y), scale, sb) << 8;
-    w += code_literal(bf16hi(v.y), scale, sb) << 12;
-    w += code_literal(bf16lo(v.z), scale, sb) << 16;
-    w += code_literal(bf16hi(v.z), scale, sb) << 20;
-    w += code_literal(bf16lo(v.w), scale, sb) << 24;
-    w += code_literal(bf16hi(v.w), scale, sb) << 28;
+    uint32_t w = 0;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) w += code_literal(x[j], scale, sb) << (4 * j);
     return w;
 }
 
@@ -107,7 +111,7 @@ __global__ __launch_bounds__(256) void int4_pack_kernel(const Int4PackArgs a, co
     wq_int4_pack_desc d;
     int64_t local = item;
     if (GROUPED) {
-        const int di = find_desc_i4(a.work_start, a.n_desc, item);
+        const int di = find_owner(a.work_start, a.n_desc, item, total_work);
         d = a.descs[di];
         local = item - a.work_start[di];
     } else {
@@ -127,13 +131,12 @@ __global__ __launch_bounds__(256) void int4_pack_kernel(const Int4PackArgs a, co
 #pragma unroll
     for (int i = 0; i < STEPS; ++i) {
         const int64_t g = g0 + i * CL;
-        uint32_t m = pk_absmax(pk_absmax(pk_absmax(pk_absmax(0u, v[i].x), v[i].y), v[i].z), v[i].w);
-        m = lanes_max_u32<L>(pk_fold(m));
-        const float scale = int4_scale_sym(u2f(m << 16));
-        const float rcp = 1.0f / scale;
-        uint32_t w = pack8_sym(v[i], scale, rcp);
-        const uint32_t sb_bits = f32_to_bf16_bits(scale);
-        if (sb_bits >= kLiteralChainScaleBits) w = pack8_literal(v[i], scale, u2f(sb_bits << 16));
+        float x[8];
+        unpack8(v[i], x);
+        const float scale = int4_scale_sym(lanes_max_f32<L>(absmax8(x)));
+        uint32_t w = pack8_sym(x, scale, rcp_refined(scale));
+        const uint32_t sb_bits = bf16_bits_hw(scale);
+        if (sb_bits >= kLiteralChainScaleBits) w = pack8_literal(x, scale, u2f(sb_bits << 16));
         if (g < d.n_groups) {
             __builtin_nontemporal_store(w, (uint32_t*)d.packed + g * L + ll);
             if (ll == 0) ((uint16_t*)d.scale)[g] = (uint16_t)sb_bits;
@@ -252,9 +255,9 @@ template <bool GROUPED>
 static int launch_pack(const Int4PackArgs& a, int64_t work, int group, hipStream_t st)
 {
     switch (group) {
-    case 32: int4_pack_kernel<4, GROUPED><<<grid_for_items(work), 256, 0, st>>>(a, work); break;
-    case 64: int4_pack_kernel<8, GROUPED><<<grid_for_items(work), 256, 0, st>>>(a, work); break;
-    case 128: int4_pack_kernel<16, GROUPED><<<grid_for_items(work), 256, 0, st>>>(a, work); break;
+    case 32: int4_pack_kernel<4, GROUPED><<<grid_for_items(work), 256, kPackOccupancyPadBytes, st>>>(a, work); break;
+    case 64: int4_pack_kernel<8, GROUPED><<<grid_for_items(work), 256, kPackOccupancyPadBytes, st>>>(a, work); break;
+    case 128: int4_pack_kernel<16, GROUPED><<<grid_for_items(work), 256, kPackOccupancyPadBytes, st>>>(a, work); break;
     default: return WQ_ERR_UNSUPPORTED;
     }
     WQ_LAUNCH_CHECK();

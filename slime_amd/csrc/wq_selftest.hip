@@ -49,16 +49,26 @@ __global__ __launch_bounds__(256) void selftest_int4_elem_kernel(uint32_t amax_l
 {
     const uint32_t a = amax_lo + blockIdx.y;
     if (a >= amax_hi || a >= kBf16Inf) return;
-    const uint32_t xb = blockIdx.x * 256u + threadIdx.x;
-    if (xb >= 65536u || (xb & 0x7FFFu) > a) return;
+    // each thread packs eight consecutive bf16 patterns with the production function; patterns beyond
+    // the group's amax (unreachable) are replaced by zero on both sides
+    const uint32_t x0 = (blockIdx.x * 256u + threadIdx.x) * 8u;
+    if (x0 >= 65536u) return;
     const float scale = int4_scale_sym(u2f(a << 16));
-    const float rcp = 1.0f / scale;
-    const float x = u2f(xb << 16);
-    const float qf = __builtin_rintf(x / scale);
-    const int qi = (int)qf;
-    const uint32_t want = (uint32_t)(qi + 8) & 0xFu;
-    const uint32_t got = f2u(div_by_scale(x, scale, rcp) + 12582920.0f) & 0xFu;
-    if (got != want || qi < -7 || qi > 7) report(out, ((uint64_t)a << 16) | xb);
+    const float rcp = rcp_refined(scale);
+    if (f2u(rcp) != f2u(1.0f / scale)) report(out, ((uint64_t)a << 16) | 0xFFFFu);
+    float x[8];
+    uint32_t want = 0;
+    bool range_ok = true;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const uint32_t xb = x0 + j;
+        x[j] = ((xb & 0x7FFFu) > a) ? 0.0f : u2f(xb << 16);
+        const int qi = (int)__builtin_rintf(x[j] / scale);
+        range_ok = range_ok && qi >= -7 && qi <= 7;
+        want |= ((uint32_t)(qi + 8) & 0xFu) << (4 * j);
+    }
+    const uint32_t got = pack8_sym(x, scale, rcp);
+    if (got != want || !range_ok) report(out, ((uint64_t)a << 16) | x0);
 }
 
 // hardware fp32 -> e4m3fn vs software, both word positions of the packed conversion
@@ -175,7 +185,7 @@ WQ_EXPORT int wq_selftest_int4_elem(uint32_t amax_lo, uint32_t amax_hi, uint64_t
     selftest_init_kernel<<<1, 1, 0, st>>>(out);
     WQ_LAUNCH_CHECK();
     if (amax_hi == amax_lo) return WQ_OK;
-    dim3 grid(256, amax_hi - amax_lo, 1);
+    dim3 grid(32, amax_hi - amax_lo, 1);  // 32 x 256 threads x 8 patterns = 65536 per amax
     selftest_int4_elem_kernel<<<grid, 256, 0, st>>>(amax_lo, amax_hi, out);
     WQ_LAUNCH_CHECK();
     return WQ_OK;

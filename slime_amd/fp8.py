@@ -232,6 +232,8 @@ class Fp8DequantPlan:
             assert x.element_size() == 1 and s.dtype == torch.float32
             M, N = x.shape
             assert tuple(s.shape) == (ceildiv(M, self.block), ceildiv(N, self.block))
+            if N >= 2 ** 31 or M * ceildiv(N, _lib.DEQ_SEG) >= 2 ** 31:
+                raise ValueError("Fp8DequantPlan: tensor too large for one descriptor; split it by rows")
             offs.append(total)
             total += _align(M * N * esz) // esz
         self.flat_y = torch.empty(max(total, 1), dtype=out_dtype, device=self.device)
