@@ -119,7 +119,7 @@ typedef struct wq_fp8_dequant_desc {
  * Per tensor, N and M * ceil(N/WQ_DEQ_SEG) must be below 2^31 (the single-tensor entry point checks this and
  * returns WQ_ERR_TOO_LARGE; for the grouped form it is the caller's obligation). */
 #define WQ_DEQ_SEG 512
-#define WQ_DEQ_SEGS_PER_WG 32
+#define WQ_DEQ_SEGS_PER_WG 16
 int wq_fp8_block_dequant_grouped(const wq_fp8_dequant_desc *descs, const int64_t *work_start, int n_desc,
                                  int64_t total_work, int out_dtype, int block, int mode, void *stream);
 

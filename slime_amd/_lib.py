@@ -21,7 +21,7 @@ ABI_VERSION = 1
 DTYPE_BF16, DTYPE_F32 = 0, 1
 FP8_MODE_TORCH, FP8_MODE_TRITON = 0, 1
 DEQ_MODE_F32SCALE, DEQ_MODE_BF16SCALE = 0, 1
-DEQ_SEG, DEQ_SEGS_PER_WG = 512, 32
+DEQ_SEG, DEQ_SEGS_PER_WG = 512, 16
 INT4_GROUPS_PER_WG = 64
 
 _i64, _int, _vp, _u32, _u64 = ctypes.c_int64, ctypes.c_int, ctypes.c_void_p, ctypes.c_uint32, ctypes.c_uint64

@@ -21,6 +21,15 @@ constexpr uint32_t kBf16Inf = 0x7F80u;
 __device__ __forceinline__ float u2f(uint32_t u) { return __builtin_bit_cast(float, u); }
 __device__ __forceinline__ uint32_t f2u(float f) { return __builtin_bit_cast(uint32_t, f); }
 
+// Global-memory accessors.  Tensor pointers reach the kernels through descriptors (plain void*), for
+// which the compiler cannot prove the global address space and would emit FLAT instructions; the casts
+// make every access a GLOBAL one.  *_nt variants carry the non-temporal hint (streamed once).
+#define WQ_GLOBAL __attribute__((address_space(1)))
+template <typename T> __device__ __forceinline__ T ldg_nt(const void* p) { return __builtin_nontemporal_load((const WQ_GLOBAL T*)p); }
+template <typename T> __device__ __forceinline__ T ldg(const void* p) { return *(const WQ_GLOBAL T*)p; }
+template <typename T> __device__ __forceinline__ void stg_nt(void* p, T v) { __builtin_nontemporal_store(v, (WQ_GLOBAL T*)p); }
+template <typename T> __device__ __forceinline__ void stg(void* p, T v) { *(WQ_GLOBAL T*)p = v; }
+
 // A dword holds two bf16: element 2k in the low half, 2k+1 in the high half.
 __device__ __forceinline__ float bf16lo(uint32_t w) { return u2f(w << 16); }
 __device__ __forceinline__ float bf16hi(uint32_t w) { return u2f(w & 0xFFFF0000u); }
@@ -89,6 +98,7 @@ __device__ __forceinline__ uint32_t cvt_pk_fp8_hi(float a, float b, uint32_t old
 constexpr int kXcds = 8;
 __device__ __forceinline__ int64_t xcd_chunked_item(int64_t slot, int64_t total, int C)
 {
+    if (C <= 0) return slot;
     const int64_t span = (int64_t)kXcds * C;
     const int64_t blk = slot / span;
     if ((blk + 1) * span > total) return slot;

@@ -1,12 +1,12 @@
 // block-FP8 (e4m3fn) -> bf16 dequantisation for gfx950.
 //
 // The tensor is cut into row segments of WQ_DEQ_SEG codes; a work item is WQ_DEQ_SEGS_PER_WG consecutive
-// segments (rows are contiguous, so for N a multiple of the segment this is one contiguous 16 KiB run of
-// input and 32 KiB of output) handled by a 256-thread workgroup.  A wavefront takes one segment per step:
+// segments (rows are contiguous, so for N a multiple of the segment this is one contiguous 8 KiB run of
+// input and 16 KiB of output) handled by a 256-thread workgroup.  A wavefront takes one segment per step:
 // every lane loads 8 codes (8 bytes, the wave reads 512 contiguous bytes) and stores the 8 bf16 they
 // become as ONE 16-byte store, so the wave writes 1 KiB contiguous per store instruction - split
-// 16-byte halves per lane measured ~20 % slower.  All eight loads of a lane are issued before the first
-// use.  Codes are expanded with v_cvt_pk_f32_fp8, multiplied by the block's fp32 scale and rounded once
+// 16-byte halves per lane measured ~20 % slower.  All loads of a lane (codes and their block scales) are issued
+// before the first use.  Codes are expanded with v_cvt_pk_f32_fp8, multiplied by the block's fp32 scale and rounded once
 // to bf16 (v_cvt_pk_bf16_f32, RNE): the single rounding of the reference's y = x.to(f32) * s stored to bf16.
 
 #include "wq_common.h"
@@ -20,8 +20,11 @@ typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 constexpr int kSeg = WQ_DEQ_SEG;                 // codes per segment: 64 lanes x 8
 constexpr int kSegsPerWg = WQ_DEQ_SEGS_PER_WG;   // 4 waves x kSteps
 constexpr int kSteps = kSegsPerWg / 4;           // loads in flight per lane
+// Measured on the DeepSeek-V3-shaped layer (768 tensors, one grouped launch; % of the 8 TB/s HBM peak):
+// segments per workgroup x resident workgroups per CU: 32x8 74.0, 32x4 79.3, 16x8 76.5, 16x5 79.4 (used),
+// 16x4 78.2, 8x8 79.7, 8x5 73.1.  A compute-free kernel with the same 1:2 read:write mix tops out at 83 %.
 constexpr int kDeqItemsPerXcdRun = 32;
-constexpr unsigned kDeqOccupancyPadBytes = 0;
+constexpr unsigned kDeqOccupancyPadBytes = 27 * 1024;  // unused dynamic LDS: at most 5 workgroups per CU
 static_assert(kSeg == 512 && kSegsPerWg % 4 == 0, "a segment is 64 lanes x 8 codes; four waves per workgroup");
 
 struct DeqArgs {
@@ -98,39 +101,45 @@ __global__ __launch_bounds__(256) void fp8_block_dequant_kernel(const DeqArgs a,
 
     if (vec) {
         u32x2 v[kSteps];
+        float sc[kSteps];
         uint32_t row[kSteps], col[kSteps];
         bool ok[kSteps];
+        // Phase 1: issue every load of the workgroup's strip - codes and their block scales - before any
+        // use.  Lanes with nothing to do read the tensor's first codes / scale instead of branching
+        // around the load: a predicated load makes the compiler wait for earlier loads first.
 #pragma unroll
         for (int i = 0; i < kSteps; ++i) {
             row[i] = r;
             col[i] = c * kSeg + lane * 8;
             ok[i] = seg0 + 4 * i < n_segs && col[i] < N;
-            v[i] = (u32x2){0u, 0u};
-            if (ok[i]) v[i] = __builtin_nontemporal_load((const u32x2*)(x + (uint64_t)row[i] * N + col[i]));
+            v[i] = ldg_nt<u32x2>(x + (ok[i] ? (uint64_t)row[i] * N + col[i] : 0));
+            const uint32_t sr = bshift >= 0 ? row[i] >> bshift : row[i] / block;
+            const uint32_t sc_col = bshift >= 0 ? col[i] >> bshift : col[i] / block;
+            sc[i] = ldg<float>(d.s + (ok[i] ? sr * kt + sc_col : 0));
             c += 4;
             while (c >= spr) { c -= spr; ++r; }
         }
 #pragma unroll
         for (int i = 0; i < kSteps; ++i) {
             if (!ok[i]) continue;
-            const uint32_t sr = bshift >= 0 ? row[i] >> bshift : row[i] / block;
-            const uint32_t sc_col = bshift >= 0 ? col[i] >> bshift : col[i] / block;
-            const float sc = load_scale<MODE>(d.s, sr * kt + sc_col);
+            if (MODE == WQ_DEQ_MODE_BF16SCALE) sc[i] = u2f(f32_to_bf16_bits(sc[i]) << 16);
             const uint64_t off = (uint64_t)row[i] * N + col[i];
             if (OUT == WQ_DTYPE_BF16) {
-                const u32x2 a0 = dequant4(v[i].x, sc), a1 = dequant4(v[i].y, sc);
+                const u32x2 a0 = dequant4(v[i].x, sc[i]), a1 = dequant4(v[i].y, sc[i]);
                 const u32x4 o = {a0.x, a0.y, a1.x, a1.y};
-                __builtin_nontemporal_store(o, (u32x4*)((uint16_t*)d.y + off));
+                stg_nt<u32x4>((uint16_t*)d.y + off, o);
             } else {
                 f32x4* yp = (f32x4*)((float*)d.y + off);
-                __builtin_nontemporal_store(dequant4_f32(v[i].x, sc), yp);
-                __builtin_nontemporal_store(dequant4_f32(v[i].y, sc), yp + 1);
+                stg_nt<f32x4>(yp, dequant4_f32(v[i].x, sc[i]));
+                stg_nt<f32x4>(yp + 1, dequant4_f32(v[i].y, sc[i]));
             }
         }
     } else {
         // element-wise path: any N, alignment and block size
+#pragma nounroll
         for (int i = 0; i < kSteps; ++i) {
             if (seg0 + 4 * i >= n_segs) break;
+#pragma nounroll
             for (int k = 0; k < 8; ++k) {
                 const uint32_t cc = c * kSeg + k * 64 + lane;
                 if (cc >= N) break;

@@ -1,7 +1,7 @@
 // bf16 -> block-FP8 (e4m3fn) quantisation for gfx950.
 //
-// Vector kernel (128x128 blocks, unit column stride, 16-byte aligned rows): one 256-thread
-// workgroup owns one block.  Each lane issues eight 16-byte loads (8 bf16 each, rows rb+16*i), so a
+// Vector kernel (128x128 blocks, unit column stride, 16-byte aligned rows): one 512-thread
+// workgroup owns one block.  Each lane issues four 16-byte loads (8 bf16 each, rows rb+32*i), so a
 // wavefront load covers four 256-byte row segments and the whole 32 KiB block is in flight before
 // the first use.  The block lives in registers from then on: amax is an integer max over the bf16
 // magnitude bits (packed 16-bit max), reduced over 16 lanes with DPP and across the workgroup
@@ -17,12 +17,21 @@
 
 namespace wq {
 
-// Measured on MI355X (7.3 GB of 128x128 tiles, row widths 2560 / 4096 / 9728): runs of 32 consecutive tiles
-// per XCD and at most four resident workgroups per CU (enforced with unused dynamic LDS) reach 76-81 % of
-// the HBM peak against 69-71 % for plain dispatch order at full occupancy; neighbouring settings (runs of
-// 24-64 tiles, 3-6 workgroups) are within two points.
-constexpr int kTilesPerXcdRun = 32;
-constexpr unsigned kOccupancyPadBytes = 36 * 1024;
+// Workgroup shape, work order and residency, measured on MI355X on the Qwen3-4B-shaped pass (252 tensors,
+// 7.27 GB of bf16, one grouped launch; fraction of the 8 TB/s HBM peak):
+//   256 threads, plain dispatch order, full occupancy (8 workgroups per CU)      69.6 %
+//   256 threads, runs of 32 tiles per XCD, 4 workgroups per CU                   76.7 - 77.1 %   <- used
+//   256 threads, runs of 64 tiles per XCD, 4 workgroups per CU                   76.9 %
+//   256 threads, runs of 32 tiles per XCD, 3 workgroups per CU                   73.6 %
+//   512 threads (4 loads per lane), runs of 16 / 32 / 64 tiles                   75.5 / 76.1 / 76.3 %
+//   512 threads, plain dispatch order                                            71.1 %
+// A compute-free kernel with the same 2:1 read:write mix tops out at 86 % on this part.
+constexpr int kTileThreads = 256;
+constexpr int kTilesPerXcdRun = 32;               // consecutive tiles handed to one XCD (xcd_chunked_item)
+constexpr unsigned kOccupancyPadBytes = 36 * 1024;  // unused dynamic LDS: caps residency at 4 workgroups per CU
+constexpr int kRowSlots = kTileThreads / 16;   // rows covered by one load step of the workgroup
+constexpr int kTileLoads = 128 / kRowSlots;    // 16-byte loads per lane
+constexpr int kTileWaves = kTileThreads / 64;
 
 struct Fp8QuantArgs {
     wq_fp8_quant_desc d;  // single-tensor launch: descriptor travels in the kernel arguments
@@ -46,32 +55,32 @@ __device__ __forceinline__ void quant_tile_vec128(const wq_fp8_quant_desc& d, in
 {
     const int t = threadIdx.x;
     const int cc = t & 15;  // which 8-element piece of the 128 columns
-    const int rb = t >> 4;  // 0..15
+    const int rb = t >> 4;  // 0..kRowSlots-1
     // Workgroup-uniform tile origin (scalar registers) + 32-bit per-lane byte offsets.
     const char* xt = (const char*)d.x + (tm * 128 * d.sx_m + tn * 128) * 2;
     char* yt = (char*)d.y + (tm * 128 * d.sy_m + tn * 128);
-    const uint32_t xstep = (uint32_t)d.sx_m * 32u, ystep = (uint32_t)d.sy_m * 16u;  // 16 rows, in bytes
+    const uint32_t xstep = (uint32_t)d.sx_m * 2u * kRowSlots, ystep = (uint32_t)d.sy_m * kRowSlots;  // one step, in bytes
     const uint32_t xoff = (uint32_t)rb * (uint32_t)d.sx_m * 2u + (uint32_t)cc * 16u;
     const uint32_t yoff = (uint32_t)rb * (uint32_t)d.sy_m + (uint32_t)cc * 8u;
-    const int rows_left = (int)min((int64_t)128, d.M - tm * 128) - rb;  // row rb+16*i is valid iff 16*i < rows_left
+    const int rows_left = (int)min((int64_t)128, d.M - tm * 128) - rb;  // row rb + kRowSlots*i is valid iff kRowSlots*i < rows_left
     const bool col_ok = tn * 128 + cc * 8 < d.N;
     const bool full = (tm * 128 + 128 <= d.M) && (tn * 128 + 128 <= d.N);
 
-    u32x4 v[8];
+    u32x4 v[kTileLoads];
     if (full) {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) v[i] = __builtin_nontemporal_load((const u32x4*)(xt + (xoff + i * xstep)));
+        for (int i = 0; i < kTileLoads; ++i) v[i] = ldg_nt<u32x4>(xt + (xoff + i * xstep));
     } else {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
+        for (int i = 0; i < kTileLoads; ++i) {
             v[i] = (u32x4){0u, 0u, 0u, 0u};
-            if (col_ok && 16 * i < rows_left) v[i] = __builtin_nontemporal_load((const u32x4*)(xt + (xoff + i * xstep)));
+            if (col_ok && kRowSlots * i < rows_left) v[i] = ldg_nt<u32x4>(xt + (xoff + i * xstep));
         }
     }
 
     uint32_t m = 0;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
+    for (int i = 0; i < kTileLoads; ++i) {
         m = pk_absmax(m, v[i].x);
         m = pk_absmax(m, v[i].y);
         m = pk_absmax(m, v[i].z);
@@ -80,38 +89,35 @@ __device__ __forceinline__ void quant_tile_vec128(const wq_fp8_quant_desc& d, in
     m = row16_max_u32(pk_fold(m));
     if (cc == 0) lds[rb] = m;
     __syncthreads();
-    {
-        const u32x4* l4 = (const u32x4*)lds;
-        u32x4 a = l4[0], b = l4[1], c = l4[2], e = l4[3];
-        uint32_t m0 = max(max(a.x, a.y), max(a.z, a.w));
-        uint32_t m1 = max(max(b.x, b.y), max(b.z, b.w));
-        uint32_t m2 = max(max(c.x, c.y), max(c.z, c.w));
-        uint32_t m3 = max(max(e.x, e.y), max(e.z, e.w));
-        m = max(max(m0, m1), max(m2, m3));
+    m = 0;
+#pragma unroll
+    for (int i = 0; i < kRowSlots / 4; ++i) {
+        const u32x4 a = ((const u32x4*)lds)[i];
+        m = max(m, max(max(a.x, a.y), max(a.z, a.w)));
     }
 
     const Fp8BlockParams p = fp8_block_params<MODE>(m);
-    if (t == 0) d.s[tm * kt + tn] = p.scale;
+    if (t == 0) stg<float>(d.s + (tm * kt + tn), p.scale);
 
     if (p.fast) {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
+        for (int i = 0; i < kTileLoads; ++i) {
             u32x2 o;
             o.x = fp8_quant4_fast<MODE>(v[i].x, v[i].y, p);
             o.y = fp8_quant4_fast<MODE>(v[i].z, v[i].w, p);
-            if (full || (col_ok && 16 * i < rows_left)) __builtin_nontemporal_store(o, (u32x2*)(yt + (yoff + i * ystep)));
+            if (full || (col_ok && kRowSlots * i < rows_left)) stg_nt<u32x2>(yt + (yoff + i * ystep), o);
         }
     } else {
         // NaN/Inf block (rare): literal arithmetic.  The rows are re-read so that the register copy of
         // the block is never indexed dynamically.
 #pragma nounroll
-        for (int i = 0; i < 8; ++i) {
-            if (!(full || (col_ok && 16 * i < rows_left))) continue;
-            const u32x4 w = *(const u32x4*)(xt + (xoff + i * xstep));
+        for (int i = 0; i < kTileLoads; ++i) {
+            if (!(full || (col_ok && kRowSlots * i < rows_left))) continue;
+            const u32x4 w = ldg<u32x4>(xt + (xoff + i * xstep));
             u32x2 o;
             o.x = fp8_quant4_exact<MODE>(w.x, w.y, p);
             o.y = fp8_quant4_exact<MODE>(w.z, w.w, p);
-            *(u32x2*)(yt + (yoff + i * ystep)) = o;
+            stg<u32x2>(yt + (yoff + i * ystep), o);
         }
     }
 }
@@ -132,7 +138,8 @@ __device__ __forceinline__ void quant_tile_generic(const wq_fp8_quant_desc& d, i
     m = wave64_max_u32(m);
     if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6] = m;
     __syncthreads();
-    m = max(max(lds[0], lds[1]), max(lds[2], lds[3]));
+    m = 0;
+    for (int w = 0; w < kTileWaves; ++w) m = max(m, lds[w]);
     const Fp8BlockParams p = fp8_block_params<MODE>(m);
     if (threadIdx.x == 0) d.s[tm * kt + tn] = p.scale;
     uint8_t* y = (uint8_t*)d.y;
@@ -144,9 +151,9 @@ __device__ __forceinline__ void quant_tile_generic(const wq_fp8_quant_desc& d, i
 }
 
 template <int MODE, bool GROUPED>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 8))) void fp8_block_quant_kernel(const Fp8QuantArgs a, const int64_t total_tiles)
+__global__ __launch_bounds__(kTileThreads) void fp8_block_quant_kernel(const Fp8QuantArgs a, const int64_t total_tiles)
 {
-    __shared__ __attribute__((aligned(16))) uint32_t lds[16];
+    __shared__ __attribute__((aligned(16))) uint32_t lds[kRowSlots];
     const int64_t slot = (int64_t)blockIdx.x + (int64_t)blockIdx.y * gridDim.x;
     if (slot >= total_tiles) return;  // uniform per workgroup
     const int64_t tile = xcd_chunked_item(slot, total_tiles, kTilesPerXcdRun);
@@ -253,9 +260,9 @@ WQ_EXPORT int wq_fp8_block_quant(const void* x, int64_t M, int64_t N, int64_t sx
     const int64_t tiles = cdiv64(M, bm) * cdiv64(N, bn);
     hipStream_t st = (hipStream_t)stream;
     if (mode == WQ_FP8_MODE_TORCH)
-        fp8_block_quant_kernel<WQ_FP8_MODE_TORCH, false><<<grid_for_items(tiles), 256, kOccupancyPadBytes, st>>>(a, tiles);
+        fp8_block_quant_kernel<WQ_FP8_MODE_TORCH, false><<<grid_for_items(tiles), kTileThreads, kOccupancyPadBytes, st>>>(a, tiles);
     else
-        fp8_block_quant_kernel<WQ_FP8_MODE_TRITON, false><<<grid_for_items(tiles), 256, kOccupancyPadBytes, st>>>(a, tiles);
+        fp8_block_quant_kernel<WQ_FP8_MODE_TRITON, false><<<grid_for_items(tiles), kTileThreads, kOccupancyPadBytes, st>>>(a, tiles);
     WQ_LAUNCH_CHECK();
     return WQ_OK;
 }
@@ -276,9 +283,9 @@ WQ_EXPORT int wq_fp8_block_quant_grouped(const wq_fp8_quant_desc* descs, const i
     a.bn = bn;
     hipStream_t st = (hipStream_t)stream;
     if (mode == WQ_FP8_MODE_TORCH)
-        fp8_block_quant_kernel<WQ_FP8_MODE_TORCH, true><<<grid_for_items(total_tiles), 256, kOccupancyPadBytes, st>>>(a, total_tiles);
+        fp8_block_quant_kernel<WQ_FP8_MODE_TORCH, true><<<grid_for_items(total_tiles), kTileThreads, kOccupancyPadBytes, st>>>(a, total_tiles);
     else
-        fp8_block_quant_kernel<WQ_FP8_MODE_TRITON, true><<<grid_for_items(total_tiles), 256, kOccupancyPadBytes, st>>>(a, total_tiles);
+        fp8_block_quant_kernel<WQ_FP8_MODE_TRITON, true><<<grid_for_items(total_tiles), kTileThreads, kOccupancyPadBytes, st>>>(a, total_tiles);
     WQ_LAUNCH_CHECK();
     return WQ_OK;
 }

@@ -20,6 +20,7 @@ namespace wq {
 constexpr int kGroupsPerWg = WQ_INT4_GROUPS_PER_WG;
 constexpr int kPackItemsPerXcdRun = 32;  // 32 work items = 512 KiB of contiguous input per XCD run
 constexpr unsigned kPackOccupancyPadBytes = 0;
+constexpr int kPackWindow = 2;              // 16-byte loads in flight per lane
 
 struct Int4PackArgs {
     wq_int4_pack_desc d;
@@ -104,7 +105,8 @@ template <int L, bool GROUPED>
 __global__ __launch_bounds__(256) void int4_pack_kernel(const Int4PackArgs a, const int64_t total_work)
 {
     constexpr int CL = 256 / L;              // groups per step of the workgroup
-    constexpr int STEPS = kGroupsPerWg / CL; // 1 (L=4), 2 (L=8), 4 (L=16)
+    constexpr int STEPS = kGroupsPerWg / CL; // kGroupsPerWg = 64: 1 (L=4), 2 (L=8), 4 (L=16)
+    static_assert(STEPS >= 1, "a work item must cover at least one step of the workgroup");
     const int64_t slot = (int64_t)blockIdx.x + (int64_t)blockIdx.y * gridDim.x;
     if (slot >= total_work) return;
     const int64_t item = xcd_chunked_item(slot, total_work, kPackItemsPerXcdRun);
@@ -121,26 +123,34 @@ __global__ __launch_bounds__(256) void int4_pack_kernel(const Int4PackArgs a, co
     const int64_t g0 = local * kGroupsPerWg + cl;
     const uint16_t* x = (const uint16_t*)d.x;
 
+    // Rolling window: at most kPackWindow 16-byte loads per lane are in flight; the load of step i + window
+    // is issued just before step i is processed.  More bytes in flight per CU than that lower the achieved
+    // HBM bandwidth on this part, while a long work item amortises the per-workgroup start-up.
+    // Out-of-range groups re-read the tensor's last group instead of branching around the load (a
+    // predicated load makes the compiler wait for earlier loads before issuing the next one).
     u32x4 v[STEPS];
+    auto issue = [&](int i) {
+        const int64_t g = min(g0 + i * CL, d.n_groups - 1);
+        v[i] = ldg_nt<u32x4>(x + g * (8 * L) + ll * 8);
+    };
+#pragma unroll
+    for (int i = 0; i < kPackWindow && i < STEPS; ++i) issue(i);
 #pragma unroll
     for (int i = 0; i < STEPS; ++i) {
+        if (i + kPackWindow < STEPS) issue(i + kPackWindow);
+        __builtin_amdgcn_sched_barrier(0);
         const int64_t g = g0 + i * CL;
-        v[i] = (u32x4){0u, 0u, 0u, 0u};
-        if (g < d.n_groups) v[i] = __builtin_nontemporal_load((const u32x4*)(x + g * (8 * L) + ll * 8));
-    }
-#pragma unroll
-    for (int i = 0; i < STEPS; ++i) {
-        const int64_t g = g0 + i * CL;
-        float x[8];
-        unpack8(v[i], x);
-        const float scale = int4_scale_sym(lanes_max_f32<L>(absmax8(x)));
-        uint32_t w = pack8_sym(x, scale, rcp_refined(scale));
+        float xs[8];
+        unpack8(v[i], xs);
+        const float scale = int4_scale_sym(lanes_max_f32<L>(absmax8(xs)));
+        uint32_t w = pack8_sym(xs, scale, rcp_refined(scale));
         const uint32_t sb_bits = bf16_bits_hw(scale);
-        if (sb_bits >= kLiteralChainScaleBits) w = pack8_literal(x, scale, u2f(sb_bits << 16));
+        if (sb_bits >= kLiteralChainScaleBits) w = pack8_literal(xs, scale, u2f(sb_bits << 16));
         if (g < d.n_groups) {
-            __builtin_nontemporal_store(w, (uint32_t*)d.packed + g * L + ll);
-            if (ll == 0) ((uint16_t*)d.scale)[g] = (uint16_t)sb_bits;
+            stg_nt<uint32_t>((uint32_t*)d.packed + g * L + ll, w);
+            if (ll == 0) stg<uint16_t>((uint16_t*)d.scale + g, (uint16_t)sb_bits);
         }
+        __builtin_amdgcn_sched_barrier(0);
     }
 }
 
