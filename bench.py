@@ -198,6 +198,42 @@ def bench_copy(dev, steps, warmup, nbytes=4 << 30):
             "hbm_frac": 2 * nbytes / ev_ms / 1e6 / HBM_PEAK_GBS}
 
 
+def bench_stream(dev, n_buckets=64, bucket_bytes=1 << 30, download=True):
+    """Host-resident weights: n_buckets x bucket_bytes of bf16 through pinned double buffers -> block-FP8 quant ->
+    (optionally) back to pinned host memory.  PCIe-bound by construction; reported next to the kernel-only rate."""
+    import torch
+
+    from oracle import c_oracle
+    from slime_amd.stream import BucketPipeline, fp8_block_quant_kernel
+
+    N = 4096
+    M = bucket_bytes // 2 // N
+    pipe = BucketPipeline(dev, fp8_block_quant_kernel(), bucket_bytes, bucket_bytes // 2, 2, depth=2, download=download)
+    pipe.time_kernels = True
+    for slot in range(2):
+        pipe.staging_buffer(slot).copy_(_gen_bf16((M, N), dev).view(-1).view(torch.uint8))
+    torch.cuda.synchronize()
+
+    def buckets():
+        for i in range(n_buckets):
+            yield pipe.staging_buffer(i % 2).view(torch.bfloat16).view(M, N)
+
+    checked = 0
+    t0 = time.perf_counter()
+    for i, (q, s) in enumerate(pipe.process(buckets())):
+        if i == 0 and download:
+            qo, so = c_oracle.fp8_block_quant(pipe.staging_buffer(0).view(torch.bfloat16).view(M, N)[:1024], (128, 128), 0)
+            assert torch.equal(q[:1024].view(torch.uint8), qo) and torch.equal(s[:8].view(torch.int32), so.view(torch.int32))
+            checked = 1
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    total = n_buckets * bucket_bytes
+    return {"workload": f"{n_buckets} x {bucket_bytes >> 20} MiB bf16 buckets from pinned host memory -> block-FP8 -> "
+                        f"{'pinned host memory' if download else 'device'}, double-buffered",
+            "bf16_GB": total / 1e9, "wall_s": wall, "end_to_end_GBps": total / wall / 1e9,
+            "kernel_only_GBps": total / (pipe.kernel_ms() / 1e3) / 1e9, "parity_buckets_checked": checked}
+
+
 def cpu_baseline(sample, budget_s: float):
     """The CPU restatement of the reference torch path (block_fp8 op sequence) on one layer's tensors."""
     import torch
@@ -234,9 +270,13 @@ def main():
     ap.add_argument("--dequant-experts", type=int, default=256)
     ap.add_argument("--no-extras", action="store_true", help="headline workload only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
-    ap.add_argument("--only", choices=["int4", "dequant", "copy"], default=None,
-                    help="profiling aid: run just one of the other kernels (or the plain copy kernel that hardware "
-                         "counters are calibrated against) and print its record")
+    ap.add_argument("--only", choices=["int4", "dequant", "copy", "stream"], default=None,
+                    help="run just one of the other legs and print its record: a kernel for profiling, the plain copy "
+                         "kernel that hardware counters are calibrated against, or the host-resident streaming run "
+                         "(64 x 1 GiB buckets, PCIe-bound)")
+    ap.add_argument("--stream-buckets", type=int, default=64)
+    ap.add_argument("--stream-bucket-mib", type=int, default=1024)
+    ap.add_argument("--stream-no-download", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures ONE GPU: the path has no cross-GPU exchange and this build has no multi-GPU "
@@ -259,6 +299,10 @@ def main():
         return
     if args.only == "copy":
         print(json.dumps(bench_copy(dev, args.steps, args.warmup)))
+        return
+    if args.only == "stream":
+        print(json.dumps(bench_stream(dev, args.stream_buckets, args.stream_bucket_mib << 20,
+                                      not args.stream_no_download)))
         return
 
     r = bench_fp8_quant(dev, args.steps, args.warmup)
