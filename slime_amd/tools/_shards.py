@@ -1,0 +1,90 @@
+"""Shard plumbing shared by the offline converters: reading safetensors shards, moving a shard's tensors to the
+GPU and back, the index / config writers and the result collector."""
+
+from __future__ import annotations
+
+import json
+import os
+import shutil
+import threading
+
+import torch
+from safetensors import safe_open
+from safetensors.torch import save_file
+
+
+def device() -> torch.device:
+    if not torch.cuda.is_available():
+        raise RuntimeError("the converters run their arithmetic on the GPU; no GPU is visible and there is no CPU path")
+    return torch.device("cuda", torch.cuda.current_device())
+
+
+def read_shard(path: str) -> dict:
+    """All tensors of one .safetensors file as CPU tensors (memory-mapped by safetensors)."""
+    out = {}
+    with safe_open(path, framework="pt", device="cpu") as f:
+        for k in f.keys():
+            out[k] = f.get_tensor(k)
+    return out
+
+
+def write_shard(tensors: dict, path: str, with_format_tag: bool = True) -> None:
+    """The FP8 and INT4 converters tag their shards with metadata {"format": "pt"}
+    (tools/convert_hf_to_fp8.py:161); the dequantising tool writes none (tools/fp8_cast_bf16.py:94)."""
+    tensors = {k: v.contiguous() for k, v in tensors.items()}
+    if with_format_tag:
+        save_file(tensors, path, metadata={"format": "pt"})
+    else:
+        save_file(tensors, path)
+
+
+def copy_side_files(input_path: str, output_path: str) -> None:
+    """Everything in the checkpoint directory that is neither a shard nor a directory is copied verbatim
+    (tools/convert_hf_to_fp8.py:170-172)."""
+    for name in os.listdir(input_path):
+        src = os.path.join(input_path, name)
+        if not name.endswith(".safetensors") and not os.path.isdir(src):
+            shutil.copyfile(src, os.path.join(output_path, name))
+
+
+def list_shards(input_path: str) -> list:
+    return sorted(f for f in os.listdir(input_path) if f.endswith(".safetensors"))
+
+
+class ConversionResult:
+    """Thread-safe accumulator of the output index.  ``param_count`` reproduces the reference's quirk: it adds
+    ``len(tensor)`` - the first dimension - of every output tensor (tools/convert_hf_to_fp8.py:110-114), and
+    that number is what lands in ``metadata.total_size``."""
+
+    def __init__(self):
+        self.lock = threading.Lock()
+        self.weight_map = {}
+        self.param_count = 0
+        self.modules_to_not_convert = []
+
+    def add_result(self, filename: str, tensors: dict, module_names=()):
+        with self.lock:
+            for k, v in tensors.items():
+                self.weight_map[k] = filename
+                self.param_count += len(v)
+            self.modules_to_not_convert.extend(module_names)
+
+
+def write_index(output_path: str, result: ConversionResult) -> None:
+    index = {"weight_map": result.weight_map, "metadata": {"total_size": result.param_count}}
+    with open(os.path.join(output_path, "model.safetensors.index.json"), "w") as f:
+        json.dump(index, f, indent=2)
+
+
+def write_config(input_path: str, output_path: str, quantization_config: dict) -> None:
+    src = os.path.join(input_path, "config.json")
+    if os.path.exists(src):
+        with open(src) as f:
+            cfg = json.load(f)
+        cfg["quantization_config"] = quantization_config
+        with open(os.path.join(output_path, "config.json"), "w") as f:
+            json.dump(cfg, f, indent=2)
+
+
+def to_device(t: torch.Tensor, dev: torch.device) -> torch.Tensor:
+    return t.to(dev, non_blocking=True)
