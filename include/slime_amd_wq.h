@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define WQ_ABI_VERSION 1
+#define WQ_ABI_VERSION 2
 
 enum {
     WQ_OK = 0,
@@ -47,11 +47,17 @@ enum { WQ_DTYPE_BF16 = 0, WQ_DTYPE_F32 = 1 };
 /* FP8 block quant arithmetic.
  * WQ_FP8_MODE_TORCH  : amax clamped at bf16(1e-12) in bf16, scale = f32(amax)/448, q = f32(x)/scale
  *                      (IEEE division), clamp +-448, RNE to e4m3fn.
- *                      Replaces block_fp8, tools/convert_hf_to_fp8.py:41-75.
+ *                      Replaces block_fp8, tools/convert_hf_to_fp8.py:41-75, as torch evaluates it on CPU
+ *                      tensors (how the reference's own test runs it, tests/test_block_fp8_zero_block.py).
+ * WQ_FP8_MODE_TORCH_DEVICE : the same function as torch evaluates it on GPU tensors (how the tool runs
+ *                      it, tools/convert_hf_to_fp8.py:127): torch's GPU kernels compute
+ *                      `tensor / python_scalar` as tensor * (1.0f/scalar), so
+ *                      scale = f32(amax) * RN(1/448), up to one ulp from the quotient; everything else
+ *                      (the IEEE x/scale, clamp, cast) is as in WQ_FP8_MODE_TORCH.
  * WQ_FP8_MODE_TRITON : fp32 amax floored at 1e-10f, scale = amax/448, q = f32(x)*(1.0f/scale).
  *                      Replaces _blockwise_cast_to_fp8_triton,
  *                      slime/backends/megatron_utils/kernels/fp8_kernel.py:24-58. */
-enum { WQ_FP8_MODE_TORCH = 0, WQ_FP8_MODE_TRITON = 1 };
+enum { WQ_FP8_MODE_TORCH = 0, WQ_FP8_MODE_TRITON = 1, WQ_FP8_MODE_TORCH_DEVICE = 2 };
 
 /* FP8 block dequant arithmetic.
  * WQ_DEQ_MODE_F32SCALE  : y = bf16(f32(x) * s).  Replaces weight_dequant, tools/fp8_cast_bf16.py:16-41.
@@ -92,11 +98,11 @@ int wq_fp8_block_quant_grouped(const wq_fp8_quant_desc *descs, const int64_t *ti
 /* Per-row and per-tensor scaling: channel_fp8 / tensor_fp8, tools/convert_hf_to_fp8.py:78-91, and the
  * per-tensor branch of _quantize_param, quantizer_fp8.py:112-117.  s has M entries (row) or 1 (tensor).
  * wq_fp8_tensor_quant needs `workspace`: one zero-initialised uint32 in device memory that the call
- * may overwrite (the cross-workgroup amax). */
+ * may overwrite (the cross-workgroup amax).  `mode` is WQ_FP8_MODE_TORCH or WQ_FP8_MODE_TORCH_DEVICE. */
 int wq_fp8_row_quant(const void *x, int64_t M, int64_t N, int64_t sx_m, int64_t sx_n,
-                     void *y, int64_t sy_m, float *s, void *stream);
+                     void *y, int64_t sy_m, float *s, int mode, void *stream);
 int wq_fp8_tensor_quant(const void *x, int64_t M, int64_t N, int64_t sx_m, int64_t sx_n,
-                        void *y, int64_t sy_m, float *s, uint32_t *workspace, void *stream);
+                        void *y, int64_t sy_m, float *s, uint32_t *workspace, int mode, void *stream);
 
 /* ---------------------------------------------------------------------------------------------
  * e4m3fn [M,N] contiguous + fp32 scale [ceil(M/block), ceil(N/block)] contiguous -> y [M,N]
@@ -153,6 +159,21 @@ typedef struct wq_int4_pack_desc {
 #define WQ_INT4_GROUPS_PER_WG 64
 int wq_int4_group_quant_pack_grouped(const wq_int4_pack_desc *descs, const int64_t *work_start, int n_desc,
                                      int64_t total_work, int group, void *stream);
+
+/* INT4 pack-quantized -> bf16: y[i,j] = bf16((nibble(i,j) - 8) * f32(scale[i, j/group])), nibble j of word c at
+ * bits [4j,4j+4).  packed int32 [M,N/8], scale bf16 [M,N/group], y bf16 [M,N], all contiguous; N % group == 0,
+ * group % 8 == 0.  Replaces _dequantize_tensor, tools/convert_k2_thinking_int4_to_bf16.py:55-84 (whose unpacking
+ * is compressed_tensors.unpack_from_int32). */
+int wq_int4_dequant(const int32_t *packed, const void *scale, void *y, int64_t M, int64_t N, int group, void *stream);
+
+/* Forward of the INT4 QAT straight-through estimator: per (1 x group) group of a contiguous bf16 [M,N],
+ * s = max(f32(amax) / 7, 1e-5), y = bf16(clamp(round_half_even(f32(x) / s), -7, 7) * s); N % group == 0 and
+ * group in {32, 64, 128}.  Replaces _FakeInt4QuantizationSTE.forward, docker/patch/latest/megatron.patch:212-246
+ * (it dequantises with the unrounded fp32 scale, unlike pack_layer).  `div7` selects how `amax / 7` is evaluated:
+ * WQ_DIV7_IEEE as torch does on CPU tensors (a division), WQ_DIV7_DEVICE as torch does on GPU tensors
+ * (amax * RN(1/7), which is also what fake_int4_quant_cuda.cu:59 computes); x / s is an IEEE division in both. */
+enum { WQ_DIV7_IEEE = 0, WQ_DIV7_DEVICE = 1 };
+int wq_int4_fake_quant_ste(const void *x, void *y, int64_t M, int64_t N, int group, int div7, void *stream);
 
 /* ---------------------------------------------------------------------------------------------
  * Self-checks and calibration helpers (used by the test-suite and the benchmark, not by callers).

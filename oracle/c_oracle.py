@@ -32,11 +32,13 @@ def lib() -> ctypes.CDLL:
             build()
         L = ctypes.CDLL(_SO)
         L.wqo_fp8_block_quant.argtypes = [_vp, _i64, _i64, _i64, _i64, _i64, _i64, _int, _vp, _vp]
-        L.wqo_fp8_channel_quant.argtypes = [_vp, _i64, _i64, _i64, _i64, _vp, _vp]
-        L.wqo_fp8_tensor_quant.argtypes = [_vp, _i64, _i64, _i64, _i64, _vp, _vp]
+        L.wqo_fp8_channel_quant.argtypes = [_vp, _i64, _i64, _i64, _i64, _int, _vp, _vp]
+        L.wqo_fp8_tensor_quant.argtypes = [_vp, _i64, _i64, _i64, _i64, _int, _vp, _vp]
         L.wqo_fp8_block_dequant.argtypes = [_vp, _vp, _i64, _i64, _i64, _int, _vp]
         L.wqo_int4_fake_quant.argtypes = [_vp, _int, _i64, _i64, _i64, _i64, _i64, _i64, _int, _vp, _vp, _vp]
         L.wqo_int4_pack_layer.argtypes = [_vp, _i64, _i64, _i64, _int, _vp, _vp, _vp]
+        L.wqo_int4_dequant.argtypes = [_vp, _vp, _i64, _i64, _i64, _vp]
+        L.wqo_int4_fake_ste.argtypes = [_vp, _i64, _i64, _i64, _int, _vp]
         for n in ("wqo_f32_to_e4m3fn_n", "wqo_e4m3fn_to_f32_n", "wqo_f32_to_bf16_n"):
             getattr(L, n).argtypes = [_vp, _vp, _i64]
             getattr(L, n).restype = None
@@ -93,22 +95,24 @@ def fp8_block_quant(w: torch.Tensor, block_size=(128, 128), mode: int = 0):
     return y, s
 
 
-def fp8_channel_quant(w: torch.Tensor):
+def fp8_channel_quant(w: torch.Tensor, mode: int = 0):
     assert _cpu(w).dtype == torch.bfloat16 and w.dim() == 2
     M, N = w.shape
     y = torch.empty(M, N, dtype=torch.uint8)
     s = torch.empty(M, 1, dtype=torch.float32)
-    _check(lib().wqo_fp8_channel_quant(w.data_ptr(), M, N, w.stride(0), w.stride(1), y.data_ptr(), s.data_ptr()),
+    _check(lib().wqo_fp8_channel_quant(w.data_ptr(), M, N, w.stride(0), w.stride(1), mode, y.data_ptr(),
+                                       s.data_ptr()),
            "fp8_channel_quant")
     return y, s
 
 
-def fp8_tensor_quant(w: torch.Tensor):
+def fp8_tensor_quant(w: torch.Tensor, mode: int = 0):
     assert _cpu(w).dtype == torch.bfloat16 and w.dim() == 2
     M, N = w.shape
     y = torch.empty(M, N, dtype=torch.uint8)
     s = torch.empty(1, dtype=torch.float32)
-    _check(lib().wqo_fp8_tensor_quant(w.data_ptr(), M, N, w.stride(0), w.stride(1), y.data_ptr(), s.data_ptr()),
+    _check(lib().wqo_fp8_tensor_quant(w.data_ptr(), M, N, w.stride(0), w.stride(1), mode, y.data_ptr(),
+                                      s.data_ptr()),
            "fp8_tensor_quant")
     return y, s
 
@@ -147,6 +151,25 @@ def int4_pack_layer(w: torch.Tensor, group_size: int, sym: bool = True):
     _check(lib().wqo_int4_pack_layer(w.data_ptr(), M, N, group_size, int(sym), packed.data_ptr(), sc.data_ptr(),
                                      None if sym else pzp.data_ptr()), "int4_pack_layer")
     return packed, sc, pzp
+
+
+def int4_dequant(packed: torch.Tensor, scale: torch.Tensor, shape, group_size: int) -> torch.Tensor:
+    M, N = shape
+    packed = _cpu(packed).contiguous()
+    scale = _cpu(scale).contiguous()
+    assert packed.dtype == torch.int32 and scale.dtype == torch.bfloat16
+    y = torch.empty(M, N, dtype=torch.bfloat16)
+    _check(lib().wqo_int4_dequant(packed.data_ptr(), scale.data_ptr(), M, N, group_size, y.data_ptr()), "int4_dequant")
+    return y
+
+
+def int4_fake_ste(x: torch.Tensor, group_size: int, div7: int = 0) -> torch.Tensor:
+    x = _cpu(x).contiguous()
+    assert x.dtype == torch.bfloat16 and x.dim() == 2
+    M, N = x.shape
+    y = torch.empty(M, N, dtype=torch.bfloat16)
+    _check(lib().wqo_int4_fake_ste(x.data_ptr(), M, N, group_size, div7, y.data_ptr()), "int4_fake_ste")
+    return y
 
 
 def num_threads() -> int:

@@ -28,7 +28,16 @@ def _cdiv(a: int, b: int) -> int:
 # ----------------------------------------------------------------------------- FP8 quant
 
 
-def block_fp8_ref(w: torch.Tensor, block_size) -> tuple[torch.Tensor, torch.Tensor]:
+def _div_scalar(t: torch.Tensor, d: float, device_arith: bool) -> torch.Tensor:
+    """``t / d`` for a Python scalar d.  torch evaluates that as a division on CPU tensors and as
+    ``t * RN(1/d)`` on GPU tensors; ``device_arith`` reproduces the second form on the CPU."""
+    if not device_arith:
+        return t / d
+    inv = (torch.ones((), dtype=torch.float32) / d).item()
+    return t * inv
+
+
+def block_fp8_ref(w: torch.Tensor, block_size, device_arith: bool = False) -> tuple[torch.Tensor, torch.Tensor]:
     """tools/convert_hf_to_fp8.py:41-75.  pad(0.0) -> view as tiles -> |.|, max over tile rows,
     max over tile cols (weight dtype) -> clamp(min=1e-12) (weight dtype) -> fp32 / 448 ->
     weight / scale (fp32 division) -> clamp(+-448) -> e4m3fn -> crop + contiguous copy."""
@@ -38,21 +47,24 @@ def block_fp8_ref(w: torch.Tensor, block_size) -> tuple[torch.Tensor, torch.Tens
     padded = F.pad(w, (0, tn * bn - cols, 0, tm * bm - rows), mode="constant", value=0.0)
     tiles = padded.reshape(tm, bm, tn, bn)
     amax = tiles.abs().max(dim=1, keepdim=True)[0].max(dim=3, keepdim=True)[0]
-    scale = amax.clamp(min=1e-12).to(torch.float32) / E4M3_MAX
+    scale = _div_scalar(amax.clamp(min=1e-12).to(torch.float32), E4M3_MAX, device_arith)
     q = (tiles / scale).clamp(min=E4M3_MIN, max=E4M3_MAX).reshape(tm * bm, tn * bn).to(E4M3)
     return q[:rows, :cols].clone(), scale.reshape(tm, tn)
 
 
-def channel_fp8_ref(w: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+def channel_fp8_ref(w: torch.Tensor, device_arith: bool = False) -> tuple[torch.Tensor, torch.Tensor]:
     """tools/convert_hf_to_fp8.py:78-83 (scale shape [M, 1])."""
     amax = w.abs().max(dim=-1, keepdim=True)[0]
-    scale = amax.clamp(min=1e-12).to(torch.float32) / E4M3_MAX
+    scale = _div_scalar(amax.clamp(min=1e-12).to(torch.float32), E4M3_MAX, device_arith)
     return (w / scale).clamp(min=E4M3_MIN, max=E4M3_MAX).to(E4M3), scale
 
 
-def tensor_fp8_ref(w: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+def tensor_fp8_ref(w: torch.Tensor, device_arith: bool = False) -> tuple[torch.Tensor, torch.Tensor]:
     """tools/convert_hf_to_fp8.py:86-91 and quantizer_fp8.py:114-116 (scale shape [1])."""
-    scale = w.abs().max().clamp(min=1e-12).to(torch.float32) / E4M3_MAX
+    scale = _div_scalar(w.abs().max().clamp(min=1e-12).to(torch.float32), E4M3_MAX, device_arith)
+    if device_arith:
+        # torch's GPU kernel converts a 0-dim GPU operand to the common dtype (bf16) before dividing
+        return (w / scale.to(w.dtype)).clamp(min=E4M3_MIN, max=E4M3_MAX).to(E4M3), scale.view(1)
     return (w / scale).clamp(min=E4M3_MIN, max=E4M3_MAX).to(E4M3), scale.view(1)
 
 
@@ -172,3 +184,27 @@ def pack_layer_ref(weight: torch.Tensor, group_size: int, sym: bool = True):
         packed_zp = torch.sum(z, dim=-1).to(torch.int32)
     qi = quantize_ref(deq, scale, zp, torch.int8 if sym else torch.uint8)
     return pack_to_int32_ref(qi, 4, sym=sym), scale, packed_zp
+
+
+def int4_dequant_ref(packed: torch.Tensor, scale: torch.Tensor, shape, group_size: int) -> torch.Tensor:
+    """tools/convert_k2_thinking_int4_to_bf16.py:55-84 with the third-party unpack written out: nibble j of a word
+    at bits [4j, 4j+4), minus 8, as int8; then (int8.to(f32) * scale.to(f32) repeated per group).to(bf16)."""
+    rows, cols = shape
+    shifts = torch.arange(8, dtype=torch.int32) * 4
+    nib = ((packed.unsqueeze(-1) >> shifts) & 0xF).view(rows, -1)[:, :cols]
+    q = (nib - 8).to(torch.int8)
+    s = torch.repeat_interleave(scale.to(torch.float32), repeats=group_size, dim=1)
+    return (q.to(torch.float32) * s).to(torch.bfloat16).contiguous()
+
+
+def fake_int4_ste_ref(x: torch.Tensor, group_size: int, device_arith: bool = False) -> torch.Tensor:
+    """docker/patch/latest/megatron.patch:212-246 (_FakeInt4QuantizationSTE.forward), op for op."""
+    m, n = x.shape
+    n_pad = _cdiv(n, group_size) * group_size
+    xp = torch.zeros((m, n_pad), dtype=x.dtype, device=x.device)
+    xp[:m, :n] = x
+    view = xp.view(m, 1, n_pad // group_size, group_size)
+    x_max = view.abs().float().amax(dim=(1, 3), keepdim=True)
+    x_scale = _div_scalar(x_max, 7, device_arith).clamp(min=1e-5)
+    x_q = torch.round(view / x_scale).clamp(-7, 7)
+    return (x_q * x_scale).view_as(xp)[:m, :n].contiguous().to(x.dtype)

@@ -6,7 +6,8 @@
  * Every function is a scalar restatement of the arithmetic of one reference function
  * (paths relative to the reference checkout):
  *
- *   wqo_fp8_block_quant   mode 0: tools/convert_hf_to_fp8.py:41-75 (block_fp8)
+ *   wqo_fp8_block_quant   mode 0: tools/convert_hf_to_fp8.py:41-75 (block_fp8) as torch evaluates it on CPU tensors
+ *                         mode 2: the same, as torch evaluates it on GPU tensors (scalar division = reciprocal multiply)
  *                         mode 1: slime/backends/megatron_utils/kernels/fp8_kernel.py:24-58
  *   wqo_fp8_channel_quant tools/convert_hf_to_fp8.py:78-83 (channel_fp8)
  *   wqo_fp8_tensor_quant  tools/convert_hf_to_fp8.py:86-91 (tensor_fp8), same arithmetic as
@@ -16,6 +17,8 @@
  *   wqo_int4_fake_quant   slime/backends/megatron_utils/kernels/int4_qat/fake_int4_quant_cuda.cu:37-267
  *   wqo_int4_pack_layer   tools/convert_hf_to_int4_direct.py:32-153 (pack_layer, quantize,
  *                         round_to_quantized_type_dtype, pack_to_int32), literal chain
+ *   wqo_int4_dequant      tools/convert_k2_thinking_int4_to_bf16.py:55-84 (_dequantize_tensor)
+ *   wqo_int4_fake_ste     docker/patch/latest/megatron.patch:212-246 (_FakeInt4QuantizationSTE.forward)
  *
  * Number formats are handled with integer bit manipulation written for this file
  * (no library conversion is used), so that the torch restatement in torch_ref.py and
@@ -140,6 +143,22 @@ static inline float scale_from_amax_mode0(float amax_bf16_exact)
     return a / FP8_MAX;
 }
 
+/* The same expression as torch's GPU kernels evaluate it (mode 2): `tensor / python_scalar` is computed there
+ * as tensor * (1.0f / scalar) (aten/src/ATen/native/cuda/BinaryDivTrueKernel.cu, the is_cpu_scalar branch), so the
+ * scale is amax * RN(1/448).  The reference tool loads its tensors onto the accelerator
+ * (tools/convert_hf_to_fp8.py:127), so this is what it writes when a GPU is present; mode 0 is what its CPU test
+ * (tests/test_block_fp8_zero_block.py) exercises. */
+static inline float scale_from_amax_mode2(float amax_bf16_exact)
+{
+    float floor_v = wqo_bf16_to_f32(BF16_1EM12_BITS);
+    float a = amax_bf16_exact;
+    if (a == a && a < floor_v) a = floor_v;
+    volatile float inv = 1.0f / FP8_MAX;
+    return a * inv;
+}
+static inline float scale_torch(float amax, int mode)
+{ return mode == 2 ? scale_from_amax_mode2(amax) : scale_from_amax_mode0(amax); }
+
 static inline uint8_t quant_elem_mode0(float x, float scale)
 {
     float q = x / scale;                               /* true fp32 division, :67 */
@@ -171,7 +190,7 @@ static inline uint8_t quant_elem_mode1(float x, float s_inv)
 WQO_API int wqo_fp8_block_quant(const uint16_t *x, int64_t M, int64_t N, int64_t sx_m, int64_t sx_n,
                                 int64_t bm, int64_t bn, int mode, uint8_t *y, float *s)
 {
-    if (M < 0 || N < 0 || bm <= 0 || bn <= 0 || (mode != 0 && mode != 1)) return 1;
+    if (M < 0 || N < 0 || bm <= 0 || bn <= 0 || mode < 0 || mode > 2) return 1;
     int64_t nt = cdiv(M, bm), kt = cdiv(N, bn);
 #pragma omp parallel for schedule(static)
     for (int64_t bi = 0; bi < nt; ++bi) {
@@ -183,13 +202,13 @@ WQO_API int wqo_fp8_block_quant(const uint16_t *x, int64_t M, int64_t N, int64_t
                 for (int64_t j = c0; j < c1; ++j)
                     amax = max_nanprop(amax, fabsf(wqo_bf16_to_f32(x[i * sx_m + j * sx_n])));
             float scale, s_inv = 0.0f;
-            if (mode == 0) scale = scale_from_amax_mode0(amax);
+            if (mode != 1) scale = scale_torch(amax, mode);
             else { scale = scale_from_amax_mode1(amax); s_inv = 1.0f / scale; }
             s[bi * kt + bj] = scale;
             for (int64_t i = r0; i < r1; ++i)
                 for (int64_t j = c0; j < c1; ++j) {
                     float v = wqo_bf16_to_f32(x[i * sx_m + j * sx_n]);
-                    y[i * N + j] = mode == 0 ? quant_elem_mode0(v, scale) : quant_elem_mode1(v, s_inv);
+                    y[i * N + j] = mode != 1 ? quant_elem_mode0(v, scale) : quant_elem_mode1(v, s_inv);
                 }
         }
     }
@@ -197,15 +216,15 @@ WQO_API int wqo_fp8_block_quant(const uint16_t *x, int64_t M, int64_t N, int64_t
 }
 
 WQO_API int wqo_fp8_channel_quant(const uint16_t *x, int64_t M, int64_t N, int64_t sx_m, int64_t sx_n,
-                                  uint8_t *y, float *s)
+                                  int mode, uint8_t *y, float *s)
 {
-    if (M < 0 || N < 0) return 1;
+    if (M < 0 || N < 0 || (mode != 0 && mode != 2)) return 1;
 #pragma omp parallel for schedule(static)
     for (int64_t i = 0; i < M; ++i) {
         float amax = 0.0f;
         for (int64_t j = 0; j < N; ++j)
             amax = max_nanprop(amax, fabsf(wqo_bf16_to_f32(x[i * sx_m + j * sx_n])));
-        float scale = scale_from_amax_mode0(amax);
+        float scale = scale_torch(amax, mode);
         s[i] = scale;
         for (int64_t j = 0; j < N; ++j)
             y[i * N + j] = quant_elem_mode0(wqo_bf16_to_f32(x[i * sx_m + j * sx_n]), scale);
@@ -217,7 +236,9 @@ WQO_API int wqo_fp8_channel_quant(const uint16_t *x, int64_t M, int64_t N, int64
  * (quantizer_fp8.py:114-116): the scale is a 0-dim fp32 tensor, which does not take part in torch's
  * type promotion, so `weight / scale` is a bf16 tensor: the fp32 quotient is rounded to bf16 BEFORE the
  * clamp and the e4m3 cast (two roundings).  block_fp8 and channel_fp8 divide by a dimensioned fp32
- * tensor and keep the fp32 quotient. */
+ * tensor and keep the fp32 quotient.  On GPU tensors (mode 2) torch additionally converts the 0-dim divisor to
+ * the result dtype before dividing: the division is by bf16(scale), the scale returned stays fp32 (observed on
+ * torch 2.10 / ROCm: every element agrees with this reading, 1.7 % disagree with the fp32 divisor). */
 static inline uint8_t quant_elem_tensor(float x, float scale)
 {
     float q = wqo_bf16_to_f32(wqo_f32_to_bf16(x / scale));
@@ -226,19 +247,20 @@ static inline uint8_t quant_elem_tensor(float x, float scale)
 }
 
 WQO_API int wqo_fp8_tensor_quant(const uint16_t *x, int64_t M, int64_t N, int64_t sx_m, int64_t sx_n,
-                                 uint8_t *y, float *s)
+                                 int mode, uint8_t *y, float *s)
 {
-    if (M < 0 || N < 0) return 1;
+    if (M < 0 || N < 0 || (mode != 0 && mode != 2)) return 1;
     float amax = 0.0f;
     for (int64_t i = 0; i < M; ++i)
         for (int64_t j = 0; j < N; ++j)
             amax = max_nanprop(amax, fabsf(wqo_bf16_to_f32(x[i * sx_m + j * sx_n])));
-    float scale = scale_from_amax_mode0(amax);
+    float scale = scale_torch(amax, mode);
+    float divisor = mode == 2 ? wqo_bf16_to_f32(wqo_f32_to_bf16(scale)) : scale;
     s[0] = scale;
 #pragma omp parallel for schedule(static)
     for (int64_t i = 0; i < M; ++i)
         for (int64_t j = 0; j < N; ++j)
-            y[i * N + j] = quant_elem_tensor(wqo_bf16_to_f32(x[i * sx_m + j * sx_n]), scale);
+            y[i * N + j] = quant_elem_tensor(wqo_bf16_to_f32(x[i * sx_m + j * sx_n]), divisor);
     return 0;
 }
 
@@ -392,6 +414,51 @@ WQO_API int wqo_int4_pack_layer(const uint16_t *w, int64_t M, int64_t N, int64_t
             }
     }
     free(q); free(zb); free(nib);
+    return 0;
+}
+
+/* ------------------------------------------------------------------ INT4 -> bf16, QAT forward */
+
+/* y[i,j] = bf16( f32(nibble(i,j) - 8) * f32(scale[i, j/gs]) ); nibble j of word c at bits [4j,4j+4).
+ * tools/convert_k2_thinking_int4_to_bf16.py:55-84 (_dequantize_tensor); the unpacking there is
+ * compressed_tensors.unpack_from_int32 (third party, not vendored: PARITY UNPINNED against it; the bit layout is
+ * the inverse of pack_to_int32, tools/convert_hf_to_int4_direct.py:32-75, which is pinned). */
+WQO_API int wqo_int4_dequant(const int32_t *packed, const uint16_t *scale, int64_t M, int64_t N, int64_t gs,
+                             uint16_t *y)
+{
+    if (M < 0 || N < 0 || gs <= 0 || N % gs != 0 || N % 8 != 0) return 1;
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < M; ++i)
+        for (int64_t j = 0; j < N; ++j) {
+            uint32_t w = (uint32_t)packed[i * (N / 8) + j / 8];
+            int q = (int)((w >> (4 * (j % 8))) & 0xFu) - 8;
+            float s = wqo_bf16_to_f32(scale[i * (N / gs) + j / gs]);
+            y[i * N + j] = wqo_f32_to_bf16((float)q * s);
+        }
+    return 0;
+}
+
+/* Forward of the INT4 QAT straight-through estimator, docker/patch/latest/megatron.patch:212-246:
+ * s = clamp(f32(amax_bf16) / 7, min=1e-5); y = bf16( clamp(round(f32(x) / s), -7, 7) * s ).  bf16 [M,N], N % gs == 0.
+ * div7 = 0: `/ 7` is a division (torch on CPU tensors); 1: a multiplication by RN(1/7) (torch on GPU tensors, the
+ * only place this function runs in the reference). */
+WQO_API int wqo_int4_fake_ste(const uint16_t *x, int64_t M, int64_t N, int64_t gs, int div7, uint16_t *y)
+{
+    if (M < 0 || N < 0 || gs <= 0 || N % gs != 0 || (div7 != 0 && div7 != 1)) return 1;
+    volatile float inv7 = 1.0f / 7.0f;
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < M; ++i)
+        for (int64_t g = 0; g < N / gs; ++g) {
+            float amax = 0.0f;
+            for (int64_t k = 0; k < gs; ++k) amax = max_nanprop(amax, fabsf(wqo_bf16_to_f32(x[i * N + g * gs + k])));
+            float s = div7 ? amax * inv7 : amax / 7.0f;
+            if (s == s && s < 1e-5f) s = 1e-5f;
+            for (int64_t k = 0; k < gs; ++k) {
+                float q = rintf(wqo_bf16_to_f32(x[i * N + g * gs + k]) / s);
+                q = clamp_nanprop(q, -7.0f, 7.0f);
+                y[i * N + g * gs + k] = wqo_f32_to_bf16(q * s);
+            }
+        }
     return 0;
 }
 

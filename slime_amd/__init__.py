@@ -6,7 +6,8 @@ own function names.  Everything computes in hand-written gfx950 HIP kernels reac
 of ``slime_amd/lib/libslime_amd_wq.so``; there is no CPU or pure-torch fallback.
 """
 
-from . import _lib
+from . import _lib, arith
+from .arith import get_torch_arithmetic, set_torch_arithmetic, torch_arithmetic
 from .fp8 import (
     Fp8DequantPlan,
     Fp8QuantPlan,
@@ -19,7 +20,15 @@ from .fp8 import (
     weight_dequant,
     weight_dequant_bf16_scale,
 )
-from .int4 import Int4PackPlan, fake_int4_quant_cuda, pack_layer, pack_to_int32, quantize
+from .int4 import (
+    Int4PackPlan,
+    dequantize_int4,
+    fake_int4_quant_cuda,
+    fake_int4_quantization_ste,
+    pack_layer,
+    pack_to_int32,
+    quantize,
+)
 from .processors import (
     _quantize_param,
     quantize_params,
@@ -33,7 +42,9 @@ quantize_weight = blockwise_cast_to_fp8_triton
 
 __all__ = [
     "Fp8DequantPlan", "Fp8QuantPlan", "Int4PackPlan", "block_fp8", "block_fp8_many",
-    "blockwise_cast_to_fp8_triton", "channel_fp8", "fake_int4_quant_cuda", "pack_layer", "pack_to_int32",
+    "blockwise_cast_to_fp8_triton", "channel_fp8", "dequantize_int4", "fake_int4_quant_cuda",
+    "fake_int4_quantization_ste", "get_torch_arithmetic", "set_torch_arithmetic", "torch_arithmetic",
+    "pack_layer", "pack_to_int32",
     "quant_fp8", "quantize", "quantize_params", "quantize_params_compressed_tensors", "quantize_params_fp8",
     "quantize_weight", "tensor_fp8", "weight_dequant", "weight_dequant_bf16_scale", "_quantize_param",
 ]

@@ -15,11 +15,12 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libslime_amd_wq.so")
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 # selectors (mirrors of the header's enums)
 DTYPE_BF16, DTYPE_F32 = 0, 1
-FP8_MODE_TORCH, FP8_MODE_TRITON = 0, 1
+FP8_MODE_TORCH, FP8_MODE_TRITON, FP8_MODE_TORCH_DEVICE = 0, 1, 2
+DIV7_IEEE, DIV7_DEVICE = 0, 1
 DEQ_MODE_F32SCALE, DEQ_MODE_BF16SCALE = 0, 1
 DEQ_SEG, DEQ_SEGS_PER_WG = 512, 16
 INT4_GROUPS_PER_WG = 64
@@ -32,13 +33,15 @@ SIGNATURES = {
     "wq_error_string": [_int],
     "wq_fp8_block_quant": [_vp, _i64, _i64, _i64, _i64, _vp, _i64, _vp, _int, _int, _int, _vp],
     "wq_fp8_block_quant_grouped": [_vp, _vp, _int, _i64, _int, _int, _int, _vp],
-    "wq_fp8_row_quant": [_vp, _i64, _i64, _i64, _i64, _vp, _i64, _vp, _vp],
-    "wq_fp8_tensor_quant": [_vp, _i64, _i64, _i64, _i64, _vp, _i64, _vp, _vp, _vp],
+    "wq_fp8_row_quant": [_vp, _i64, _i64, _i64, _i64, _vp, _i64, _vp, _int, _vp],
+    "wq_fp8_tensor_quant": [_vp, _i64, _i64, _i64, _i64, _vp, _i64, _vp, _vp, _int, _vp],
     "wq_fp8_block_dequant": [_vp, _vp, _vp, _int, _i64, _i64, _int, _int, _vp],
     "wq_fp8_block_dequant_grouped": [_vp, _vp, _int, _i64, _int, _int, _int, _vp],
     "wq_int4_fake_quant": [_vp, _int, _i64, _i64, _i64, _i64, _int, _int, _int, _vp, _vp, _vp, _vp],
     "wq_int4_group_quant_pack": [_vp, _i64, _i64, _i64, _int, _vp, _vp, _vp],
     "wq_int4_group_quant_pack_grouped": [_vp, _vp, _int, _i64, _int, _vp],
+    "wq_int4_dequant": [_vp, _vp, _vp, _i64, _i64, _int, _vp],
+    "wq_int4_fake_quant_ste": [_vp, _vp, _i64, _i64, _int, _int, _vp],
     "wq_selftest_fp8_elem": [_u32, _u32, _int, _vp, _vp],
     "wq_selftest_int4_elem": [_u32, _u32, _vp, _vp],
     "wq_selftest_cvt_fp8": [_u64, _u64, _vp, _vp],

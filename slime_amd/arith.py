@@ -1,0 +1,54 @@
+"""Which of torch's two evaluations of ``tensor / python_scalar`` the torch-formulated functions reproduce.
+
+The reference computes its FP8 scales as ``amax.to(float32) / 448`` (tools/convert_hf_to_fp8.py:65,80,87;
+quantizer_fp8.py:114) and the INT4 QAT scale as ``amax / 7`` (docker/patch/latest/megatron.patch:240).  torch
+evaluates such an expression as an IEEE division on CPU tensors and as a multiplication by the rounded
+reciprocal on GPU tensors; the two differ in the last bit for about half of all amax values.  The reference
+runs these functions on the accelerator (convert_hf_to_fp8.py:127) and its test-suite on the CPU
+(tests/test_block_fp8_zero_block.py), so both results are "the reference's".
+
+``"device"`` (default): bit-identical to the reference running on a GPU.
+``"cpu"``: bit-identical to the reference running on CPU tensors.
+The Triton-formulated ``blockwise_cast_to_fp8_triton`` and ``fake_int4_quant_cuda`` are not affected.
+"""
+
+from __future__ import annotations
+
+import contextlib
+import os
+
+from . import _lib
+
+_KINDS = ("device", "cpu")
+_kind = os.environ.get("SLIME_AMD_TORCH_ARITHMETIC", "device")
+if _kind not in _KINDS:
+    raise ValueError(f"SLIME_AMD_TORCH_ARITHMETIC must be one of {_KINDS}, got {_kind!r}")
+
+
+def get_torch_arithmetic() -> str:
+    return _kind
+
+
+def set_torch_arithmetic(kind: str) -> None:
+    global _kind
+    if kind not in _KINDS:
+        raise ValueError(f"torch arithmetic must be one of {_KINDS}, got {kind!r}")
+    _kind = kind
+
+
+@contextlib.contextmanager
+def torch_arithmetic(kind: str):
+    prev = _kind
+    set_torch_arithmetic(kind)
+    try:
+        yield
+    finally:
+        set_torch_arithmetic(prev)
+
+
+def fp8_torch_mode() -> int:
+    return _lib.FP8_MODE_TORCH_DEVICE if _kind == "device" else _lib.FP8_MODE_TORCH
+
+
+def div7_rule() -> int:
+    return _lib.DIV7_DEVICE if _kind == "device" else _lib.DIV7_IEEE

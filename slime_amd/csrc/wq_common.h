@@ -175,6 +175,14 @@ __device__ __forceinline__ float fp8_scale_torch(uint32_t amax_bf16_bits)
     uint32_t a = amax_bf16_bits < kBf16Floor1em12 ? kBf16Floor1em12 : amax_bf16_bits;
     return u2f(a << 16) / kFp8Max;
 }
+// mode TORCH_DEVICE: the same expression as torch's GPU kernels evaluate it.  There `tensor / python_scalar` is
+// computed as tensor * (1.0f / scalar), so the scale is f32(amax) * RN(1/448) - up to one ulp away from the
+// quotient above.
+__device__ __forceinline__ float fp8_scale_torch_device(uint32_t amax_bf16_bits)
+{
+    uint32_t a = amax_bf16_bits < kBf16Floor1em12 ? kBf16Floor1em12 : amax_bf16_bits;
+    return u2f(a << 16) * (1.0f / kFp8Max);
+}
 // mode TRITON: fp32 amax floored at 1e-10f.
 __device__ __forceinline__ float fp8_scale_triton(uint32_t amax_bf16_bits)
 {
@@ -182,6 +190,9 @@ __device__ __forceinline__ float fp8_scale_triton(uint32_t amax_bf16_bits)
     a = (a != a) ? a : fmaxf(a, 1e-10f);
     return a / kFp8Max;
 }
+
+// The two torch modes divide every element by the scale; the Triton mode multiplies by its reciprocal.
+constexpr bool fp8_mode_divides(int mode) { return mode != WQ_FP8_MODE_TRITON; }
 
 // Per-block constants of the element function.
 struct Fp8BlockParams {
@@ -194,7 +205,9 @@ template <int MODE>
 __device__ __forceinline__ Fp8BlockParams fp8_block_params(uint32_t amax_bf16_bits)
 {
     Fp8BlockParams p;
-    p.scale = MODE == WQ_FP8_MODE_TORCH ? fp8_scale_torch(amax_bf16_bits) : fp8_scale_triton(amax_bf16_bits);
+    p.scale = MODE == WQ_FP8_MODE_TORCH          ? fp8_scale_torch(amax_bf16_bits)
+              : MODE == WQ_FP8_MODE_TORCH_DEVICE ? fp8_scale_torch_device(amax_bf16_bits)
+                                                 : fp8_scale_triton(amax_bf16_bits);
     p.rcp = 1.0f / p.scale;
     p.fast = amax_bf16_bits < kBf16Inf;
     return p;
@@ -238,7 +251,7 @@ template <int MODE>
 __device__ __forceinline__ uint32_t fp8_quant4_fast(uint32_t w0, uint32_t w1, const Fp8BlockParams& p)
 {
     float q0, q1, q2, q3;
-    if (MODE == WQ_FP8_MODE_TORCH) {
+    if (fp8_mode_divides(MODE)) {
         q0 = div_by_scale(bf16lo(w0), p.scale, p.rcp);
         q1 = div_by_scale(bf16hi(w0), p.scale, p.rcp);
         q2 = div_by_scale(bf16lo(w1), p.scale, p.rcp);
@@ -253,14 +266,14 @@ __device__ __forceinline__ uint32_t fp8_quant4_fast(uint32_t w0, uint32_t w1, co
     // so the clamp of the reference is a no-op here and is skipped.
     uint32_t r = cvt_pk_fp8_lo(q0, q1, 0u);
     r = cvt_pk_fp8_hi(q2, q3, r);
-    if (MODE == WQ_FP8_MODE_TORCH) r |= bf16x4_signs_to_bytes(w0, w1);
+    if (fp8_mode_divides(MODE)) r |= bf16x4_signs_to_bytes(w0, w1);
     return r;
 }
 
 template <int MODE>
 __device__ __forceinline__ uint32_t fp8_quant1_exact(float x, const Fp8BlockParams& p)
 {
-    return MODE == WQ_FP8_MODE_TORCH ? fp8_elem_exact_torch(x, p.scale) : fp8_elem_exact_triton(x, p.rcp);
+    return fp8_mode_divides(MODE) ? fp8_elem_exact_torch(x, p.scale) : fp8_elem_exact_triton(x, p.rcp);
 }
 
 template <int MODE>

@@ -177,10 +177,17 @@ __global__ __launch_bounds__(kTileThreads) void fp8_block_quant_kernel(const Fp8
 
 // ---- per-row (channel) and per-tensor scaling -------------------------------------------------
 
+// The row and tensor forms exist only in the torch formulation; the scale rule is a run-time choice there.
+__device__ __forceinline__ Fp8BlockParams torch_params(uint32_t amax_bf16_bits, int mode)
+{
+    return mode == WQ_FP8_MODE_TORCH_DEVICE ? fp8_block_params<WQ_FP8_MODE_TORCH_DEVICE>(amax_bf16_bits)
+                                            : fp8_block_params<WQ_FP8_MODE_TORCH>(amax_bf16_bits);
+}
+
 // One workgroup per row: amax over the row, then quantise.  Second pass re-reads the row (L2).
 __global__ __launch_bounds__(256) void fp8_row_quant_kernel(const uint16_t* __restrict__ x, int64_t M, int64_t N,
                                                            int64_t sx_m, int64_t sx_n, uint8_t* __restrict__ y,
-                                                           int64_t sy_m, float* __restrict__ s)
+                                                           int64_t sy_m, float* __restrict__ s, int mode)
 {
     __shared__ uint32_t lds[4];
     const int64_t row = (int64_t)blockIdx.x + (int64_t)blockIdx.y * gridDim.x;
@@ -192,7 +199,7 @@ __global__ __launch_bounds__(256) void fp8_row_quant_kernel(const uint16_t* __re
     if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6] = m;
     __syncthreads();
     m = max(max(lds[0], lds[1]), max(lds[2], lds[3]));
-    const Fp8BlockParams p = fp8_block_params<WQ_FP8_MODE_TORCH>(m);
+    const Fp8BlockParams p = torch_params(m, mode);
     if (threadIdx.x == 0) s[row] = p.scale;
     uint8_t* yr = y + row * sy_m;
     for (int64_t j = threadIdx.x; j < N; j += 256)
@@ -218,26 +225,46 @@ __global__ __launch_bounds__(256) void fp8_tensor_amax_kernel(const uint16_t* __
 __global__ __launch_bounds__(256) void fp8_tensor_apply_kernel(const uint16_t* __restrict__ x, int64_t M, int64_t N,
                                                               int64_t sx_m, int64_t sx_n, uint8_t* __restrict__ y,
                                                               int64_t sy_m, float* __restrict__ s,
-                                                              const uint32_t* __restrict__ ws)
+                                                              const uint32_t* __restrict__ ws, int mode)
 {
-    const Fp8BlockParams p = fp8_block_params<WQ_FP8_MODE_TORCH>(*ws);
+    const Fp8BlockParams p = torch_params(*ws, mode);
     if (blockIdx.x == 0 && threadIdx.x == 0) s[0] = p.scale;
     const int64_t total = M * N;
+    // The reference divides a bf16 tensor by a 0-dim fp32 tensor, which torch evaluates as a bf16
+    // result: the fp32 quotient is rounded to bf16 before the clamp and the e4m3 cast.  On GPU tensors
+    // torch also converts the 0-dim divisor to the result dtype first, so the division there is by
+    // bf16(scale) while the scale returned stays fp32.
+    const float divisor = mode == WQ_FP8_MODE_TORCH_DEVICE ? u2f(f32_to_bf16_bits(p.scale) << 16) : p.scale;
     for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < total; e += (int64_t)gridDim.x * 256) {
         int64_t i = e / N, j = e - i * N;
-        // The reference divides a bf16 tensor by a 0-dim fp32 tensor, which torch evaluates as a bf16
-        // result: the fp32 quotient is rounded to bf16 before the clamp and the e4m3 cast.
-        float q = u2f((uint32_t)x[i * sx_m + j * sx_n] << 16) / p.scale;
+        float q = u2f((uint32_t)x[i * sx_m + j * sx_n] << 16) / divisor;
         q = u2f(f32_to_bf16_bits(q) << 16);
         if (q == q) q = fminf(fmaxf(q, -kFp8Max), kFp8Max);
         y[i * sy_m + j] = (uint8_t)f32_to_e4m3fn_sw(q);
     }
 }
 
+static bool known_mode(int mode)
+{
+    return mode == WQ_FP8_MODE_TORCH || mode == WQ_FP8_MODE_TRITON || mode == WQ_FP8_MODE_TORCH_DEVICE;
+}
+
+template <bool GROUPED>
+static void launch_block_quant(const Fp8QuantArgs& a, int64_t tiles, int mode, hipStream_t st)
+{
+    const dim3 g = grid_for_items(tiles);
+    if (mode == WQ_FP8_MODE_TORCH)
+        fp8_block_quant_kernel<WQ_FP8_MODE_TORCH, GROUPED><<<g, kTileThreads, kOccupancyPadBytes, st>>>(a, tiles);
+    else if (mode == WQ_FP8_MODE_TORCH_DEVICE)
+        fp8_block_quant_kernel<WQ_FP8_MODE_TORCH_DEVICE, GROUPED><<<g, kTileThreads, kOccupancyPadBytes, st>>>(a, tiles);
+    else
+        fp8_block_quant_kernel<WQ_FP8_MODE_TRITON, GROUPED><<<g, kTileThreads, kOccupancyPadBytes, st>>>(a, tiles);
+}
+
 static int check_desc_host(const void* x, int64_t M, int64_t N, const void* y, const float* s, int bm, int bn, int mode)
 {
     if (M < 0 || N < 0 || bm <= 0 || bn <= 0) return WQ_ERR_SHAPE;
-    if (mode != WQ_FP8_MODE_TORCH && mode != WQ_FP8_MODE_TRITON) return WQ_ERR_MODE;
+    if (!known_mode(mode)) return WQ_ERR_MODE;
     if (M > 0 && N > 0 && (!x || !y || !s)) return WQ_ERR_NULL;
     if ((int64_t)bm * bn > (1 << 30)) return WQ_ERR_TOO_LARGE;
     return WQ_OK;
@@ -259,10 +286,7 @@ WQ_EXPORT int wq_fp8_block_quant(const void* x, int64_t M, int64_t N, int64_t sx
     a.bn = bn;
     const int64_t tiles = cdiv64(M, bm) * cdiv64(N, bn);
     hipStream_t st = (hipStream_t)stream;
-    if (mode == WQ_FP8_MODE_TORCH)
-        fp8_block_quant_kernel<WQ_FP8_MODE_TORCH, false><<<grid_for_items(tiles), kTileThreads, kOccupancyPadBytes, st>>>(a, tiles);
-    else
-        fp8_block_quant_kernel<WQ_FP8_MODE_TRITON, false><<<grid_for_items(tiles), kTileThreads, kOccupancyPadBytes, st>>>(a, tiles);
+    launch_block_quant<false>(a, tiles, mode, st);
     WQ_LAUNCH_CHECK();
     return WQ_OK;
 }
@@ -271,7 +295,7 @@ WQ_EXPORT int wq_fp8_block_quant_grouped(const wq_fp8_quant_desc* descs, const i
                                          int64_t total_tiles, int bm, int bn, int mode, void* stream)
 {
     if (n_desc < 0 || total_tiles < 0 || bm <= 0 || bn <= 0) return WQ_ERR_SHAPE;
-    if (mode != WQ_FP8_MODE_TORCH && mode != WQ_FP8_MODE_TRITON) return WQ_ERR_MODE;
+    if (!known_mode(mode)) return WQ_ERR_MODE;
     if (n_desc == 0 || total_tiles == 0) return WQ_OK;
     if (!descs || !tile_start) return WQ_ERR_NULL;
     if ((int64_t)bm * bn > (1 << 30)) return WQ_ERR_TOO_LARGE;
@@ -282,30 +306,29 @@ WQ_EXPORT int wq_fp8_block_quant_grouped(const wq_fp8_quant_desc* descs, const i
     a.bm = bm;
     a.bn = bn;
     hipStream_t st = (hipStream_t)stream;
-    if (mode == WQ_FP8_MODE_TORCH)
-        fp8_block_quant_kernel<WQ_FP8_MODE_TORCH, true><<<grid_for_items(total_tiles), kTileThreads, kOccupancyPadBytes, st>>>(a, total_tiles);
-    else
-        fp8_block_quant_kernel<WQ_FP8_MODE_TRITON, true><<<grid_for_items(total_tiles), kTileThreads, kOccupancyPadBytes, st>>>(a, total_tiles);
+    launch_block_quant<true>(a, total_tiles, mode, st);
     WQ_LAUNCH_CHECK();
     return WQ_OK;
 }
 
 WQ_EXPORT int wq_fp8_row_quant(const void* x, int64_t M, int64_t N, int64_t sx_m, int64_t sx_n, void* y,
-                               int64_t sy_m, float* s, void* stream)
+                               int64_t sy_m, float* s, int mode, void* stream)
 {
     if (M < 0 || N < 0) return WQ_ERR_SHAPE;
+    if (mode != WQ_FP8_MODE_TORCH && mode != WQ_FP8_MODE_TORCH_DEVICE) return WQ_ERR_MODE;
     if (M == 0) return WQ_OK;
     if (!s || (N > 0 && (!x || !y))) return WQ_ERR_NULL;
     fp8_row_quant_kernel<<<grid_for_items(M), 256, 0, (hipStream_t)stream>>>((const uint16_t*)x, M, N, sx_m, sx_n,
-                                                                      (uint8_t*)y, sy_m, s);
+                                                                      (uint8_t*)y, sy_m, s, mode);
     WQ_LAUNCH_CHECK();
     return WQ_OK;
 }
 
 WQ_EXPORT int wq_fp8_tensor_quant(const void* x, int64_t M, int64_t N, int64_t sx_m, int64_t sx_n, void* y,
-                                  int64_t sy_m, float* s, uint32_t* workspace, void* stream)
+                                  int64_t sy_m, float* s, uint32_t* workspace, int mode, void* stream)
 {
     if (M < 0 || N < 0) return WQ_ERR_SHAPE;
+    if (mode != WQ_FP8_MODE_TORCH && mode != WQ_FP8_MODE_TORCH_DEVICE) return WQ_ERR_MODE;
     if (!s || !workspace || (M * N > 0 && (!x || !y))) return WQ_ERR_NULL;
     const int64_t total = M * N;
     int blocks = (int)min((int64_t)(256 * 16), max((int64_t)1, cdiv64(total, 256 * 8)));
@@ -313,7 +336,7 @@ WQ_EXPORT int wq_fp8_tensor_quant(const void* x, int64_t M, int64_t N, int64_t s
     fp8_tensor_amax_kernel<<<blocks, 256, 0, st>>>((const uint16_t*)x, M, N, sx_m, sx_n, workspace);
     WQ_LAUNCH_CHECK();
     fp8_tensor_apply_kernel<<<blocks, 256, 0, st>>>((const uint16_t*)x, M, N, sx_m, sx_n, (uint8_t*)y, sy_m, s,
-                                                   workspace);
+                                                   workspace, mode);
     WQ_LAUNCH_CHECK();
     return WQ_OK;
 }

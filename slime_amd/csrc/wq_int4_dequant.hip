@@ -1,0 +1,165 @@
+// INT4 pack-quantized -> bf16, and the quantise-dequantise forward of the INT4 QAT straight-through
+// estimator, for gfx950.
+//
+// int4_dequant_kernel: every lane turns one packed int32 (8 nibbles) into 8 bf16 and writes them with ONE
+// 16-byte store, so a wavefront reads 256 contiguous bytes and writes 1 KiB contiguous per step; eight steps
+// per lane are all in flight before first use.  f32(nibble - 8) * f32(scale) has at most 12 significant bits,
+// so the fp32 product is exact and the only rounding is the final one to bf16, as in the reference's
+// (int8.to(f32) * scale.to(f32)).to(bf16).
+//
+// int4_fake_ste_kernel: a 128-element group is owned by 16 adjacent lanes (32 / 64: 4 / 8 lanes), one 16-byte
+// load and one 16-byte store per lane; x / s is an IEEE division, amax / 7 a division or a multiplication by RN(1/7)
+// (torch evaluates `tensor / 7` the first way on CPU tensors and the second way on GPU tensors).
+
+#include "wq_common.h"
+
+namespace wq {
+
+typedef float f32x2d __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2d __attribute__((ext_vector_type(2)));
+
+constexpr int kDqSteps = 8;                       // packed words per lane
+constexpr int kDqWordsPerWg = 256 * kDqSteps;     // 8 KiB of packed input, 32 KiB of bf16 output
+constexpr int kDqItemsPerXcdRun = 32;
+
+__device__ __forceinline__ uint32_t pack2_bf16(float a, float b)
+{
+    f32x2d v = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2d));
+}
+
+__global__ __launch_bounds__(256) void int4_dequant_kernel(const uint32_t* __restrict__ packed,
+                                                          const uint16_t* __restrict__ scale,
+                                                          uint16_t* __restrict__ y, int64_t n_words, int group,
+                                                          int64_t total_items)
+{
+    const int64_t slot = (int64_t)blockIdx.x + (int64_t)blockIdx.y * gridDim.x;
+    if (slot >= total_items) return;
+    const int64_t item = xcd_chunked_item(slot, total_items, kDqItemsPerXcdRun);
+    const int64_t w0 = item * kDqWordsPerWg + threadIdx.x;
+    const int gshift = (group & (group - 1)) == 0 ? __builtin_ctz((unsigned)group) : -1;
+    uint32_t w[kDqSteps];
+    uint32_t sb[kDqSteps];
+#pragma unroll
+    for (int i = 0; i < kDqSteps; ++i) {
+        // lanes past the end re-read the last word instead of branching around the load
+        const int64_t k = min(w0 + i * 256, n_words - 1);
+        w[i] = ldg_nt<uint32_t>(packed + k);
+        const int64_t g = gshift >= 0 ? (k * 8) >> gshift : (k * 8) / group;   // rows are whole groups: flat group index
+        sb[i] = ldg<uint16_t>(scale + g);
+    }
+#pragma unroll
+    for (int i = 0; i < kDqSteps; ++i) {
+        const int64_t k = w0 + i * 256;
+        if (k >= n_words) continue;
+        const float s = u2f(sb[i] << 16);
+        float f[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) f[j] = (float)((int)((w[i] >> (4 * j)) & 0xFu) - 8) * s;
+        const u32x4 o = {pack2_bf16(f[0], f[1]), pack2_bf16(f[2], f[3]), pack2_bf16(f[4], f[5]), pack2_bf16(f[6], f[7])};
+        stg_nt<u32x4>(y + k * 8, o);
+    }
+}
+
+// ---- QAT straight-through forward ------------------------------------------------------------------
+
+constexpr int kSteGroupsPerWg = 64;
+constexpr int kSteItemsPerXcdRun = 32;
+
+template <int L>
+__device__ __forceinline__ float ste_lanes_max(float v)
+{
+    v = fmaxf(v, u2f(dpp_u32<0xB1>(f2u(v))));
+    v = fmaxf(v, u2f(dpp_u32<0x4E>(f2u(v))));
+    if (L >= 8) v = fmaxf(v, u2f(dpp_u32<0x141>(f2u(v))));
+    if (L >= 16) v = fmaxf(v, u2f(dpp_u32<0x140>(f2u(v))));
+    return v;
+}
+
+template <int L>
+__global__ __launch_bounds__(256) void int4_fake_ste_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ y,
+                                                           int64_t n_groups, int64_t total_items, int div7)
+{
+    constexpr int CL = 256 / L;
+    constexpr int STEPS = kSteGroupsPerWg / CL;
+    const int64_t slot = (int64_t)blockIdx.x + (int64_t)blockIdx.y * gridDim.x;
+    if (slot >= total_items) return;
+    const int64_t item = xcd_chunked_item(slot, total_items, kSteItemsPerXcdRun);
+    const int cl = threadIdx.x / L, ll = threadIdx.x % L;
+    const int64_t g0 = item * kSteGroupsPerWg + cl;
+    u32x4 v[STEPS];
+#pragma unroll
+    for (int i = 0; i < STEPS; ++i) {
+        const int64_t g = min(g0 + i * CL, n_groups - 1);
+        v[i] = ldg_nt<u32x4>(x + g * (8 * L) + ll * 8);
+    }
+#pragma unroll
+    for (int i = 0; i < STEPS; ++i) {
+        const int64_t g = g0 + i * CL;
+        const uint32_t wd[4] = {v[i].x, v[i].y, v[i].z, v[i].w};
+        float xs[8];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) { xs[2 * j] = bf16lo(wd[j]); xs[2 * j + 1] = bf16hi(wd[j]); }
+        // amax in bf16 (exact), converted to fp32: x_view.abs().float().amax(); torch.amax propagates NaN, and so
+        // does the integer max on magnitude bits
+        uint32_t mb = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) mb = pk_absmax(mb, wd[j]);
+        mb = pk_fold(mb);
+        mb = max(mb, dpp_u32<0xB1>(mb));
+        mb = max(mb, dpp_u32<0x4E>(mb));
+        if (L >= 8) mb = max(mb, dpp_u32<0x141>(mb));
+        if (L >= 16) mb = max(mb, dpp_u32<0x140>(mb));
+        float s = div7 == WQ_DIV7_DEVICE ? u2f(mb << 16) * (1.0f / 7.0f) : u2f(mb << 16) / 7.0f;
+        s = (s != s) ? s : fmaxf(s, 1e-5f);           // clamp(min=1e-5) keeps NaN
+        float o[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            float q = __builtin_rintf(xs[j] / s);
+            if (q == q) q = fminf(fmaxf(q, -7.0f), 7.0f);
+            o[j] = q * s;
+        }
+        if (g < n_groups) {
+            const u32x4 r = {pack2_bf16(o[0], o[1]), pack2_bf16(o[2], o[3]), pack2_bf16(o[4], o[5]), pack2_bf16(o[6], o[7])};
+            stg_nt<u32x4>(y + g * (8 * L) + ll * 8, r);
+        }
+    }
+}
+
+}  // namespace wq
+
+using namespace wq;
+
+WQ_EXPORT int wq_int4_dequant(const int32_t* packed, const void* scale, void* y, int64_t M, int64_t N, int group,
+                              void* stream)
+{
+    if (M < 0 || N < 0 || group <= 0 || group % 8 != 0 || N % group != 0) return WQ_ERR_SHAPE;
+    if (M == 0 || N == 0) return WQ_OK;
+    if (!packed || !scale || !y) return WQ_ERR_NULL;
+    if (((uintptr_t)y & 15) || ((uintptr_t)packed & 3) || ((uintptr_t)scale & 1)) return WQ_ERR_ALIGN;
+    const int64_t n_words = M * (N / 8);
+    const int64_t items = cdiv64(n_words, kDqWordsPerWg);
+    int4_dequant_kernel<<<grid_for_items(items), 256, 0, (hipStream_t)stream>>>(
+        (const uint32_t*)packed, (const uint16_t*)scale, (uint16_t*)y, n_words, group, items);
+    WQ_LAUNCH_CHECK();
+    return WQ_OK;
+}
+
+WQ_EXPORT int wq_int4_fake_quant_ste(const void* x, void* y, int64_t M, int64_t N, int group, int div7, void* stream)
+{
+    if (M < 0 || N < 0 || group <= 0 || N % group != 0) return WQ_ERR_SHAPE;
+    if (div7 != WQ_DIV7_IEEE && div7 != WQ_DIV7_DEVICE) return WQ_ERR_MODE;
+    if (group != 32 && group != 64 && group != 128) return WQ_ERR_UNSUPPORTED;
+    if (M == 0 || N == 0) return WQ_OK;
+    if (!x || !y) return WQ_ERR_NULL;
+    if (((uintptr_t)x & 15) || ((uintptr_t)y & 15)) return WQ_ERR_ALIGN;
+    const int64_t n_groups = M * (N / group);
+    const int64_t items = cdiv64(n_groups, kSteGroupsPerWg);
+    hipStream_t st = (hipStream_t)stream;
+    const dim3 g = grid_for_items(items);
+    if (group == 32) int4_fake_ste_kernel<4><<<g, 256, 0, st>>>((const uint16_t*)x, (uint16_t*)y, n_groups, items, div7);
+    else if (group == 64) int4_fake_ste_kernel<8><<<g, 256, 0, st>>>((const uint16_t*)x, (uint16_t*)y, n_groups, items, div7);
+    else int4_fake_ste_kernel<16><<<g, 256, 0, st>>>((const uint16_t*)x, (uint16_t*)y, n_groups, items, div7);
+    WQ_LAUNCH_CHECK();
+    return WQ_OK;
+}

@@ -165,13 +165,14 @@ WQ_EXPORT int wq_selftest_fp8_elem(uint32_t amax_lo, uint32_t amax_hi, int mode,
 {
     if (!out) return WQ_ERR_NULL;
     if (amax_hi < amax_lo || amax_hi > 0x8000u) return WQ_ERR_SHAPE;
-    if (mode != WQ_FP8_MODE_TORCH && mode != WQ_FP8_MODE_TRITON) return WQ_ERR_MODE;
+    if (mode != WQ_FP8_MODE_TORCH && mode != WQ_FP8_MODE_TRITON && mode != WQ_FP8_MODE_TORCH_DEVICE) return WQ_ERR_MODE;
     hipStream_t st = (hipStream_t)stream;
     selftest_init_kernel<<<1, 1, 0, st>>>(out);
     WQ_LAUNCH_CHECK();
     if (amax_hi == amax_lo) return WQ_OK;
     dim3 grid(64, amax_hi - amax_lo, 1);
     if (mode == WQ_FP8_MODE_TORCH) selftest_fp8_elem_kernel<WQ_FP8_MODE_TORCH><<<grid, 256, 0, st>>>(amax_lo, amax_hi, out);
+    else if (mode == WQ_FP8_MODE_TORCH_DEVICE) selftest_fp8_elem_kernel<WQ_FP8_MODE_TORCH_DEVICE><<<grid, 256, 0, st>>>(amax_lo, amax_hi, out);
     else selftest_fp8_elem_kernel<WQ_FP8_MODE_TRITON><<<grid, 256, 0, st>>>(amax_lo, amax_hi, out);
     WQ_LAUNCH_CHECK();
     return WQ_OK;

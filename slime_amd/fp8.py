@@ -19,7 +19,7 @@ from typing import Sequence
 
 import torch
 
-from . import _lib
+from . import _lib, arith
 
 FP8_DTYPE = torch.float8_e4m3fn
 FP8_INFO = torch.finfo(FP8_DTYPE)
@@ -57,8 +57,9 @@ def block_fp8(weight: torch.Tensor, block_size) -> tuple[torch.Tensor, torch.Ten
     """-> (qweight float8_e4m3fn [M,N] contiguous, scale float32 [ceil(M/bn), ceil(N/bk)]).
 
     Arithmetic of tools/convert_hf_to_fp8.py:41-75: zero padding of edge blocks, amax clamped at
-    1e-12 in the weight dtype, scale = f32(amax)/448, q = clamp(f32(w)/scale), RNE to e4m3fn."""
-    return _block_quant(weight, int(block_size[0]), int(block_size[1]), _lib.FP8_MODE_TORCH, "block_fp8")
+    1e-12 in the weight dtype, scale = f32(amax)/448, q = clamp(f32(w)/scale), RNE to e4m3fn.  `/448` is
+    evaluated as torch does on GPU tensors unless ``arith.set_torch_arithmetic("cpu")`` is in force."""
+    return _block_quant(weight, int(block_size[0]), int(block_size[1]), arith.fp8_torch_mode(), "block_fp8")
 
 
 def channel_fp8(weight: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
@@ -70,7 +71,8 @@ def channel_fp8(weight: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
     if M:
         with torch.cuda.device(weight.device):
             rc = _lib.load().wq_fp8_row_quant(weight.data_ptr(), M, N, weight.stride(0), weight.stride(1),
-                                              q.data_ptr(), N, s.data_ptr(), _lib.stream_ptr(weight.device))
+                                              q.data_ptr(), N, s.data_ptr(), arith.fp8_torch_mode(),
+                                              _lib.stream_ptr(weight.device))
         _lib.check(rc, "channel_fp8")
     return q, s
 
@@ -84,7 +86,7 @@ def tensor_fp8(weight: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
     ws = torch.zeros((1,), dtype=torch.int32, device=weight.device)
     with torch.cuda.device(weight.device):
         rc = _lib.load().wq_fp8_tensor_quant(weight.data_ptr(), M, N, weight.stride(0), weight.stride(1),
-                                             q.data_ptr(), N, s.data_ptr(), ws.data_ptr(),
+                                             q.data_ptr(), N, s.data_ptr(), ws.data_ptr(), arith.fp8_torch_mode(),
                                              _lib.stream_ptr(weight.device))
     _lib.check(rc, "tensor_fp8")
     return q, s
@@ -159,15 +161,16 @@ class Fp8QuantPlan:
     Outputs live in two flat buffers owned by the plan (``flat_q`` bytes, ``flat_s`` fp32); ``outputs``
     holds per-tensor views ``(qweight [M,N] e4m3fn, scale [tm,tn])`` in input order.  The plan reads
     the weights' current contents on every run, so it can be reused across weight-sync steps as long
-    as the input tensors stay at the same addresses.  mode: 0 = ``block_fp8`` arithmetic,
+    as the input tensors stay at the same addresses.  mode: None = ``block_fp8`` arithmetic under the
+    current ``arith`` setting, 0 / 2 = ``block_fp8`` as torch evaluates it on CPU / GPU tensors,
     1 = ``blockwise_cast_to_fp8_triton`` arithmetic.
     """
 
-    def __init__(self, weights: Sequence[torch.Tensor], block_size=(128, 128), mode: int = 0):
+    def __init__(self, weights: Sequence[torch.Tensor], block_size=(128, 128), mode: int | None = None):
         if not weights:
             raise ValueError("Fp8QuantPlan: empty weight list")
         self.bm, self.bn = int(block_size[0]), int(block_size[1])
-        self.mode = int(mode)
+        self.mode = arith.fp8_torch_mode() if mode is None else int(mode)
         self.device = weights[0].device
         self.weights = list(weights)
         q_off, s_off, q_total, s_total = [], [], 0, 0
@@ -207,7 +210,7 @@ class Fp8QuantPlan:
         return self.outputs
 
 
-def block_fp8_many(weights: Sequence[torch.Tensor], block_size=(128, 128), mode: int = 0):
+def block_fp8_many(weights: Sequence[torch.Tensor], block_size=(128, 128), mode: int | None = None):
     """One-launch ``block_fp8`` over a list of weights -> list of (qweight, scale)."""
     return Fp8QuantPlan(weights, block_size, mode).run() if weights else []
 

@@ -19,7 +19,7 @@ from typing import Sequence
 
 import torch
 
-from . import _lib
+from . import _lib, arith
 
 
 def _dtype_sel(t: torch.Tensor, what: str) -> int:
@@ -191,3 +191,75 @@ class Int4PackPlan:
                                                               _lib.stream_ptr(self.device))
         _lib.check(rc, "Int4PackPlan.run")
         return self.outputs
+
+
+# ------------------------------------------------------------------------------------ inverse and QAT forward
+
+
+def dequantize_int4(weight_packed: torch.Tensor, weight_scale: torch.Tensor, weight_shape, group_size: int) -> torch.Tensor:
+    """pack-quantized INT4 -> bf16: ``((nibble - 8).to(f32) * scale.to(f32)).to(bf16)`` with the scale of each
+    ``group_size`` columns, the arithmetic of ``_dequantize_tensor`` in
+    tools/convert_k2_thinking_int4_to_bf16.py:55-84 (its unpacking step is ``compressed_tensors.unpack_from_int32``:
+    nibble j of a word at bits [4j, 4j+4), offset 8).  ``weight_shape`` is the ``.weight_shape`` tensor or a tuple."""
+    _lib.require_gpu(weight_packed, "dequantize_int4")
+    shape = tuple(int(v) for v in (weight_shape.view(-1).tolist() if isinstance(weight_shape, torch.Tensor) else weight_shape))
+    if len(shape) != 2:
+        raise ValueError(f"dequantize_int4: expected a 2-D weight shape, got {shape}")
+    M, N = shape
+    if weight_packed.dtype != torch.int32 or tuple(weight_packed.shape) != (M, -(-N // 8)):
+        raise ValueError(f"dequantize_int4: weight_packed {tuple(weight_packed.shape)} {weight_packed.dtype} does not "
+                         f"match shape {shape}")
+    if group_size <= 0 or N % group_size != 0 or group_size % 8 != 0:
+        raise ValueError(f"dequantize_int4: group_size {group_size} must be a multiple of 8 that divides N={N}")
+    scale = weight_scale.unsqueeze(1) if weight_scale.dim() == 1 else weight_scale
+    if scale.numel() != M * (N // group_size):
+        raise ValueError(f"Scale shape {tuple(weight_scale.shape)} incompatible with weight shape {shape}")
+    scale = scale.to(torch.bfloat16).contiguous()
+    packed = weight_packed.contiguous()
+    y = torch.empty((M, N), dtype=torch.bfloat16, device=packed.device)
+    if M and N:
+        with torch.cuda.device(packed.device):
+            rc = _lib.load().wq_int4_dequant(packed.data_ptr(), scale.data_ptr(), y.data_ptr(), M, N, int(group_size),
+                                             _lib.stream_ptr(packed.device))
+        _lib.check(rc, "dequantize_int4")
+    return y
+
+
+class _FakeInt4QuantizationSTE(torch.autograd.Function):
+    """Quantise-dequantise forward, identity backward (docker/patch/latest/megatron.patch:212-255)."""
+
+    @staticmethod
+    def forward(ctx, x, group_size):
+        _lib.require_gpu(x, "fake_int4_quantization_ste")
+        m, n = x.shape
+        if x.dtype == torch.bfloat16 and group_size in (32, 64, 128) and n % group_size == 0:
+            xc = x.contiguous()
+            y = torch.empty_like(xc)
+            if m and n:
+                with torch.cuda.device(x.device):
+                    rc = _lib.load().wq_int4_fake_quant_ste(xc.data_ptr(), y.data_ptr(), m, n, int(group_size),
+                                                            arith.div7_rule(), _lib.stream_ptr(x.device))
+                _lib.check(rc, "fake_int4_quantization_ste")
+            return y
+        # ragged widths, other group sizes or dtypes: the reference's own tensor ops, on the GPU
+        n_pad = -(-n // group_size) * group_size
+        xp = torch.zeros((m, n_pad), dtype=x.dtype, device=x.device)
+        xp[:, :n] = x
+        view = xp.view(m, 1, n_pad // group_size, group_size)
+        amax = view.abs().float().amax(dim=(1, 3), keepdim=True)
+        # `amax / 7` is torch's GPU evaluation (a reciprocal multiply); a tensor divisor forces the IEEE division
+        seven = 7 if arith.get_torch_arithmetic() == "device" else torch.full((), 7.0, device=x.device)
+        scale = (amax / seven).clamp(min=1e-5)
+        deq = torch.round(view / scale).clamp(-7, 7) * scale
+        return deq.view_as(xp)[:, :n].contiguous().to(x.dtype)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        return grad_output, None
+
+
+def fake_int4_quantization_ste(x: torch.Tensor, group_size: int) -> torch.Tensor:
+    out = _FakeInt4QuantizationSTE.apply(x, group_size)
+    if hasattr(x, "main_grad"):
+        out.main_grad = x.main_grad
+    return out

@@ -130,12 +130,14 @@ class BucketPipeline:
         return sum(s.elapsed_time(e) for s, e in self.kernel_events)
 
 
-def fp8_block_quant_kernel(block_size=(128, 128), mode: int = _lib.FP8_MODE_TORCH) -> Callable[[torch.Tensor], tuple]:
+def fp8_block_quant_kernel(block_size=(128, 128), mode: int | None = None) -> Callable[[torch.Tensor], tuple]:
     """Kernel adaptor for BucketPipeline: bf16 [M,N] -> (e4m3fn [M,N], fp32 scale_inv)."""
+    from . import arith
     from .fp8 import _block_quant
 
     def run(w: torch.Tensor):
-        return _block_quant(w, int(block_size[0]), int(block_size[1]), mode, "stream.fp8_block_quant")
+        m = arith.fp8_torch_mode() if mode is None else mode
+        return _block_quant(w, int(block_size[0]), int(block_size[1]), m, "stream.fp8_block_quant")
 
     return run
 

@@ -69,7 +69,7 @@ def process_file(input_path, output_path, filename, strategy, block_size, result
     if todo:
         on_gpu = [_shards.to_device(weights[k], dev) for k in todo]
         if strategy not in ("tensor", "channel"):
-            plan = Fp8QuantPlan(on_gpu, block_size, mode=0)
+            plan = Fp8QuantPlan(on_gpu, block_size)
             plan.run()
             flat_q, flat_s = plan.flat_q.cpu(), plan.flat_s.cpu()     # two copies for the whole shard
             qbase, sbase = plan.flat_q.data_ptr(), plan.flat_s.data_ptr()

@@ -2,8 +2,10 @@
 
 Inputs are seeded; expected outputs come from the op-for-op torch restatement of the reference
 (oracle/torch_ref.py) run on the CPU - the same torch primitives, in the same order and dtypes, as
-tools/convert_hf_to_fp8.py:41-75, fp8_kernel.py:24-58 (read as IEEE arithmetic), tools/fp8_cast_bf16.py:25-28
-and tools/convert_hf_to_int4_direct.py:32-153.  The reference's own Python was NOT imported or run to make
+tools/convert_hf_to_fp8.py:41-75, fp8_kernel.py:24-58 (read as IEEE arithmetic), tools/fp8_cast_bf16.py:25-28,
+tools/convert_hf_to_int4_direct.py:32-153, tools/convert_k2_thinking_int4_to_bf16.py:55-84 and
+docker/patch/latest/megatron.patch:212-246.  The `*_dev` entries hold the same functions with `tensor / scalar`
+evaluated as torch's GPU kernels do (a multiplication by the rounded reciprocal).  The reference's own Python was NOT imported or run to make
 them: its functions on this path are pinned by the checks in tests/test_oracle_*.py, and its INT4 kernel
 cannot run without a CUDA device.  Also stored: the data of the reference's known-answer test
 tests/test_hf_to_megatron.py:345-358.
@@ -47,6 +49,8 @@ def main():
         qc, sc = T.blockwise_cast_ref(w, (128, 128))
         out[f"{name}/w"] = w.contiguous()
         out[f"{name}/q_block"], out[f"{name}/s_block"] = q.contiguous(), s.contiguous()
+        qd, sd = T.block_fp8_ref(w, (128, 128), device_arith=True)      # as torch evaluates `/ 448` on GPU tensors
+        out[f"{name}/q_block_dev"], out[f"{name}/s_block_dev"] = qd.contiguous(), sd.contiguous()
         out[f"{name}/q_cast"], out[f"{name}/s_cast"] = qc.contiguous(), sc.contiguous()
         out[f"{name}/deq"] = T.weight_dequant_ref(q, s, 128).contiguous()
     kat_w = torch.linspace(-2, 2, 128 * 128).view(128, 128).to(torch.float8_e4m3fn)
@@ -68,6 +72,9 @@ def main():
         i4[f"{name}/w"] = w
         i4[f"{name}/q"], i4[f"{name}/scale"] = q, sc.contiguous()
         i4[f"{name}/packed"], i4[f"{name}/pack_scale"] = p.contiguous(), s2.contiguous()
+        i4[f"{name}/deq"] = T.int4_dequant_ref(p, s2, shape, gs)
+        i4[f"{name}/ste"] = T.fake_int4_ste_ref(w, gs)
+        i4[f"{name}/ste_dev"] = T.fake_int4_ste_ref(w, gs, device_arith=True)
         qa, sa, za = T.fake_int4_quant_ref(w, (1, gs), False)
         i4[f"{name}/q_asym"], i4[f"{name}/scale_asym"], i4[f"{name}/zero_asym"] = qa, sa.contiguous(), za.contiguous()
         if shape[0] % 8 == 0:

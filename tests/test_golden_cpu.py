@@ -20,7 +20,7 @@ def test_fp8_golden():
     assert len(_cases(f)) >= 5
     for case in _cases(f):
         w = f[f"{case}/w"]
-        for mode, tag in ((0, "block"), (1, "cast")):
+        for mode, tag in ((0, "block"), (1, "cast"), (2, "block_dev")):
             q, s = C.fp8_block_quant(w, (128, 128), mode)
             assert torch.equal(q, f[f"{case}/q_{tag}"].view(torch.uint8)), (case, tag)
             assert I.same_bits(s, f[f"{case}/s_{tag}"]), (case, tag)
@@ -43,6 +43,9 @@ def test_int4_golden():
         assert I.same_bits(q, f[f"{case}/q"]) and I.same_bits(s, f[f"{case}/scale"]), case
         p, s2, _ = C.int4_pack_layer(w, gs, True)
         assert torch.equal(p, f[f"{case}/packed"]) and I.same_bits(s2, f[f"{case}/pack_scale"]), case
+        assert I.same_bits(C.int4_dequant(p, s2, tuple(w.shape), gs), f[f"{case}/deq"]), case
+        assert I.same_bits(C.int4_fake_ste(w, gs, 0), f[f"{case}/ste"]), case
+        assert I.same_bits(C.int4_fake_ste(w, gs, 1), f[f"{case}/ste_dev"]), case
         qa, sa, za = C.int4_fake_quant(w, (1, gs), False)
         assert I.same_bits(qa, f[f"{case}/q_asym"]) and I.same_bits(sa, f[f"{case}/scale_asym"])
         assert I.same_bits(za, f[f"{case}/zero_asym"]), case

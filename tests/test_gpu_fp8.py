@@ -23,9 +23,16 @@ def _bits32(t):
     return t.cpu().contiguous().view(torch.int32)
 
 
+ARITH = {0: "cpu", 2: "device"}     # oracle mode -> torch arithmetic setting of the host layer
+DEFAULT_MODE = 2                    # the host layer's default: torch's GPU evaluation of `/ 448`
+
+
 def _check_block(w_cpu, w_gpu, block=(128, 128), mode=0):
-    fn = slime_amd.block_fp8 if mode == 0 else slime_amd.blockwise_cast_to_fp8_triton
-    q, s = fn(w_gpu, block)
+    if mode == 1:
+        q, s = slime_amd.blockwise_cast_to_fp8_triton(w_gpu, block)
+    else:
+        with slime_amd.torch_arithmetic(ARITH[mode]):
+            q, s = slime_amd.block_fp8(w_gpu, block)
     assert q.dtype == E4M3 and q.is_contiguous() and s.dtype == torch.float32
     qo, so = C.fp8_block_quant(w_cpu, block, mode)
     assert q.shape == qo.shape and s.shape == so.shape
@@ -40,16 +47,17 @@ SHAPES = [(128, 128), (256, 384), (300, 200), (7, 7168), (1, 1), (1, 8), (129, 1
 
 
 @pytest.mark.parametrize("shape", SHAPES)
-@pytest.mark.parametrize("mode", [0, 1])
+@pytest.mark.parametrize("mode", [0, 1, 2])
 def test_block_quant_shapes(cuda, shape, mode):
     w = I.zero_blocks(I.weights(*shape, seed=sum(shape)), 0.2, seed=1)
     _check_block(w, w.to(cuda), mode=mode)
 
 
-def test_block_quant_config1_roundtrip(cuda):
+@pytest.mark.parametrize("mode", [0, 2])
+def test_block_quant_config1_roundtrip(cuda, mode):
     # [4096,4096] N(0,0.02), 0.1% of entries x20, seed 0: quant then dequant of its own output
     w = I.weights(4096, 4096, seed=0)
-    q, s = _check_block(w, w.to(cuda))
+    q, s = _check_block(w, w.to(cuda), mode=mode)
     torch.set_default_dtype(torch.bfloat16)
     try:
         d = slime_amd.weight_dequant(q, s)
@@ -65,13 +73,13 @@ def test_block_quant_config1_roundtrip(cuda):
 def test_block_quant_tall_ragged(cuda):
     # [151937, 2560]: vocabulary-sized, 1-row remainder block row
     w = I.weights(151937, 2560, seed=5, outlier_p=0)
-    _check_block(w, w.to(cuda))
+    _check_block(w, w.to(cuda), mode=DEFAULT_MODE)
 
 
 @pytest.mark.parametrize("block", [(32, 32), (64, 128), (128, 64), (1, 128), (16, 48), (256, 256)])
 def test_block_quant_other_block_sizes(cuda, block):
     w = I.weights(200, 330, seed=2)
-    for mode in (0, 1):
+    for mode in (0, 1, 2):
         _check_block(w, w.to(cuda), block, mode)
 
 
@@ -81,7 +89,7 @@ def test_block_quant_strided_and_unaligned(cuda):
     views = [lambda t: t[:, 128:640], lambda t: t.t(), lambda t: t[::2, ::3], lambda t: t[100:357, 5:700],
              lambda t: t[:, 8:], lambda t: t[:, 1:769], lambda t: t[3:, :768]]
     for v in views:
-        for mode in (0, 1):
+        for mode in (0, 1, 2):
             _check_block(v(base), v(bg), mode=mode)
 
 
@@ -90,11 +98,24 @@ def test_block_quant_special_blocks(cuda):
               I.near_max_block(seed=4, amax=1.2e-38), torch.zeros(128, 128, dtype=torch.bfloat16),
               -torch.zeros(128, 128, dtype=torch.bfloat16)]
     w = torch.cat(blocks, dim=1)
-    for mode in (0, 1):
+    for mode in (0, 1, 2):
         q, s = _check_block(w, w.to(cuda), mode=mode)
     assert _bits32(s)[0, 4].item() != 0
-    q, s = slime_amd.block_fp8(w.to(cuda), (128, 128))
-    assert _bits32(s)[0, 4].item() == 0x27212492 and (_codes(q)[:, 640:] == 0x80).all()
+    # zero block: f32(bf16(1e-12)) / 448, and the same times RN(1/448)
+    for arith, bits in (("cpu", 0x27212492), ("device", _zero_block_scale_bits_device())):
+        with slime_amd.torch_arithmetic(arith):
+            q, s = slime_amd.block_fp8(w.to(cuda), (128, 128))
+        assert _bits32(s)[0, 4].item() == bits and (_codes(q)[:, 640:] == 0x80).all()
+
+
+def _zero_block_scale_bits_device():
+    from fractions import Fraction
+
+    from tests import exact_arith as X
+
+    floor_v = Fraction(0x8D | 0x80, 128) * Fraction(2) ** (0x57 - 127)      # bf16 bits 0x2B8D
+    v = X.rn_f32(floor_v * X.rn_f32(Fraction(1, 448)))
+    return torch.tensor(float(v), dtype=torch.float32).view(torch.int32).item()
 
 
 def test_block_quant_every_bf16_value(cuda):
@@ -107,7 +128,7 @@ def test_block_quant_every_bf16_value(cuda):
         x = vals[vals.abs() <= amax]
         x = torch.cat([x, torch.zeros((-x.numel()) % (128 * 128), dtype=torch.bfloat16)]).view(-1, 128)
         x[::128, 0] = amax
-        for mode in (0, 1):
+        for mode in (0, 1, 2):
             _check_block(x, x.to(cuda), mode=mode)
 
 
@@ -118,7 +139,7 @@ def test_block_quant_nan_inf(cuda):
     w[10, 131] = -float("inf")
     q, s = slime_amd.block_fp8(w.to(cuda), (128, 128))
     q, s = _codes(q), s.cpu()
-    qo, so = C.fp8_block_quant(w, (128, 128), 0)
+    qo, so = C.fp8_block_quant(w, (128, 128), DEFAULT_MODE)
     assert s[0, 0].isnan() and ((q[:, :128] & 0x7F) == 0x7F).all()
     assert s[0, 1].isinf()
     nan_o = (qo & 0x7F) == 0x7F
@@ -148,10 +169,12 @@ def test_channel_and_tensor_quant(cuda, shape):
     w[1] = 0
     for gpu_fn, ora, sshape in ((slime_amd.channel_fp8, C.fp8_channel_quant, (shape[0], 1)),
                                 (slime_amd.tensor_fp8, C.fp8_tensor_quant, (1,))):
-        q, s = gpu_fn(w.to(cuda))
-        qo, so = ora(w)
-        assert tuple(s.shape) == sshape
-        assert torch.equal(_codes(q), qo) and torch.equal(_bits32(s), _bits32(so))
+        for mode, arith in ARITH.items():
+            with slime_amd.torch_arithmetic(arith):
+                q, s = gpu_fn(w.to(cuda))
+            qo, so = ora(w, mode)
+            assert tuple(s.shape) == sshape
+            assert torch.equal(_codes(q), qo) and torch.equal(_bits32(s), _bits32(so))
     q, s = slime_amd.quant_fp8(w.to(cuda), "channel")
     assert tuple(s.shape) == (shape[0], 1)
     q, s = slime_amd.quant_fp8(w.to(cuda), "block", (128, 128))
@@ -213,7 +236,8 @@ def test_quant_plan_equals_single_calls(cuda):
     wg = [w.to(cuda) for w in ws]
     wg[2] = wg[2].t().contiguous().t()      # a strided member: generic path inside the grouped launch
     ws[2] = ws[2]
-    for mode in (0, 1):
+    assert slime_amd.Fp8QuantPlan(wg[:1], (128, 128)).mode == DEFAULT_MODE
+    for mode in (0, 1, 2):
         plan = slime_amd.Fp8QuantPlan(wg, (128, 128), mode)
         outs = plan.run()
         for w, (q, s) in zip(ws, outs):
@@ -245,7 +269,7 @@ def test_qwen3_4b_layer_all_linears(cuda):
     ws = {n: I.weights(*sh, seed=100 + i, outlier_p=0) for i, (n, sh) in enumerate(shapes.items())}
     outs = slime_amd.block_fp8_many([w.to(cuda) for w in ws.values()], (128, 128))
     for (n, w), (q, s) in zip(ws.items(), outs):
-        qo, so = C.fp8_block_quant(w, (128, 128), 0)
+        qo, so = C.fp8_block_quant(w, (128, 128), DEFAULT_MODE)
         assert torch.equal(_codes(q), qo) and torch.equal(_bits32(s), _bits32(so)), n
 
 
@@ -255,12 +279,54 @@ def test_golden_fixtures(cuda):
     f = load_file(os.path.join(GOLDEN, "fp8_golden.safetensors"))
     for case in sorted({k.split("/")[0] for k in f}):
         w = f[f"{case}/w"]
-        q, s = slime_amd.block_fp8(w.to(cuda), (128, 128))
-        assert torch.equal(_codes(q), f[f"{case}/q_block"].view(torch.uint8)), case
-        assert torch.equal(_bits32(s), _bits32(f[f"{case}/s_block"])), case
+        for arith, tag in (("cpu", "block"), ("device", "block_dev")):
+            with slime_amd.torch_arithmetic(arith):
+                q, s = slime_amd.block_fp8(w.to(cuda), (128, 128))
+            assert torch.equal(_codes(q), f[f"{case}/q_{tag}"].view(torch.uint8)), (case, arith)
+            assert torch.equal(_bits32(s), _bits32(f[f"{case}/s_{tag}"])), (case, arith)
         q, s = slime_amd.blockwise_cast_to_fp8_triton(w.to(cuda), (128, 128))
         assert torch.equal(_codes(q), f[f"{case}/q_cast"].view(torch.uint8)), case
         assert torch.equal(_bits32(s), _bits32(f[f"{case}/s_cast"])), case
         d = slime_amd.fp8._dequant(f[f"{case}/q_block"].to(cuda), f[f"{case}/s_block"].to(cuda), 128, 0,
                                    torch.bfloat16, "golden")
         assert I.same_bits(d.cpu(), f[f"{case}/deq"]), case
+
+
+# ------------------------------------------------------------------ torch's own GPU kernels as a second witness
+
+def test_torch_evaluates_scalar_division_as_reciprocal_multiply_on_gpu(cuda):
+    # the premise of the "device" arithmetic: for every finite positive bf16 amax, torch's GPU `t / 448` and
+    # `t / 7` are t * RN(1/448) and t * RN(1/7), and differ from the CPU results somewhere
+    t = torch.arange(0, 0x7F80, dtype=torch.int32).to(torch.int16).view(torch.bfloat16).float()
+    for d in (448.0, 7):
+        on_gpu = (t.to(cuda) / d).cpu()
+        inv = (torch.ones((), dtype=torch.float32) / d).item()
+        assert I.same_bits(on_gpu, t * inv)
+        assert not I.same_bits(on_gpu, t / d)
+
+
+def _every_value_blocks(n_amax, seed):
+    g = I.gen(seed)
+    vals = I.finite_bf16_values()
+    rows = []
+    for ab in torch.randint(0x0080, 0x7F80, (n_amax,), generator=g).tolist() + [0x2B8D, 0x7F7F, 0x0001]:
+        amax = torch.tensor([ab], dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+        x = vals[vals.abs() <= amax][: 128 * 128 * 3]
+        x = torch.cat([x, torch.zeros((-x.numel()) % (128 * 128), dtype=torch.bfloat16)]).view(-1, 128)
+        x[::128, 0] = amax
+        rows.append(x)
+    return torch.cat(rows, dim=0)
+
+
+def test_torch_ops_on_the_gpu_agree_with_the_kernels(cuda):
+    # the reference's own op sequence, executed by torch on the GPU, against the HIP kernels in "device" arithmetic
+    ws = [I.zero_blocks(I.weights(300, 200, seed=21), 0.2, seed=2), I.weights(1024, 2560, seed=22),
+          _every_value_blocks(12, seed=23)]
+    for w in ws:
+        wg = w.to(cuda)
+        for ref, mine in ((lambda x: T.block_fp8_ref(x, (128, 128)), lambda x: slime_amd.block_fp8(x, (128, 128))),
+                          (T.channel_fp8_ref, slime_amd.channel_fp8), (T.tensor_fp8_ref, slime_amd.tensor_fp8)):
+            qr, sr = ref(wg)
+            q, s = mine(wg)
+            assert torch.equal(_bits32(s), _bits32(sr))
+            assert torch.equal(_codes(q), _codes(qr))

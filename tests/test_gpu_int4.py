@@ -137,6 +137,11 @@ def test_int4_golden(cuda):
         assert I.same_bits(q.cpu(), f[f"{case}/q"]) and I.same_bits(s.cpu(), f[f"{case}/scale"]), case
         p, s2, _ = slime_amd.pack_layer(w, gs, True)
         assert torch.equal(p.cpu(), f[f"{case}/packed"]) and I.same_bits(s2.cpu(), f[f"{case}/pack_scale"]), case
+        d = slime_amd.dequantize_int4(p, s2, torch.tensor(list(w.shape)), gs)
+        assert I.same_bits(d.cpu(), f[f"{case}/deq"]), case
+        for arith, tag in (("cpu", "ste"), ("device", "ste_dev")):
+            with slime_amd.torch_arithmetic(arith):
+                assert I.same_bits(slime_amd.fake_int4_quantization_ste(w, gs).cpu(), f[f"{case}/{tag}"]), (case, arith)
         if f"{case}/packed_asym" in f:
             pa, _, pz = slime_amd.pack_layer(w, gs, False)
             assert torch.equal(pa.cpu(), f[f"{case}/packed_asym"]) and torch.equal(pz.cpu(), f[f"{case}/packed_zp"])
@@ -153,3 +158,121 @@ def test_pack_helpers_on_gpu(cuda):
     x = I.weights(8, 256, seed=1)
     sc = (x.float().abs().view(8, 2, 128).amax(-1) / 7).to(torch.bfloat16)
     assert torch.equal(slime_amd.quantize(x.to(cuda), sc.to(cuda), None).cpu(), T.quantize_ref(x, sc, None))
+
+
+# ------------------------------------------------------------------ INT4 -> bf16
+
+def _same_or_both_nan(a, b):
+    nan = b.isnan()
+    return torch.equal(a.isnan(), nan) and torch.equal(a[~nan].view(torch.int16), b[~nan].view(torch.int16))
+
+
+@pytest.mark.parametrize("shape,gs", [((768, 2048), 128), ((2048, 768), 128), ((16, 256), 128), ((33, 768), 128),
+                                      ((1, 128), 128), ((7, 7168), 128), ((24, 96), 32), ((333, 1024), 64),
+                                      ((5, 40), 8), ((3, 96), 48), ((1000, 2560), 128)])
+def test_int4_dequant(cuda, shape, gs):
+    g = I.gen(shape[0] + gs)
+    packed = torch.randint(-2 ** 31, 2 ** 31, (shape[0], shape[1] // 8), generator=g, dtype=torch.int64).to(torch.int32)
+    scale = (I.log_uniform_scales(shape[0], shape[1] // gs, seed=gs) * 0.1).to(torch.bfloat16)
+    got = slime_amd.dequantize_int4(packed.to(cuda), scale.to(cuda), shape, gs)
+    assert got.dtype == torch.bfloat16 and tuple(got.shape) == shape and got.is_contiguous()
+    assert I.same_bits(got.cpu(), C.int4_dequant(packed, scale, shape, gs))
+
+
+def test_int4_dequant_every_nibble_times_every_scale(cuda):
+    # 16 nibble values x all 65536 bf16 scale bit patterns (NaN scales: NaN-ness only)
+    scale = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16).view(-1, 1)
+    word = sum(((j * 2 + 1) % 16) << (4 * j) for j in range(8))          # nibbles 1,3,..,15
+    word2 = sum(((j * 2) % 16) << (4 * j) for j in range(8))              # nibbles 0,2,..,14
+    packed = torch.tensor([word, word2], dtype=torch.int64).to(torch.int32).repeat(65536, 1)
+    got = slime_amd.dequantize_int4(packed.to(cuda), scale.to(cuda), (65536, 16), 16).cpu()
+    assert _same_or_both_nan(got, C.int4_dequant(packed, scale, (65536, 16), 16))
+
+
+def test_int4_dequant_inverts_pack_layer(cuda):
+    w = I.weights(768, 2048, seed=12)
+    p, s, _ = slime_amd.pack_layer(w.to(cuda), 128, True)
+    d = slime_amd.dequantize_int4(p, s, (768, 2048), 128)
+    assert I.same_bits(d.cpu(), C.int4_dequant(*C.int4_pack_layer(w, 128, True)[:2], (768, 2048), 128))
+    # a second pack of the dequantised weight reproduces the words wherever the group's largest code was +-7
+    step = s.float().repeat_interleave(128, 1)
+    assert ((d.float() - w.to(cuda).float()).abs() <= step * (0.5 + 7 * 2.0 ** -8) + d.float().abs() * 2.0 ** -8).all()
+
+
+def test_int4_dequant_errors(cuda):
+    p = torch.zeros(4, 16, dtype=torch.int32, device=cuda)
+    s = torch.ones(4, 1, dtype=torch.bfloat16, device=cuda)
+    with pytest.raises(ValueError):
+        slime_amd.dequantize_int4(p, s, (4, 128), 100)
+    with pytest.raises(ValueError):
+        slime_amd.dequantize_int4(p, s, (4, 256), 128)
+    with pytest.raises(ValueError, match="incompatible"):
+        slime_amd.dequantize_int4(p, s.repeat(1, 2), (4, 128), 128)
+    with pytest.raises(RuntimeError):
+        slime_amd.dequantize_int4(p.cpu(), s.cpu(), (4, 128), 128)
+
+
+# ------------------------------------------------------------------ QAT straight-through forward
+
+ARITH = {0: "cpu", 1: "device"}
+
+
+@pytest.mark.parametrize("shape,gs", [((768, 2048), 128), ((16, 256), 128), ((33, 768), 128), ((1, 128), 128),
+                                      ((7, 7168), 128), ((24, 96), 32), ((333, 1024), 64), ((1000, 2560), 128)])
+def test_fake_ste_forward(cuda, shape, gs):
+    w = I.weights(*shape, seed=shape[1] + gs, outlier_p=0.01)
+    w[0, :gs] = 0
+    for div7, arith in ARITH.items():
+        with slime_amd.torch_arithmetic(arith):
+            y = slime_amd.fake_int4_quantization_ste(w.to(cuda), gs)
+        assert y.dtype == torch.bfloat16 and y.shape == w.shape
+        assert I.same_bits(y.cpu(), C.int4_fake_ste(w, gs, div7)), arith
+
+
+def test_fake_ste_special_values_and_every_bf16_value(cuda):
+    rows = [I.subnormal_block(4, 1024, seed=1), I.near_max_block(4, 1024, seed=2, amax=7e-5),
+            I.near_max_block(4, 1024, seed=3, amax=3.0e38), torch.zeros(4, 1024, dtype=torch.bfloat16),
+            -torch.zeros(4, 1024, dtype=torch.bfloat16), I.weights(4, 1024, seed=4, std=1e-6)]
+    vals = I.finite_bf16_values()
+    g = I.gen(3)
+    for ab in torch.randint(1, 0x7F80, (12,), generator=g).tolist() + [0x3728, 0x3727, 0x7F7F]:
+        amax = torch.tensor([ab], dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+        x = vals[vals.abs() <= amax]
+        x = torch.cat([x, torch.zeros((-x.numel()) % 1024, dtype=torch.bfloat16)]).view(-1, 128)
+        x[:, 0] = amax
+        rows.append(x.reshape(-1, 1024))
+    w = torch.cat(rows)
+    nan_row = I.weights(2, 1024, seed=9)
+    nan_row[0, 5] = float("nan")
+    nan_row[1, 300] = float("inf")
+    w = torch.cat([w, nan_row])
+    for div7, arith in ARITH.items():
+        with slime_amd.torch_arithmetic(arith):
+            y = slime_amd.fake_int4_quantization_ste(w.to(cuda), 128).cpu()
+        assert _same_or_both_nan(y, C.int4_fake_ste(w, 128, div7)), arith
+
+
+def test_fake_ste_matches_torch_ops_on_the_gpu(cuda):
+    # the reference's own op sequence executed by torch on the GPU, against the kernel ("device" arithmetic)
+    from oracle import torch_ref as T
+
+    for shape, gs in (((512, 2048), 128), ((64, 96), 32), ((100, 1024), 64)):
+        w = I.weights(*shape, seed=shape[0], outlier_p=0.01).to(cuda)
+        assert I.same_bits(slime_amd.fake_int4_quantization_ste(w, gs).cpu(), T.fake_int4_ste_ref(w, gs).cpu())
+
+
+def test_fake_ste_ragged_and_gradient(cuda):
+    from oracle import torch_ref as T
+
+    w = I.weights(6, 100, seed=3)
+    for div7, arith in ARITH.items():
+        with slime_amd.torch_arithmetic(arith):
+            y = slime_amd.fake_int4_quantization_ste(w.to(cuda), 64)          # N % group != 0: zero-padded groups
+        assert I.same_bits(y.cpu(), T.fake_int4_ste_ref(w, 64, device_arith=bool(div7))), arith
+    x = I.weights(16, 256, seed=4).to(cuda).requires_grad_(True)
+    x.main_grad = torch.zeros(16, 256, device=cuda)
+    y = slime_amd.fake_int4_quantization_ste(x, 128)
+    assert y.main_grad is x.main_grad
+    gy = torch.randn(16, 256, device=cuda).to(torch.bfloat16)
+    y.backward(gy)
+    assert torch.equal(x.grad, gy)                                            # straight-through: identity

@@ -30,7 +30,7 @@ def test_fp8_qkv_params(cuda):
     out = slime_amd.quantize_params(None, L + "mlp.linear_fc2.weight", [("model.layers.0.mlp.down_proj.weight",
                                                                          ws["k_proj"].to(cuda))], cfg2)
     assert [n for n, _ in out] == ["model.layers.0.mlp.down_proj.weight", "model.layers.0.mlp.down_proj.weight_scale"]
-    qo, so = C.fp8_tensor_quant(ws["k_proj"])
+    qo, so = C.fp8_tensor_quant(ws["k_proj"], 2)
     assert torch.equal(out[0][1].cpu().view(torch.uint8), qo) and I.same_bits(out[1][1].cpu(), so)
     # untouched parameter: same list object comes back
     p = [("model.embed_tokens.weight", ws["k_proj"].to(cuda))]

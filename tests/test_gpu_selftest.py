@@ -21,7 +21,7 @@ def _run(fn, *args):
     return count, first & 0xFFFFFFFFFFFFFFFF
 
 
-@pytest.mark.parametrize("mode", [0, 1])
+@pytest.mark.parametrize("mode", [0, 1, 2])
 def test_fp8_element_function_whole_domain(cuda, mode):
     # every finite bf16 amax x every bf16 x with |x| <= amax: 2^31 pairs
     count, first = _run(_lib.load().wq_selftest_fp8_elem, 0, 0x7F80, mode)

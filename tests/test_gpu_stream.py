@@ -17,7 +17,7 @@ def test_stream_fp8_ragged_buckets(cuda):
                           max(w.numel() for w in ws), 2, depth=2)
     n = 0
     for w, (q, s) in zip(ws, pipe.process(iter(ws))):
-        qo, so = C.fp8_block_quant(w, (128, 128), 0)
+        qo, so = C.fp8_block_quant(w, (128, 128), 2)
         assert q.device.type == "cpu" and torch.equal(q.view(torch.uint8), qo)
         assert torch.equal(s.view(torch.int32), so.view(torch.int32))
         n += 1

@@ -67,7 +67,7 @@ def test_convert_hf_to_fp8_block_and_cast_back(ckpt, tmp_path, cuda):
     assert len(converted) == 4
     for k, w in tensors.items():
         if k in converted:
-            qo, so = C.fp8_block_quant(w, (128, 128), 0)
+            qo, so = C.fp8_block_quant(w, (128, 128), 2)
             assert got[k].dtype == torch.float8_e4m3fn and torch.equal(got[k].view(torch.uint8), qo), k
             s = got[k.replace(".weight", ".weight_scale_inv")]
             assert s.dtype == torch.float32 and torch.equal(s.view(torch.int32), so.view(torch.int32)), k
@@ -103,7 +103,7 @@ def test_convert_hf_to_fp8_other_strategies(ckpt, tmp_path, cuda, strategy):
     for f in ("model-00001-of-00002.safetensors", "model-00002-of-00002.safetensors"):
         got.update(load_file(str(out / f)))
     k = "model.layers.0.mlp.experts.0.gate_proj.weight"
-    qo, so = (C.fp8_tensor_quant if strategy == "tensor" else C.fp8_channel_quant)(tensors[k])
+    qo, so = (C.fp8_tensor_quant if strategy == "tensor" else C.fp8_channel_quant)(tensors[k], 2)
     assert torch.equal(got[k].view(torch.uint8), qo)
     s = got[k.replace(".weight", ".weight_scale")]
     assert s.shape == so.shape and torch.equal(s.view(torch.int32), so.view(torch.int32))

@@ -116,6 +116,23 @@ def test_modes_differ_where_they_should():
     assert ((q0[d].int() - q1[d].int()).abs() == 1).all()
 
 
+def test_device_arithmetic_scale_is_a_reciprocal_multiply_for_every_amax():
+    # mode 2 over all finite bf16 amax values: scale == RN(max(amax, floor) * RN(1/448)) in exact arithmetic, and
+    # it differs from the quotient of mode 0 for a large share of them (a mode 2 that divides would pass nothing)
+    bits = torch.arange(1, 0x7F80, 37, dtype=torch.int32)
+    w = torch.zeros(bits.numel(), 4, dtype=torch.bfloat16)
+    w[:, 1] = bits.to(torch.int16).view(torch.bfloat16)
+    _, s2 = C.fp8_block_quant(w, (1, 4), 2)
+    _, s0 = C.fp8_block_quant(w, (1, 4), 0)
+    inv = rn_f32(Fraction(1, 448))
+    n_diff = 0
+    for a, got2, got0 in zip(w[:, 1].float().tolist(), s2[:, 0].tolist(), s0[:, 0].tolist()):
+        a = max(Fraction(a), BF16_1EM12)
+        assert Fraction(got2) == rn_f32(a * inv) and Fraction(got0) == rn_f32(a / 448)
+        n_diff += got2 != got0
+    assert n_diff > bits.numel() // 4
+
+
 # ------------------------------------------------------------------ exact rational arithmetic, tiny blocks
 
 def _exact_block_quant(w, bm, bn, mode):
@@ -131,18 +148,20 @@ def _exact_block_quant(w, bm, bn, mode):
             amax = max(abs(vals[i][j]) for i, j in cells)
             if mode == 0:
                 scale = rn_f32(max(amax, BF16_1EM12) / 448)
+            elif mode == 2:     # torch's GPU evaluation of `/ 448`: multiply by RN(1/448)
+                scale = rn_f32(max(amax, BF16_1EM12) * rn_f32(Fraction(1, 448)))
             else:
                 scale = rn_f32(max(amax, F32_1EM10) / 448)
                 inv = rn_f32(1 / scale)
             scales[bi][bj] = scale
             for i, j in cells:
-                q = rn_f32(vals[i][j] / scale) if mode == 0 else rn_f32(vals[i][j] * inv)
+                q = rn_f32(vals[i][j] / scale) if mode != 1 else rn_f32(vals[i][j] * inv)
                 q = min(max(q, Fraction(-448)), Fraction(448))
                 codes[i][j] = e4m3_code(rn_e4m3(q), negative_zero=(vals[i][j] < 0 or neg0[i][j]))
     return codes, scales
 
 
-@pytest.mark.parametrize("mode", [0, 1])
+@pytest.mark.parametrize("mode", [0, 1, 2])
 def test_block_quant_matches_exact_arithmetic(mode):
     w = I.weights(10, 14, seed=11, std=0.05, outlier_p=0.05)
     w[0, 0] = -0.0
@@ -160,11 +179,14 @@ SHAPES = [(128, 128), (256, 384), (300, 200), (7, 7168), (1, 1), (129, 127), (41
 
 
 @pytest.mark.parametrize("shape", SHAPES)
-@pytest.mark.parametrize("mode", [0, 1])
+@pytest.mark.parametrize("mode", [0, 1, 2])
 def test_c_equals_torch_block_quant(shape, mode):
     w = I.zero_blocks(I.weights(*shape, seed=sum(shape)), 0.2, seed=1)
     q, s = C.fp8_block_quant(w, (128, 128), mode)
-    qr, sr = (T.block_fp8_ref if mode == 0 else T.blockwise_cast_ref)(w, (128, 128))
+    if mode == 1:
+        qr, sr = T.blockwise_cast_ref(w, (128, 128))
+    else:
+        qr, sr = T.block_fp8_ref(w, (128, 128), device_arith=(mode == 2))
     assert torch.equal(q, _codes(qr))
     assert torch.equal(_bits32(s), _bits32(sr))
 
@@ -236,12 +258,13 @@ def test_nan_and_inf_blocks():
 def test_c_equals_torch_channel_and_tensor(shape):
     w = I.weights(*shape, seed=8)
     w[1] = 0
-    q, s = C.fp8_channel_quant(w)
-    qr, sr = T.channel_fp8_ref(w)
-    assert torch.equal(q, _codes(qr)) and torch.equal(_bits32(s), _bits32(sr)) and s.shape == sr.shape
-    q, s = C.fp8_tensor_quant(w)
-    qr, sr = T.tensor_fp8_ref(w)
-    assert torch.equal(q, _codes(qr)) and torch.equal(_bits32(s), _bits32(sr)) and s.shape == sr.shape
+    for mode in (0, 2):
+        q, s = C.fp8_channel_quant(w, mode)
+        qr, sr = T.channel_fp8_ref(w, device_arith=(mode == 2))
+        assert torch.equal(q, _codes(qr)) and torch.equal(_bits32(s), _bits32(sr)) and s.shape == sr.shape
+        q, s = C.fp8_tensor_quant(w, mode)
+        qr, sr = T.tensor_fp8_ref(w, device_arith=(mode == 2))
+        assert torch.equal(q, _codes(qr)) and torch.equal(_bits32(s), _bits32(sr)) and s.shape == sr.shape
 
 
 # ------------------------------------------------------------------ dequant
