@@ -146,6 +146,54 @@ def bench_int4_pack(dev, steps, warmup, layers):
     return out
 
 
+def bench_int4_inverse(dev, steps, warmup, layers, which):
+    """INT4 -> bf16 (`which == "int4deq"`) or the QAT quantise-dequantise forward (`"ste"`) over the expert weights
+    of `layers` Qwen3-30B-A3B layers; the 128 experts of a projection are one [128*rows, cols] tensor, one launch
+    each (no grouped form exists for these two)."""
+    import torch
+
+    import slime_amd
+    from oracle import c_oracle
+
+    tensors = []
+    for _ in range(layers):
+        for rows, cols in ((128 * 768, 2048), (128 * 768, 2048), (128 * 2048, 768)):
+            w = _gen_bf16((rows, cols), dev, outliers=True)
+            if which == "int4deq":
+                p, sc, _ = slime_amd.pack_layer(w, 128, True)
+                tensors.append((p, sc, (rows, cols)))
+                del w
+            else:
+                tensors.append(w)
+    outs = [None] * len(tensors)
+
+    def run():
+        for i, t in enumerate(tensors):
+            outs[i] = None          # free the previous output first: the allocator reuses the block
+            outs[i] = (slime_amd.dequantize_int4(t[0], t[1], t[2], 128) if which == "int4deq"
+                       else slime_amd.fake_int4_quantization_ste(t, 128))
+
+    wall_ms, ev_ms, ev_min = _time_launches(run, steps, warmup)
+    elements = sum((t[2][0] * t[2][1]) if which == "int4deq" else t.numel() for t in tensors)
+    algo_bytes = elements * 2 + elements // 2 + elements // 128 * 2 if which == "int4deq" else elements * 4
+    for idx in (0, len(tensors) - 1):
+        if which == "int4deq":
+            p, sc, shape = tensors[idx]
+            want = c_oracle.int4_dequant(p[:1024].cpu(), sc[:1024].cpu(), (1024, shape[1]), 128)
+        else:
+            want = c_oracle.int4_fake_ste(tensors[idx][:1024].cpu(), 128, 1)
+        assert torch.equal(outs[idx][:1024].cpu().view(torch.int16), want.view(torch.int16))
+    out = {"workload": f"Qwen3-30B-A3B experts, {layers} layers x (gate, up [128x768,2048], down [128x2048,768]), "
+                       + ("INT4 group 128 -> bf16" if which == "int4deq" else "INT4 QAT quantise-dequantise forward")
+                       + f", {len(tensors)} launches per step",
+           "launches": len(tensors), "bf16_GB": 2 * elements / 1e9, "kernel_ms": ev_ms, "wall_ms": wall_ms,
+           "bf16_GBps": 2 * elements / ev_ms / 1e6, "algo_GBps": algo_bytes / ev_ms / 1e6,
+           "hbm_frac": algo_bytes / ev_ms / 1e6 / HBM_PEAK_GBS, "parity_tensors_checked": 2}
+    del tensors, outs
+    torch.cuda.empty_cache()
+    return out
+
+
 def bench_fp8_dequant(dev, steps, warmup, experts):
     import torch
 
@@ -270,7 +318,7 @@ def main():
     ap.add_argument("--dequant-experts", type=int, default=256)
     ap.add_argument("--no-extras", action="store_true", help="headline workload only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
-    ap.add_argument("--only", choices=["int4", "dequant", "copy", "stream"], default=None,
+    ap.add_argument("--only", choices=["int4", "dequant", "int4deq", "ste", "copy", "stream"], default=None,
                     help="run just one of the other legs and print its record: a kernel for profiling, the plain copy "
                          "kernel that hardware counters are calibrated against, or the host-resident streaming run "
                          "(64 x 1 GiB buckets, PCIe-bound)")
@@ -296,6 +344,9 @@ def main():
         return
     if args.only == "dequant":
         print(json.dumps(bench_fp8_dequant(dev, args.steps, args.warmup, args.dequant_experts)))
+        return
+    if args.only in ("int4deq", "ste"):
+        print(json.dumps(bench_int4_inverse(dev, args.steps, args.warmup, min(args.int4_layers, 8), args.only)))
         return
     if args.only == "copy":
         print(json.dumps(bench_copy(dev, args.steps, args.warmup)))
@@ -337,6 +388,9 @@ def main():
             extras["int4_group_quant_pack"] = bench_int4_pack(dev, args.steps, args.warmup, args.int4_layers)
         if args.dequant_experts > 0:
             extras["fp8_block_dequant"] = bench_fp8_dequant(dev, args.steps, args.warmup, args.dequant_experts)
+        if args.int4_layers > 0:
+            extras["int4_dequant"] = bench_int4_inverse(dev, args.steps, args.warmup, min(args.int4_layers, 8), "int4deq")
+            extras["int4_qat_forward"] = bench_int4_inverse(dev, args.steps, args.warmup, min(args.int4_layers, 8), "ste")
         line["other_workloads"] = extras
     print(json.dumps(line))
 
