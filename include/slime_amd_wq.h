@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define WQ_ABI_VERSION 2
+#define WQ_ABI_VERSION 3
 
 enum {
     WQ_OK = 0,
@@ -174,6 +174,48 @@ int wq_int4_dequant(const int32_t *packed, const void *scale, void *y, int64_t M
  * (amax * RN(1/7), which is also what fake_int4_quant_cuda.cu:59 computes); x / s is an IEEE division in both. */
 enum { WQ_DIV7_IEEE = 0, WQ_DIV7_DEVICE = 1 };
 int wq_int4_fake_quant_ste(const void *x, void *y, int64_t M, int64_t N, int group, int div7, void *stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Byte-level delta of a tensor against its snapshot (delta weight sync).
+ *
+ * wq_delta_xor replaces, for one tensor, the xor branch of diff_and_compress in
+ * UpdateWeightFromDiskDelta._encode_delta, slime/backends/megatron_utils/update_weight/
+ * update_weight_from_disk_delta.py:224-246 - `diff = new ^ old; changed = count_nonzero(diff)`, the snapshot
+ * update `snapshot[name] = new` - and checksum("adler32", new), slime/utils/disk_delta.py:28-58, in one pass:
+ *   diff[i] = new[i] ^ old[i]            (skipped when diff == NULL)
+ *   old[i]  = new[i]                     (when update_old != 0)
+ *   result[0] = number of bytes with new[i] != old[i];  result[1] = zlib-compatible adler32 of new[0..n)
+ * All buffers are DEVICE memory; new/old/diff 16-byte aligned, n in bytes (any value >= 0).  `workspace` is
+ * device scratch of wq_delta_workspace_bytes(n) bytes (8-byte aligned) that needs no initialisation and, after
+ * the call, holds the per-chunk counts wq_delta_overwrite_encode consumes.  `result` is 2 x uint64, device.
+ *
+ * wq_delta_overwrite_encode replaces overwrite_encode(new, new != old), slime/utils/disk_delta.py:21-25:
+ *   out = [count u32 LE][positions u32 LE x count, ascending][new[position] x count]
+ * Call wq_delta_xor first on the same (new, old, n, workspace) with update_old == 0, read back
+ * count = result[0], size `out` to 4 + 5 * count bytes (4-byte aligned), then call this.  n <= 2^32 - 1. */
+#define WQ_DELTA_CHUNK 16384
+int64_t wq_delta_workspace_bytes(int64_t n);
+int wq_delta_xor(const void *new_bytes, void *old_bytes, void *diff, int64_t n, int update_old,
+                 void *workspace, uint64_t *result, void *stream);
+int wq_delta_overwrite_encode(const void *new_bytes, const void *old_bytes, int64_t n, void *workspace,
+                              uint32_t count, void *out, void *stream);
+
+/* wq_delta_xor over a bucket of tensors with two launches in total (the shape a weight-sync bucket wants:
+ * update_weight_from_disk_delta.py:252-270 walks the gathered tensors one by one).  `descs` is a DEVICE array
+ * whose fields mean what the arguments of wq_delta_xor mean (a tensor with n == 0 is allowed); `chunk_start`
+ * is a DEVICE int64[n_desc+1] exclusive prefix sum of ceil(n / WQ_DELTA_CHUNK); total_chunks = chunk_start[n_desc].
+ * With write_diff == 0 the `diff` fields are ignored.  The entry point cannot check alignment of the pointers
+ * inside `descs`: the caller guarantees what wq_delta_xor checks. */
+typedef struct wq_delta_desc {
+    const void *new_bytes;
+    void *old_bytes;
+    void *diff;
+    int64_t n;
+    void *workspace;     /* wq_delta_workspace_bytes(n) bytes */
+    uint64_t *result;    /* 2 x uint64 */
+} wq_delta_desc;
+int wq_delta_xor_grouped(const wq_delta_desc *descs, const int64_t *chunk_start, int n_desc,
+                         int64_t total_chunks, int write_diff, int update_old, void *stream);
 
 /* ---------------------------------------------------------------------------------------------
  * Self-checks and calibration helpers (used by the test-suite and the benchmark, not by callers).

@@ -15,7 +15,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libslime_amd_wq.so")
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 # selectors (mirrors of the header's enums)
 DTYPE_BF16, DTYPE_F32 = 0, 1
@@ -42,6 +42,10 @@ SIGNATURES = {
     "wq_int4_group_quant_pack_grouped": [_vp, _vp, _int, _i64, _int, _vp],
     "wq_int4_dequant": [_vp, _vp, _vp, _i64, _i64, _int, _vp],
     "wq_int4_fake_quant_ste": [_vp, _vp, _i64, _i64, _int, _int, _vp],
+    "wq_delta_workspace_bytes": [_i64],
+    "wq_delta_xor": [_vp, _vp, _vp, _i64, _int, _vp, _vp, _vp],
+    "wq_delta_overwrite_encode": [_vp, _vp, _i64, _vp, ctypes.c_uint32, _vp, _vp],
+    "wq_delta_xor_grouped": [_vp, _vp, _int, _i64, _int, _int, _vp],
     "wq_selftest_fp8_elem": [_u32, _u32, _int, _vp, _vp],
     "wq_selftest_int4_elem": [_u32, _u32, _vp, _vp],
     "wq_selftest_cvt_fp8": [_u64, _u64, _vp, _vp],
@@ -77,7 +81,8 @@ def load() -> ctypes.CDLL:
             except AttributeError as exc:
                 raise WqLibraryError(f"{LIB_PATH} does not export {name}; rebuild the library") from exc
             fn.argtypes = argtypes
-            fn.restype = ctypes.c_char_p if name == "wq_error_string" else _int
+            fn.restype = (ctypes.c_char_p if name == "wq_error_string"
+                          else _i64 if name == "wq_delta_workspace_bytes" else _int)
         if lib.wq_abi_version() != ABI_VERSION:
             raise WqLibraryError(f"ABI mismatch: library {lib.wq_abi_version()}, binding {ABI_VERSION}; rebuild")
         _lib = lib

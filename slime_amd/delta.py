@@ -1,0 +1,215 @@
+"""Byte-level delta of weights against a snapshot kept in HBM (delta weight sync), on MI355X.
+
+The reference diffs every gathered HF tensor against a CPU snapshot with numpy in a thread pool
+(``UpdateWeightFromDiskDelta._encode_delta``, slime/backends/megatron_utils/update_weight/
+update_weight_from_disk_delta.py:198-274; helpers in slime/utils/disk_delta.py:21-58).  Here the snapshot
+lives in device memory - 288 GB of HBM hold a full model next to the live weights - and one kernel pass per
+tensor yields the xor diff, the changed-byte count, the adler32 of the new bytes and the updated snapshot;
+only the diff of a tensor that did change has to cross PCIe for compression.
+
+``xor_diff`` / ``overwrite_encode`` / ``checksum`` are the per-tensor operations, ``DeltaEncoder`` the
+snapshot-keeping loop body (``diff_and_compress`` + ``collect`` without the zstd step, which stays on the
+host).  Only the ``adler32`` checksum is computed on the GPU: xxh3-128 and blake3 are sequential by design.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+
+CHUNK = 16384        # WQ_DELTA_CHUNK: bytes of a tensor one workgroup handles
+
+
+def _as_bytes(t: torch.Tensor, what: str) -> torch.Tensor:
+    _lib.require_gpu(t, what)
+    flat = t.detach().contiguous().view(torch.uint8).reshape(-1)
+    if flat.data_ptr() % 16:
+        flat = flat.clone()
+    return flat
+
+
+def _workspace(n: int, device) -> torch.Tensor:
+    return torch.empty(_lib.load().wq_delta_workspace_bytes(n) // 8, dtype=torch.int64, device=device)
+
+
+def _xor_pass(new: torch.Tensor, old: torch.Tensor, diff, update_old: bool, workspace, result) -> None:
+    with torch.cuda.device(new.device):
+        rc = _lib.load().wq_delta_xor(new.data_ptr(), old.data_ptr(), diff.data_ptr() if diff is not None else None,
+                                      new.numel(), int(update_old), workspace.data_ptr(), result.data_ptr(),
+                                      _lib.stream_ptr(new.device))
+    _lib.check(rc, "delta xor pass")
+
+
+def xor_diff(new: torch.Tensor, old: torch.Tensor, update_snapshot: bool = False):
+    """-> (diff uint8 [nbytes] = new ^ old, result int64 [2] on the device = [changed bytes, adler32(new)]).
+
+    ``old`` must be a contiguous uint8 tensor of the same byte size; with ``update_snapshot`` it is overwritten
+    with the new bytes in the same pass.  Nothing synchronises: read ``result`` when the values are needed."""
+    nw = _as_bytes(new, "xor_diff")
+    _check_old(nw, old)
+    diff = torch.empty_like(nw)
+    result = torch.empty(2, dtype=torch.int64, device=nw.device)
+    _xor_pass(nw, old, diff, update_snapshot, _workspace(nw.numel(), nw.device), result)
+    return diff, result
+
+
+def _align(n: int, a: int = 256) -> int:
+    return (n + a - 1) // a * a
+
+
+def xor_diff_many(news, olds, update_snapshot: bool = False, want_diff: bool = True):
+    """``xor_diff`` over a bucket of tensors with two kernel launches in total.
+
+    -> (diffs: list of uint8 views into one flat buffer, or None without ``want_diff``;
+        results: int64 [len(news), 2] on the device = [changed bytes, adler32(new)] per tensor)."""
+    if len(news) != len(olds):
+        raise ValueError("xor_diff_many: need one snapshot per tensor")
+    if not news:
+        return ([] if want_diff else None), torch.empty((0, 2), dtype=torch.int64)
+    flat = [_as_bytes(t, "xor_diff_many") for t in news]
+    device = flat[0].device
+    lib = _lib.load()
+    d_off, w_off, d_total, w_total = [], [], 0, 0
+    for nw, old in zip(flat, olds):
+        _check_old(nw, old)
+        d_off.append(d_total)
+        w_off.append(w_total)
+        d_total += _align(nw.numel())
+        w_total += _align(lib.wq_delta_workspace_bytes(nw.numel()))
+    flat_diff = torch.empty(max(d_total, 1), dtype=torch.uint8, device=device) if want_diff else None
+    flat_ws = torch.empty(w_total // 8, dtype=torch.int64, device=device)
+    results = torch.empty((len(flat), 2), dtype=torch.int64, device=device)
+    rows, starts, chunks = [], [0], 0
+    for i, (nw, old) in enumerate(zip(flat, olds)):
+        n = nw.numel()
+        rows.append([nw.data_ptr(), old.data_ptr(), flat_diff.data_ptr() + d_off[i] if want_diff else 0, n,
+                     flat_ws.data_ptr() + w_off[i], results.data_ptr() + 16 * i])
+        chunks += -(-n // CHUNK)
+        starts.append(chunks)
+    descs = torch.tensor(rows, dtype=torch.int64).to(device)
+    start_t = torch.tensor(starts, dtype=torch.int64).to(device)
+    with torch.cuda.device(device):
+        rc = lib.wq_delta_xor_grouped(descs.data_ptr(), start_t.data_ptr(), len(flat), chunks, int(want_diff),
+                                      int(update_snapshot), _lib.stream_ptr(device))
+    _lib.check(rc, "xor_diff_many")
+    diffs = [flat_diff[o:o + nw.numel()] for o, nw in zip(d_off, flat)] if want_diff else None
+    return diffs, results
+
+
+def _check_old(nw: torch.Tensor, old: torch.Tensor) -> None:
+    if old.dtype != torch.uint8 or old.dim() != 1 or not old.is_contiguous() or old.numel() != nw.numel():
+        raise ValueError(f"snapshot must be a contiguous uint8 vector of {nw.numel()} bytes, got "
+                         f"{tuple(old.shape)} {old.dtype}")
+    if old.device != nw.device or old.data_ptr() % 16:
+        raise ValueError("snapshot must live on the tensor's device at a 16-byte aligned address")
+
+
+def overwrite_encode(new: torch.Tensor, old: torch.Tensor) -> torch.Tensor:
+    """The 'overwrite' delta of slime/utils/disk_delta.py:21-25 for ``changed_mask = new != old``:
+    uint8 vector [count u32 LE][positions u32 LE x count][new values x count].  Synchronises once (the output
+    size depends on the count)."""
+    nw = _as_bytes(new, "overwrite_encode")
+    _check_old(nw, old)
+    if nw.numel() > 0xFFFFFFFF:
+        raise ValueError("overwrite_encode: positions are uint32; tensor too large")
+    ws = _workspace(nw.numel(), nw.device)
+    result = torch.empty(2, dtype=torch.int64, device=nw.device)
+    _xor_pass(nw, old, None, False, ws, result)
+    count = int(result[0].item())
+    out = torch.empty(4 + 5 * count, dtype=torch.uint8, device=nw.device)
+    with torch.cuda.device(nw.device):
+        rc = _lib.load().wq_delta_overwrite_encode(nw.data_ptr(), old.data_ptr(), nw.numel(), ws.data_ptr(), count,
+                                                   out.data_ptr(), _lib.stream_ptr(nw.device))
+    _lib.check(rc, "overwrite_encode")
+    return out
+
+
+def checksum(algorithm: str, buf: torch.Tensor) -> str:
+    """``checksum("adler32", tensor)`` of slime/utils/disk_delta.py:55-58 on the GPU -> 8 hex digits.
+    Other algorithms raise KeyError, as the reference does for unknown names: they are host-side digests."""
+    if algorithm != "adler32":
+        raise KeyError(f"checksum algorithm {algorithm!r} is not computed on the GPU (adler32 only)")
+    nw = _as_bytes(buf, "checksum")
+    result = torch.empty(2, dtype=torch.int64, device=nw.device)
+    _xor_pass(nw, nw, None, False, _workspace(nw.numel(), nw.device), result)
+    return f"{int(result[1].item()):08x}"
+
+
+class DeltaEncoder:
+    """Snapshot in HBM + the per-tensor body of ``_encode_delta``.
+
+    ``capture(name, tensor)`` seeds the snapshot (``_capture_baseline``, update_weight_from_disk_delta.py:96-128).
+    ``encode(name, tensor)`` returns ``(diff_or_None, checksum_or_None, changed)`` like ``diff_and_compress`` minus
+    compression: ``diff`` is the xor bytes or the overwrite encoding (device uint8 tensor), ``None`` when nothing
+    changed; the snapshot is updated either way (``collect``: ``snapshot[name] = new``).  ``changed_bytes`` /
+    ``total_bytes`` accumulate as in the reference."""
+
+    def __init__(self, delta_encoding: str = "xor", checksum_algorithm: str = "adler32"):
+        if delta_encoding not in ("xor", "overwrite"):
+            raise ValueError(f"unknown delta encoding {delta_encoding!r}")
+        self.delta_encoding = delta_encoding
+        self.checksum_algorithm = checksum_algorithm
+        self.snapshot: dict[str, torch.Tensor] = {}
+        self.changed_bytes = self.total_bytes = 0
+
+    def capture(self, name: str, tensor: torch.Tensor) -> None:
+        self.snapshot[name] = _as_bytes(tensor, "DeltaEncoder.capture").clone()
+
+    def encode_bucket(self, named_tensors):
+        """``encode`` for a list of (name, tensor) with two kernel launches and one synchronisation (xor encoding
+        only).  -> list of (name, diff_or_None, checksum_or_None, changed) in input order."""
+        if self.delta_encoding != "xor":
+            return [(name,) + self.encode(name, t) for name, t in named_tensors]
+        named_tensors = list(named_tensors)
+        diffs, results = xor_diff_many([t for _, t in named_tensors], [self.snapshot[n] for n, _ in named_tensors],
+                                       update_snapshot=True)
+        out = []
+        for (name, t), diff, (changed, adler) in zip(named_tensors, diffs, results.tolist()):
+            self.total_bytes += diff.numel()
+            if not changed:
+                out.append((name, None, None, 0))
+                continue
+            self.changed_bytes += changed
+            if self.checksum_algorithm == "adler32":
+                digest = f"{adler:08x}"
+            else:
+                from .delta_host import host_checksum
+
+                digest = host_checksum(self.checksum_algorithm, t)
+            out.append((name, diff, digest, changed))
+        return out
+
+    def encode(self, name: str, tensor: torch.Tensor):
+        nw = _as_bytes(tensor, "DeltaEncoder.encode")
+        old = self.snapshot[name]
+        _check_old(nw, old)
+        n = nw.numel()
+        self.total_bytes += n
+        ws = _workspace(n, nw.device)
+        result = torch.empty(2, dtype=torch.int64, device=nw.device)
+        if self.delta_encoding == "xor":
+            diff = torch.empty_like(nw)
+            _xor_pass(nw, old, diff, True, ws, result)
+            changed, adler = (int(v) for v in result.tolist())
+        else:
+            _xor_pass(nw, old, None, False, ws, result)
+            changed, adler = (int(v) for v in result.tolist())
+            diff = None
+            if changed:
+                diff = torch.empty(4 + 5 * changed, dtype=torch.uint8, device=nw.device)
+                with torch.cuda.device(nw.device):
+                    rc = _lib.load().wq_delta_overwrite_encode(nw.data_ptr(), old.data_ptr(), n, ws.data_ptr(), changed,
+                                                               diff.data_ptr(), _lib.stream_ptr(nw.device))
+                _lib.check(rc, "DeltaEncoder.encode")
+            old.copy_(nw)
+        if not changed:
+            return None, None, 0
+        self.changed_bytes += changed
+        if self.checksum_algorithm == "adler32":
+            digest = f"{adler:08x}"
+        else:
+            from .delta_host import host_checksum
+
+            digest = host_checksum(self.checksum_algorithm, nw)
+        return diff, digest, changed

@@ -1,0 +1,48 @@
+"""Pins the delta part of the oracle: the numpy restatement against closed forms, an independent bytewise
+adler32, and the apply round trip."""
+
+import zlib
+
+import numpy as np
+
+from oracle import delta_ref as D
+
+
+def _pair(n, density, seed):
+    rng = np.random.default_rng(seed)
+    old = rng.integers(0, 256, n, dtype=np.uint8)
+    new = old.copy()
+    idx = rng.random(n) < density
+    new[idx] = rng.integers(0, 256, int(idx.sum()), dtype=np.uint8)     # some draws equal the old byte: unchanged
+    return new, old
+
+
+def test_adler32_known_answers_and_bytewise_witness():
+    assert D.adler32_ref(np.zeros(0, np.uint8)) == "00000001"
+    assert D.adler32_ref(np.frombuffer(b"Wikipedia", np.uint8)) == "11e60398"       # the textbook example
+    for n in (1, 15, 16, 17, 5552, 5553, 70000):
+        x = np.random.default_rng(n).integers(0, 256, n, dtype=np.uint8)
+        assert D.adler32_ref(x) == D.adler32_bytewise(x) == f"{zlib.adler32(x.tobytes()):08x}"
+    assert D.adler32_ref(np.full(100000, 255, np.uint8)) == D.adler32_bytewise(np.full(100000, 255, np.uint8))
+
+
+def test_xor_delta_is_an_involution_and_counts_changed_bytes():
+    new, old = _pair(10000, 0.1, 1)
+    diff, changed = D.xor_delta_ref(new, old)
+    assert np.array_equal(diff ^ old, new) and np.array_equal(diff ^ new, old)
+    assert changed == int((new != old).sum()) and 0 < changed < 1500
+    assert D.xor_delta_ref(old, old)[1] == 0
+
+
+def test_overwrite_encoding_layout_and_round_trip():
+    new, old = _pair(5000, 0.05, 2)
+    enc, changed = D.overwrite_delta_ref(new, old)
+    assert enc.dtype == np.uint8 and enc.size == 4 + 5 * changed
+    assert int.from_bytes(enc[:4].tobytes(), "little") == changed
+    pos = np.frombuffer(enc[4:4 + 4 * changed].tobytes(), "<u4")
+    assert np.all(np.diff(pos.astype(np.int64)) > 0) and np.array_equal(pos, np.flatnonzero(new != old))
+    assert np.array_equal(enc[4 + 4 * changed:], new[pos])
+    assert np.array_equal(D.overwrite_apply_ref(old, enc), new)
+    assert np.array_equal(D.overwrite_apply_ref(D.overwrite_apply_ref(old, enc), enc), new)     # idempotent
+    enc0, c0 = D.overwrite_delta_ref(old, old)
+    assert c0 == 0 and enc0.tolist() == [0, 0, 0, 0]
