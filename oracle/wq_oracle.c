@@ -31,9 +31,12 @@
  *     of the reference's tests/test_block_fp8_zero_block.py:38-75 and the known-answer
  *     test tests/test_hf_to_megatron.py:345-358.
  *   - fp8 mode 1 (Triton kernel): the restatement assumes IEEE round-to-nearest for both
- *     divisions and the multiply.  No reference test or vector exists and the Triton
- *     lowering of "/" on the reference's platform is not guaranteed IEEE-exact:
- *     PARITY UNPINNED against the reference-on-GPU; the IEEE restatement is the contract.
+ *     divisions and the multiply.  No reference test or vector exists, and on NVIDIA hardware
+ *     Triton's "/" is not guaranteed IEEE-exact (PARITY UNPINNED there).  On MI355X it is
+ *     pinned: oracle/triton_ref.py restates the kernel in Triton and the GPU tests find it
+ *     bit-identical to this file's reading for every bf16 amax and every bf16 value.
+ *   - fp8 mode 2 and the bf16 divisor of the per-tensor form: pinned by torch's own GPU
+ *     kernels run on the same inputs (tests/test_gpu_fp8.py).
  *   - wqo_int4_fake_quant: the reference kernel is CUDA-only, has no test and cannot be
  *     built here without generated (hipified) code: PARITY UNPINNED against reference
  *     output.  Pinned to the source text by exact rational arithmetic on small inputs,
