@@ -21,6 +21,7 @@ typedef __bf16 bf16x2d __attribute__((ext_vector_type(2)));
 constexpr int kDqSteps = 8;                       // packed words per lane
 constexpr int kDqWordsPerWg = 256 * kDqSteps;     // 8 KiB of packed input, 32 KiB of bf16 output
 constexpr int kDqItemsPerXcdRun = 32;
+constexpr int kDqOccupancyPadBytes = 45 * 1024;           // unused dynamic LDS that caps workgroups per CU
 
 __device__ __forceinline__ uint32_t pack2_bf16(float a, float b)
 {
@@ -65,6 +66,7 @@ __global__ __launch_bounds__(256) void int4_dequant_kernel(const uint32_t* __res
 
 constexpr int kSteGroupsPerWg = 64;
 constexpr int kSteItemsPerXcdRun = 32;
+constexpr int kSteOccupancyPadBytes = 36 * 1024;
 
 template <int L>
 __device__ __forceinline__ float ste_lanes_max(float v)
@@ -113,14 +115,27 @@ __global__ __launch_bounds__(256) void int4_fake_ste_kernel(const uint16_t* __re
         float s = div7 == WQ_DIV7_DEVICE ? u2f(mb << 16) * (1.0f / 7.0f) : u2f(mb << 16) / 7.0f;
         s = (s != s) ? s : fmaxf(s, 1e-5f);           // clamp(min=1e-5) keeps NaN
         float o[8];
+        // Finite amax under the reciprocal-multiply rule: s is the scale of the pack kernel, for which
+        // q0 = x*r, q = fma(fma(-q0, s, x), r, q0) rounds to the same integer as the IEEE quotient for every bf16 x
+        // of the group (the exhaustive check of the pack function covers exactly these pairs).  |q| <= 7 there, so
+        // the clamp is a no-op; adding and subtracting 1.5 * 2^23 rounds half to even.  The result carries the
+        // sign of x, zero included (round and clamp keep it, s is positive); it is restored on the bf16 pairs.
+        const bool fast = div7 == WQ_DIV7_DEVICE && mb < kBf16Inf;
+        if (fast) {
+            const float r = rcp_refined(s);
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            float q = __builtin_rintf(xs[j] / s);
-            if (q == q) q = fminf(fmaxf(q, -7.0f), 7.0f);
-            o[j] = q * s;
+            for (int j = 0; j < 8; ++j) o[j] = ((div_by_scale(xs[j], s, r) + 12582912.0f) - 12582912.0f) * s;
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                float q = __builtin_rintf(xs[j] / s);
+                if (q == q) q = fminf(fmaxf(q, -7.0f), 7.0f);
+                o[j] = q * s;
+            }
         }
         if (g < n_groups) {
-            const u32x4 r = {pack2_bf16(o[0], o[1]), pack2_bf16(o[2], o[3]), pack2_bf16(o[4], o[5]), pack2_bf16(o[6], o[7])};
+            u32x4 r = {pack2_bf16(o[0], o[1]), pack2_bf16(o[2], o[3]), pack2_bf16(o[4], o[5]), pack2_bf16(o[6], o[7])};
+            if (fast) r = (r & 0x7FFF7FFFu) | (v[i] & 0x80008000u);
             stg_nt<u32x4>(y + g * (8 * L) + ll * 8, r);
         }
     }
@@ -139,7 +154,7 @@ WQ_EXPORT int wq_int4_dequant(const int32_t* packed, const void* scale, void* y,
     if (((uintptr_t)y & 15) || ((uintptr_t)packed & 3) || ((uintptr_t)scale & 1)) return WQ_ERR_ALIGN;
     const int64_t n_words = M * (N / 8);
     const int64_t items = cdiv64(n_words, kDqWordsPerWg);
-    int4_dequant_kernel<<<grid_for_items(items), 256, 0, (hipStream_t)stream>>>(
+    int4_dequant_kernel<<<grid_for_items(items), 256, kDqOccupancyPadBytes, (hipStream_t)stream>>>(
         (const uint32_t*)packed, (const uint16_t*)scale, (uint16_t*)y, n_words, group, items);
     WQ_LAUNCH_CHECK();
     return WQ_OK;
@@ -157,9 +172,9 @@ WQ_EXPORT int wq_int4_fake_quant_ste(const void* x, void* y, int64_t M, int64_t 
     const int64_t items = cdiv64(n_groups, kSteGroupsPerWg);
     hipStream_t st = (hipStream_t)stream;
     const dim3 g = grid_for_items(items);
-    if (group == 32) int4_fake_ste_kernel<4><<<g, 256, 0, st>>>((const uint16_t*)x, (uint16_t*)y, n_groups, items, div7);
-    else if (group == 64) int4_fake_ste_kernel<8><<<g, 256, 0, st>>>((const uint16_t*)x, (uint16_t*)y, n_groups, items, div7);
-    else int4_fake_ste_kernel<16><<<g, 256, 0, st>>>((const uint16_t*)x, (uint16_t*)y, n_groups, items, div7);
+    if (group == 32) int4_fake_ste_kernel<4><<<g, 256, kSteOccupancyPadBytes, st>>>((const uint16_t*)x, (uint16_t*)y, n_groups, items, div7);
+    else if (group == 64) int4_fake_ste_kernel<8><<<g, 256, kSteOccupancyPadBytes, st>>>((const uint16_t*)x, (uint16_t*)y, n_groups, items, div7);
+    else int4_fake_ste_kernel<16><<<g, 256, kSteOccupancyPadBytes, st>>>((const uint16_t*)x, (uint16_t*)y, n_groups, items, div7);
     WQ_LAUNCH_CHECK();
     return WQ_OK;
 }
