@@ -6,7 +6,7 @@ own function names.  Everything computes in hand-written gfx950 HIP kernels reac
 of ``slime_amd/lib/libslime_amd_wq.so``; there is no CPU or pure-torch fallback.
 """
 
-from . import _lib, arith
+from . import _lib, arith, delta
 from .arith import get_torch_arithmetic, set_torch_arithmetic, torch_arithmetic
 from .fp8 import (
     Fp8DequantPlan,
