@@ -233,6 +233,42 @@ def bench_delta(dev, steps, warmup):
     return out
 
 
+def bench_single_tensor_forms(dev, steps, warmup):
+    """The per-row / per-tensor FP8 forms and the fake-INT4 quantiser on one vocabulary-sized tensor
+    [151936, 2560] bf16 (778 MB), through the Python layer (output allocation included in the timing)."""
+    import torch
+
+    import slime_amd
+    from oracle import c_oracle
+
+    w = _gen_bf16((151936, 2560), dev, outliers=True)
+    el = w.numel()
+    head = w[:512].cpu()
+    out = {}
+    cases = (("fp8_channel_quant", lambda: slime_amd.channel_fp8(w), 3 * el + 4 * w.shape[0]),
+             ("fp8_tensor_quant", lambda: slime_amd.tensor_fp8(w), 5 * el),
+             ("int4_fake_quant_sym", lambda: slime_amd.fake_int4_quant_cuda(w, (1, 128), True), 4 * el + 4 * el // 128),
+             ("int4_fake_quant_asym", lambda: slime_amd.fake_int4_quant_cuda(w, (1, 128), False), 4 * el + 4 * el // 128))
+    for name, fn, algo in cases:
+        wall_ms, ev_ms, ev_min = _time_launches(fn, steps, warmup)
+        out[name] = {"kernel_ms": ev_ms, "bf16_GBps": 2 * el / ev_ms / 1e6, "algo_GBps": algo / ev_ms / 1e6,
+                     "hbm_frac": algo / ev_ms / 1e6 / HBM_PEAK_GBS}
+    q, s = slime_amd.channel_fp8(w)
+    qo, so = c_oracle.fp8_channel_quant(head, 2)
+    assert torch.equal(q[:512].cpu().view(torch.uint8), qo) and torch.equal(s[:512].cpu().view(torch.int32), so.view(torch.int32))
+    for sym in (True, False):
+        q, s, z = slime_amd.fake_int4_quant_cuda(w, (1, 128), sym)
+        qo, so, zo = c_oracle.int4_fake_quant(head, (1, 128), sym)
+        assert torch.equal(q[:512].cpu().view(torch.int16), qo.view(torch.int16))
+        assert torch.equal(s[:512].cpu().view(torch.int16), so.view(torch.int16))
+        assert torch.equal(z[:512].cpu().view(torch.int16), zo.view(torch.int16))
+    out["workload"] = ("one bf16 [151936, 2560] tensor (778 MB); algorithmic bytes per element: channel 3, tensor 5 (two "
+                       "reads), fake INT4 4; parity checked on the first 512 rows")
+    del w
+    torch.cuda.empty_cache()
+    return out
+
+
 def bench_fp8_dequant(dev, steps, warmup, experts):
     import torch
 
@@ -357,7 +393,7 @@ def main():
     ap.add_argument("--dequant-experts", type=int, default=256)
     ap.add_argument("--no-extras", action="store_true", help="headline workload only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
-    ap.add_argument("--only", choices=["int4", "dequant", "int4deq", "ste", "delta", "copy", "stream"], default=None,
+    ap.add_argument("--only", choices=["int4", "dequant", "int4deq", "ste", "delta", "forms", "copy", "stream"], default=None,
                     help="run just one of the other legs and print its record: a kernel for profiling, the plain copy "
                          "kernel that hardware counters are calibrated against, or the host-resident streaming run "
                          "(64 x 1 GiB buckets, PCIe-bound)")
@@ -386,6 +422,9 @@ def main():
         return
     if args.only in ("int4deq", "ste"):
         print(json.dumps(bench_int4_inverse(dev, args.steps, args.warmup, min(args.int4_layers, 8), args.only)))
+        return
+    if args.only == "forms":
+        print(json.dumps(bench_single_tensor_forms(dev, args.steps, args.warmup)))
         return
     if args.only == "delta":
         print(json.dumps(bench_delta(dev, args.steps, args.warmup)))
@@ -434,6 +473,7 @@ def main():
             extras["int4_dequant"] = bench_int4_inverse(dev, args.steps, args.warmup, min(args.int4_layers, 8), "int4deq")
             extras["int4_qat_forward"] = bench_int4_inverse(dev, args.steps, args.warmup, min(args.int4_layers, 8), "ste")
         extras["delta_xor"] = bench_delta(dev, args.steps, args.warmup)
+        extras["single_tensor_forms"] = bench_single_tensor_forms(dev, args.steps, args.warmup)
         line["other_workloads"] = extras
     print(json.dumps(line))
 

@@ -244,6 +244,150 @@ __global__ __launch_bounds__(256) void fp8_tensor_apply_kernel(const uint16_t* _
     }
 }
 
+// ---- per-row / per-tensor scale, contiguous operands ------------------------------------------------
+
+constexpr int kRowsPerXcdRun = 32;
+constexpr int kRowPieceElems = 256 * 8;      // elements of a row one load step of the workgroup covers
+
+// One workgroup per row, the row held in registers (STEPS 16-byte pieces per lane, rows of up to 2048 * STEPS
+// elements): amax, scale, and the same division-free element function as the block kernel - the scale rule and
+// the (amax, x) domain are the block quantiser's, so the same exhaustive check covers it.
+template <int STEPS>
+__global__ __launch_bounds__(256) void fp8_row_quant_vec_kernel(const uint16_t* __restrict__ x, int64_t M, int64_t N,
+                                                               int64_t sx_m, uint8_t* __restrict__ y, int64_t sy_m,
+                                                               float* __restrict__ s, int mode)
+{
+    __shared__ __attribute__((aligned(16))) uint32_t lds[16];
+    const int64_t slot = (int64_t)blockIdx.x + (int64_t)blockIdx.y * gridDim.x;
+    if (slot >= M) return;
+    const int64_t row = xcd_chunked_item(slot, M, kRowsPerXcdRun);
+    const char* xr = (const char*)(x + row * sx_m);
+    char* yr = (char*)(y + row * sy_m);
+    const int n_pieces = (int)(N / 8);
+    const int t = threadIdx.x;
+    u32x4 v[STEPS];
+#pragma unroll
+    for (int i = 0; i < STEPS; ++i) {
+        // lanes past the end of the row re-read its last piece instead of branching around the load
+        const int piece = min(i * 256 + t, n_pieces - 1);
+        v[i] = ldg_nt<u32x4>(xr + (uint32_t)piece * 16u);
+    }
+    uint32_t m = 0;
+#pragma unroll
+    for (int i = 0; i < STEPS; ++i) {
+        if (i * 256 + t >= n_pieces) v[i] = (u32x4){0u, 0u, 0u, 0u};
+        m = pk_absmax(m, v[i].x);
+        m = pk_absmax(m, v[i].y);
+        m = pk_absmax(m, v[i].z);
+        m = pk_absmax(m, v[i].w);
+    }
+    m = row16_max_u32(pk_fold(m));
+    if ((t & 15) == 0) lds[t >> 4] = m;
+    __syncthreads();
+    m = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const u32x4 a = ((const u32x4*)lds)[i];
+        m = max(m, max(max(a.x, a.y), max(a.z, a.w)));
+    }
+    const Fp8BlockParams p = torch_params(m, mode);
+    if (t == 0) stg<float>(s + row, p.scale);
+    if (p.fast) {
+#pragma unroll
+        for (int i = 0; i < STEPS; ++i) {
+            const int piece = i * 256 + t;
+            u32x2 o;
+            o.x = fp8_quant4_fast<WQ_FP8_MODE_TORCH>(v[i].x, v[i].y, p);
+            o.y = fp8_quant4_fast<WQ_FP8_MODE_TORCH>(v[i].z, v[i].w, p);
+            if (piece < n_pieces) stg_nt<u32x2>(yr + (uint32_t)piece * 8u, o);
+        }
+    } else {
+        // NaN/Inf row (rare): literal arithmetic on re-read data
+#pragma nounroll
+        for (int i = 0; i < STEPS; ++i) {
+            const int piece = i * 256 + t;
+            if (piece >= n_pieces) continue;
+            const u32x4 w = ldg<u32x4>(xr + (uint32_t)piece * 16u);
+            u32x2 o;
+            o.x = fp8_quant4_exact<WQ_FP8_MODE_TORCH>(w.x, w.y, p);
+            o.y = fp8_quant4_exact<WQ_FP8_MODE_TORCH>(w.z, w.w, p);
+            stg<u32x2>(yr + (uint32_t)piece * 8u, o);
+        }
+    }
+}
+
+// Per-tensor amax of a contiguous tensor: a bounded grid, four 16-byte pieces per lane in flight, one atomic per
+// workgroup.
+__global__ __launch_bounds__(256) void fp8_tensor_amax_vec_kernel(const uint16_t* __restrict__ x, int64_t n_pieces,
+                                                                 uint32_t* __restrict__ ws)
+{
+    __shared__ uint32_t lds[4];
+    uint32_t m = 0;
+    const char* xb = (const char*)x;
+    for (int64_t p0 = (int64_t)blockIdx.x * 1024 + threadIdx.x; p0 < n_pieces; p0 += (int64_t)gridDim.x * 1024) {
+        u32x4 v[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = ldg_nt<u32x4>(xb + min(p0 + i * 256, n_pieces - 1) * 16);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            // a piece past the end was read from the last valid one: harmless for a maximum
+            m = pk_absmax(m, v[i].x);
+            m = pk_absmax(m, v[i].y);
+            m = pk_absmax(m, v[i].z);
+            m = pk_absmax(m, v[i].w);
+        }
+    }
+    m = wave64_max_u32(pk_fold(m));
+    if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6] = m;
+    __syncthreads();
+    if (threadIdx.x == 0) atomicMax(ws, max(max(lds[0], lds[1]), max(lds[2], lds[3])));
+}
+
+typedef float f32x2q __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2q __attribute__((ext_vector_type(2)));
+
+// Two elements of the per-tensor form: IEEE quotient, rounded to bf16 (the reference's bf16 tensor), NaN-propagating
+// clamp, e4m3fn.  Returns the two codes in the low 16 bits.
+__device__ __forceinline__ uint32_t tensor_quant2(uint32_t w, float divisor)
+{
+    f32x2q q = {bf16lo(w) / divisor, bf16hi(w) / divisor};
+    const uint32_t b = __builtin_bit_cast(uint32_t, __builtin_convertvector(q, bf16x2q));
+    float q0 = bf16lo(b), q1 = bf16hi(b);
+    const bool nan0 = q0 != q0, nan1 = q1 != q1;
+    q0 = fminf(fmaxf(q0, -kFp8Max), kFp8Max);
+    q1 = fminf(fmaxf(q1, -kFp8Max), kFp8Max);
+    uint32_t r = cvt_pk_fp8_lo(q0, q1, 0u) & 0xFFFFu;
+    if (nan0) r = (r & 0xFF00u) | 0x7Fu;
+    if (nan1) r = (r & 0x00FFu) | 0x7F00u;
+    return r;
+}
+
+__global__ __launch_bounds__(256) void fp8_tensor_apply_vec_kernel(const uint16_t* __restrict__ x, int64_t n_pieces,
+                                                                  uint8_t* __restrict__ y, float* __restrict__ s,
+                                                                  const uint32_t* __restrict__ ws, int mode,
+                                                                  int64_t items)
+{
+    const int64_t slot = (int64_t)blockIdx.x + (int64_t)blockIdx.y * gridDim.x;
+    if (slot >= items) return;
+    const int64_t item = xcd_chunked_item(slot, items, kRowsPerXcdRun);
+    const Fp8BlockParams p = torch_params(*ws, mode);
+    if (slot == 0 && threadIdx.x == 0) s[0] = p.scale;
+    const float divisor = mode == WQ_FP8_MODE_TORCH_DEVICE ? u2f(f32_to_bf16_bits(p.scale) << 16) : p.scale;
+    const char* xb = (const char*)x;
+    const int64_t p0 = item * 1024 + threadIdx.x;
+    u32x4 v[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = ldg_nt<u32x4>(xb + min(p0 + i * 256, n_pieces - 1) * 16);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int64_t piece = p0 + i * 256;
+        u32x2 o;
+        o.x = tensor_quant2(v[i].x, divisor) | (tensor_quant2(v[i].y, divisor) << 16);
+        o.y = tensor_quant2(v[i].z, divisor) | (tensor_quant2(v[i].w, divisor) << 16);
+        if (piece < n_pieces) stg_nt<u32x2>(y + piece * 8, o);
+    }
+}
+
 static bool known_mode(int mode)
 {
     return mode == WQ_FP8_MODE_TORCH || mode == WQ_FP8_MODE_TRITON || mode == WQ_FP8_MODE_TORCH_DEVICE;
@@ -318,8 +462,17 @@ WQ_EXPORT int wq_fp8_row_quant(const void* x, int64_t M, int64_t N, int64_t sx_m
     if (mode != WQ_FP8_MODE_TORCH && mode != WQ_FP8_MODE_TORCH_DEVICE) return WQ_ERR_MODE;
     if (M == 0) return WQ_OK;
     if (!s || (N > 0 && (!x || !y))) return WQ_ERR_NULL;
-    fp8_row_quant_kernel<<<grid_for_items(M), 256, 0, (hipStream_t)stream>>>((const uint16_t*)x, M, N, sx_m, sx_n,
-                                                                      (uint8_t*)y, sy_m, s, mode);
+    hipStream_t st = (hipStream_t)stream;
+    const bool vec = sx_n == 1 && N > 0 && (N & 7) == 0 && N <= 8 * kRowPieceElems && (sx_m & 7) == 0 && (sy_m & 7) == 0 &&
+                     ((uintptr_t)x & 15) == 0 && ((uintptr_t)y & 7) == 0;
+    const uint16_t* xp = (const uint16_t*)x;
+    uint8_t* yp = (uint8_t*)y;
+    const dim3 g = grid_for_items(M);
+    if (!vec) fp8_row_quant_kernel<<<g, 256, 0, st>>>(xp, M, N, sx_m, sx_n, yp, sy_m, s, mode);
+    else if (N <= kRowPieceElems) fp8_row_quant_vec_kernel<1><<<g, 256, 0, st>>>(xp, M, N, sx_m, yp, sy_m, s, mode);
+    else if (N <= 2 * kRowPieceElems) fp8_row_quant_vec_kernel<2><<<g, 256, 0, st>>>(xp, M, N, sx_m, yp, sy_m, s, mode);
+    else if (N <= 4 * kRowPieceElems) fp8_row_quant_vec_kernel<4><<<g, 256, 0, st>>>(xp, M, N, sx_m, yp, sy_m, s, mode);
+    else fp8_row_quant_vec_kernel<8><<<g, 256, 0, st>>>(xp, M, N, sx_m, yp, sy_m, s, mode);
     WQ_LAUNCH_CHECK();
     return WQ_OK;
 }
@@ -331,8 +484,21 @@ WQ_EXPORT int wq_fp8_tensor_quant(const void* x, int64_t M, int64_t N, int64_t s
     if (mode != WQ_FP8_MODE_TORCH && mode != WQ_FP8_MODE_TORCH_DEVICE) return WQ_ERR_MODE;
     if (!s || !workspace || (M * N > 0 && (!x || !y))) return WQ_ERR_NULL;
     const int64_t total = M * N;
-    int blocks = (int)min((int64_t)(256 * 16), max((int64_t)1, cdiv64(total, 256 * 8)));
     hipStream_t st = (hipStream_t)stream;
+    const bool vec = total > 0 && sx_n == 1 && sx_m == N && sy_m == N && (total & 7) == 0 && ((uintptr_t)x & 15) == 0 &&
+                     ((uintptr_t)y & 7) == 0;
+    if (vec) {
+        const int64_t n_pieces = total / 8;
+        const int64_t items = cdiv64(n_pieces, 1024);
+        const int blocks = (int)min((int64_t)2048, items);
+        fp8_tensor_amax_vec_kernel<<<blocks, 256, 0, st>>>((const uint16_t*)x, n_pieces, workspace);
+        WQ_LAUNCH_CHECK();
+        fp8_tensor_apply_vec_kernel<<<grid_for_items(items), 256, 0, st>>>((const uint16_t*)x, n_pieces, (uint8_t*)y, s,
+                                                                          workspace, mode, items);
+        WQ_LAUNCH_CHECK();
+        return WQ_OK;
+    }
+    int blocks = (int)min((int64_t)(256 * 16), max((int64_t)1, cdiv64(total, 256 * 8)));
     fp8_tensor_amax_kernel<<<blocks, 256, 0, st>>>((const uint16_t*)x, M, N, sx_m, sx_n, workspace);
     WQ_LAUNCH_CHECK();
     fp8_tensor_apply_kernel<<<blocks, 256, 0, st>>>((const uint16_t*)x, M, N, sx_m, sx_n, (uint8_t*)y, sy_m, s,

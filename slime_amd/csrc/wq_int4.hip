@@ -261,6 +261,108 @@ __global__ __launch_bounds__(256) void int4_fake_quant_kernel(const T* __restric
     }
 }
 
+// Fast form of the kernel above for the layout the callers use: bf16, contiguous rows, (1 x 32 | 64 | 128) groups
+// that tile the row.  A group is owned by L adjacent lanes (one 16-byte load, one 16-byte store per lane).  The
+// symmetric branch with a finite amax uses the division-free element function of the pack kernel (same scale rule,
+// same (amax, x) domain, same exhaustive check); codes carry the sign of x, zero included, as rintf(x / scale) does.
+constexpr int kFakeGroupsPerWg = 64;
+constexpr int kFakeItemsPerXcdRun = 32;
+constexpr unsigned kFakeOccupancyPadBytes = 36 * 1024;
+
+template <int L>
+__device__ __forceinline__ float lanes_min_f32(float v)
+{
+    v = fminf(v, u2f(dpp_u32<0xB1>(f2u(v))));
+    v = fminf(v, u2f(dpp_u32<0x4E>(f2u(v))));
+    if (L >= 8) v = fminf(v, u2f(dpp_u32<0x141>(f2u(v))));
+    if (L >= 16) v = fminf(v, u2f(dpp_u32<0x140>(f2u(v))));
+    return v;
+}
+
+__device__ __forceinline__ uint32_t pack2_bf16_hw(float a, float b)
+{
+    f32x2_t v = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+}
+
+template <int L, bool SYM>
+__global__ __launch_bounds__(256) void int4_fake_quant_vec_kernel(const uint16_t* __restrict__ x, int64_t sx_m,
+                                                                 int groups_per_row, uint16_t* __restrict__ q,
+                                                                 uint16_t* __restrict__ scale_out,
+                                                                 uint16_t* __restrict__ zero_out, int64_t n_groups,
+                                                                 int64_t total_items)
+{
+    constexpr int CL = 256 / L;
+    constexpr int STEPS = kFakeGroupsPerWg / CL;
+    const int64_t slot = (int64_t)blockIdx.x + (int64_t)blockIdx.y * gridDim.x;
+    if (slot >= total_items) return;
+    const int64_t item = xcd_chunked_item(slot, total_items, kFakeItemsPerXcdRun);
+    const int cl = threadIdx.x / L, ll = threadIdx.x % L;
+    const int64_t g0 = item * kFakeGroupsPerWg + cl;
+    u32x4 v[STEPS];
+#pragma unroll
+    for (int i = 0; i < STEPS; ++i) {
+        const int64_t g = min(g0 + i * CL, n_groups - 1);
+        const int64_t row = g / groups_per_row, gc = g - row * groups_per_row;
+        v[i] = ldg_nt<u32x4>(x + row * sx_m + gc * (8 * L) + ll * 8);
+    }
+#pragma unroll
+    for (int i = 0; i < STEPS; ++i) {
+        const int64_t g = g0 + i * CL;
+        float xs[8];
+        unpack8(v[i], xs);
+        float o[8];
+        float scale, zero = 0.0f;
+        bool restore_sign = false;
+        if (SYM) {
+            const float amax = lanes_max_f32<L>(absmax8(xs));
+            scale = int4_scale_sym(amax);
+            if (amax < INFINITY) {
+                const float r = rcp_refined(scale);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) o[j] = (div_by_scale(xs[j], scale, r) + 12582912.0f) - 12582912.0f;
+                restore_sign = true;
+            } else {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) o[j] = __builtin_rintf(xs[j] / scale);
+            }
+        } else {
+            float vmax = fmaxf(fmaxf(fmaxf(xs[0], xs[1]), fmaxf(xs[2], xs[3])), fmaxf(fmaxf(xs[4], xs[5]), fmaxf(xs[6], xs[7])));
+            float vmin = fminf(fminf(fminf(xs[0], xs[1]), fminf(xs[2], xs[3])), fminf(fminf(xs[4], xs[5]), fminf(xs[6], xs[7])));
+            vmax = lanes_max_f32<L>(vmax);
+            vmin = lanes_min_f32<L>(vmin);
+            scale = fmaxf((vmax - vmin) * (1.0f / 15.0f), 1e-5f);
+            zero = fminf(fmaxf(-__builtin_rintf(vmin / scale), 0.0f), 15.0f) + 0.0f;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) o[j] = __builtin_rintf(xs[j] / scale) + zero;
+        }
+        if (g < n_groups) {
+            u32x4 r = {pack2_bf16_hw(o[0], o[1]), pack2_bf16_hw(o[2], o[3]), pack2_bf16_hw(o[4], o[5]),
+                       pack2_bf16_hw(o[6], o[7])};
+            if (restore_sign) r = (r & 0x7FFF7FFFu) | (v[i] & 0x80008000u);
+            stg_nt<u32x4>(q + g * (8 * L) + ll * 8, r);
+            if (ll == 0) {
+                stg<uint16_t>(scale_out + g, (uint16_t)f32_to_bf16_bits(scale));
+                stg<uint16_t>(zero_out + g, (uint16_t)f32_to_bf16_bits(zero));
+            }
+        }
+    }
+}
+
+template <bool SYM>
+static bool launch_fake_vec(const uint16_t* x, int64_t M, int64_t N, int64_t sx_m, int bn, uint16_t* q, uint16_t* sc,
+                            uint16_t* zp, hipStream_t st)
+{
+    const int64_t n_groups = M * (N / bn);
+    const int64_t items = cdiv64(n_groups, kFakeGroupsPerWg);
+    const dim3 g = grid_for_items(items);
+    const int gpr = (int)(N / bn);
+    if (bn == 32) int4_fake_quant_vec_kernel<4, SYM><<<g, 256, kFakeOccupancyPadBytes, st>>>(x, sx_m, gpr, q, sc, zp, n_groups, items);
+    else if (bn == 64) int4_fake_quant_vec_kernel<8, SYM><<<g, 256, kFakeOccupancyPadBytes, st>>>(x, sx_m, gpr, q, sc, zp, n_groups, items);
+    else int4_fake_quant_vec_kernel<16, SYM><<<g, 256, kFakeOccupancyPadBytes, st>>>(x, sx_m, gpr, q, sc, zp, n_groups, items);
+    return true;
+}
+
 template <bool GROUPED>
 static int launch_pack(const Int4PackArgs& a, int64_t work, int group, hipStream_t st)
 {
@@ -324,7 +426,12 @@ WQ_EXPORT int wq_int4_fake_quant(const void* x, int dtype, int64_t M, int64_t N,
     if (!x || !q || !scale || !zero) return WQ_ERR_NULL;
     const int64_t groups = cdiv64(M, bm) * cdiv64(N, bn);
     hipStream_t st = (hipStream_t)stream;
-    if (dtype == WQ_DTYPE_BF16)
+    const bool vec = dtype == WQ_DTYPE_BF16 && bm == 1 && (bn == 32 || bn == 64 || bn == 128) && sx_n == 1 && N % bn == 0 &&
+                     (sx_m & 7) == 0 && N / bn < (1ll << 31) && ((uintptr_t)x & 15) == 0 && ((uintptr_t)q & 15) == 0;
+    if (vec) {
+        if (sym) launch_fake_vec<true>((const uint16_t*)x, M, N, sx_m, bn, (uint16_t*)q, (uint16_t*)scale, (uint16_t*)zero, st);
+        else launch_fake_vec<false>((const uint16_t*)x, M, N, sx_m, bn, (uint16_t*)q, (uint16_t*)scale, (uint16_t*)zero, st);
+    } else if (dtype == WQ_DTYPE_BF16)
         int4_fake_quant_kernel<uint16_t><<<grid_for_items(cdiv64(groups, 4)), 256, 0, st>>>(
             (const uint16_t*)x, M, N, sx_m, sx_n, bm, bn, sym, (uint16_t*)q, (uint16_t*)scale, (uint16_t*)zero);
     else

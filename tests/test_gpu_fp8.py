@@ -163,10 +163,11 @@ def test_reference_suite_invariants_on_gpu(cuda):
     assert not torch.isnan(q.float()).any() and (deq - w.float()).abs().max() < 0.5
 
 
-@pytest.mark.parametrize("shape", [(64, 256), (3, 1000), (257, 129), (1024, 2560)])
+@pytest.mark.parametrize("shape", [(64, 256), (3, 1000), (257, 129), (1024, 2560), (7, 7168), (130, 9728), (5, 20000),
+                                   (33, 8200), (1, 8), (300, 16384), (2, 16392)])
 def test_channel_and_tensor_quant(cuda, shape):
     w = I.weights(*shape, seed=8)
-    w[1] = 0
+    w[shape[0] // 2] = 0
     for gpu_fn, ora, sshape in ((slime_amd.channel_fp8, C.fp8_channel_quant, (shape[0], 1)),
                                 (slime_amd.tensor_fp8, C.fp8_tensor_quant, (1,))):
         for mode, arith in ARITH.items():
@@ -330,3 +331,56 @@ def test_torch_ops_on_the_gpu_agree_with_the_kernels(cuda):
             q, s = mine(wg)
             assert torch.equal(_bits32(s), _bits32(sr))
             assert torch.equal(_codes(q), _codes(qr))
+
+
+def test_channel_and_tensor_quant_views_and_specials(cuda):
+    base = I.weights(300, 4104, seed=31)
+    base[5, 100] = float("nan")
+    base[9, 7] = float("inf")
+    base[11] = 0
+    base[12] = -0.0
+    base[13, :2048] = I.subnormal_block(1, 2048, seed=3)[0]
+    bg = base.to(cuda)
+    views = [lambda t: t, lambda t: t[:, 8:4104], lambda t: t[:, :4096], lambda t: t[::2], lambda t: t[:, 4:],
+             lambda t: t.t(), lambda t: t[20:], lambda t: t[20:, :2048]]
+    for v in views:
+        for mode, arith in ARITH.items():
+            with slime_amd.torch_arithmetic(arith):
+                q, s = slime_amd.channel_fp8(v(bg))
+            qo, so = C.fp8_channel_quant(v(base), mode)
+            so_c, s_c = so, s.cpu()
+            assert torch.equal(s_c.isnan(), so_c.isnan())
+            ok = ~so_c.isnan().view(-1)
+            assert torch.equal(_bits32(s_c)[ok], _bits32(so_c)[ok])
+            qc = _codes(q)
+            nan_o = (qo & 0x7F) == 0x7F
+            assert torch.equal((qc & 0x7F) == 0x7F, nan_o) and torch.equal(qc[~nan_o], qo[~nan_o])
+    clean = I.weights(256, 4096, seed=32)
+    for v in (lambda t: t, lambda t: t[:, 8:], lambda t: t[::2], lambda t: t.t()):
+        for mode, arith in ARITH.items():
+            with slime_amd.torch_arithmetic(arith):
+                q, s = slime_amd.tensor_fp8(v(clean.to(cuda)))
+            qo, so = C.fp8_tensor_quant(v(clean), mode)
+            assert torch.equal(_codes(q), qo) and torch.equal(_bits32(s), _bits32(so))
+    with_nan = clean.clone()
+    with_nan[3, 3] = float("nan")
+    q, s = slime_amd.tensor_fp8(with_nan.to(cuda))
+    assert s.isnan().all() and ((_codes(q) & 0x7F) == 0x7F).all()
+
+
+def test_channel_quant_every_bf16_value(cuda):
+    rows = []
+    vals = I.finite_bf16_values()
+    g = I.gen(17)
+    for ab in torch.randint(1, 0x7F80, (20,), generator=g).tolist() + [0x2B8C, 0x2B8D, 0x7F7F, 1]:
+        amax = torch.tensor([ab], dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+        x = vals[vals.abs() <= amax][:4096 * 3]
+        x = torch.cat([x, torch.zeros((-x.numel()) % 4096, dtype=torch.bfloat16)]).view(-1, 4096)
+        x[:, 0] = amax
+        rows.append(x)
+    w = torch.cat(rows)
+    for mode, arith in ARITH.items():
+        with slime_amd.torch_arithmetic(arith):
+            q, s = slime_amd.channel_fp8(w.to(cuda))
+        qo, so = C.fp8_channel_quant(w, mode)
+        assert torch.equal(_codes(q), qo) and torch.equal(_bits32(s), _bits32(so))

@@ -82,6 +82,54 @@ def test_fake_quant(cuda, block, sym):
         assert I.same_bits(q.cpu(), qo) and I.same_bits(s.cpu(), so) and I.same_bits(z.cpu(), zo)
 
 
+def _fake_quant_same(q, s, z, qo, so, zo):
+    nan = qo.isnan()
+    assert torch.equal(q.isnan(), nan) and torch.equal(q[~nan].view(torch.int16), qo[~nan].view(torch.int16))
+    assert I.same_bits(s, so) and I.same_bits(z, zo)
+
+
+@pytest.mark.parametrize("gs", [32, 64, 128])
+@pytest.mark.parametrize("sym", [True, False])
+def test_fake_quant_row_groups_fast_layout(cuda, gs, sym):
+    # contiguous-row bf16 with groups that tile the row: the layout pack_layer and the QAT callers use
+    w = I.weights(333, 1024, seed=gs, outlier_p=0.01)
+    w[0, :gs] = 0
+    w[1, :gs] = -0.0
+    w[2, :256] = I.subnormal_block(1, 256, seed=1)[0]
+    w[3, :256] = I.near_max_block(1, 256, seed=2, amax=3.0e38)[0]
+    w[4, :256] = I.weights(1, 256, seed=4, std=1e-6)[0]
+    wg = w.to(cuda)
+    for view in (lambda t: t, lambda t: t[:, 128:896], lambda t: t[::3], lambda t: t[5:, 256:]):
+        q, s, z = slime_amd.fake_int4_quant_cuda(view(wg), (1, gs), sym)
+        _fake_quant_same(q.cpu(), s.cpu(), z.cpu(), *C.int4_fake_quant(view(w), (1, gs), sym))
+    bad = w.clone()
+    bad[7, 5] = float("nan")
+    bad[8, 130] = float("inf")
+    bad[9, :gs] = float("nan")
+    q, s, z = slime_amd.fake_int4_quant_cuda(bad.to(cuda), (1, gs), sym)
+    qo, so, zo = C.int4_fake_quant(bad, (1, gs), sym)
+    ok = torch.ones(333, dtype=torch.bool)
+    ok[7:10] = False                                 # rows with NaN / Inf: only NaN-ness of the codes is specified
+    _fake_quant_same(q.cpu()[ok], s.cpu()[ok], z.cpu()[ok], qo[ok], so[ok], zo[ok])
+    assert torch.equal(q.cpu()[~ok].isnan(), qo[~ok].isnan())
+
+
+@pytest.mark.parametrize("sym", [True, False])
+def test_fake_quant_every_bf16_value(cuda, sym):
+    vals = I.finite_bf16_values()
+    g = I.gen(13)
+    rows = []
+    for ab in torch.randint(1, 0x7F80, (16,), generator=g).tolist() + [0x3728, 0x3727, 0x7F7F, 1]:
+        amax = torch.tensor([ab], dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+        x = vals[vals.abs() <= amax]
+        x = torch.cat([x, torch.zeros((-x.numel()) % 1024, dtype=torch.bfloat16)]).view(-1, 128)
+        x[:, 0] = amax
+        rows.append(x.reshape(-1, 1024))
+    w = torch.cat(rows)
+    q, s, z = slime_amd.fake_int4_quant_cuda(w.to(cuda), (1, 128), sym)
+    _fake_quant_same(q.cpu(), s.cpu(), z.cpu(), *C.int4_fake_quant(w, (1, 128), sym))
+
+
 def test_fake_quant_ragged_big(cuda):
     w = I.weights(4100, 3000, seed=2)
     q, s, z = slime_amd.fake_int4_quant_cuda(w.to(cuda), (1, 128), True)
