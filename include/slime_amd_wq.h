@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define WQ_ABI_VERSION 3
+#define WQ_ABI_VERSION 4
 
 enum {
     WQ_OK = 0,
@@ -159,6 +159,15 @@ typedef struct wq_int4_pack_desc {
 #define WQ_INT4_GROUPS_PER_WG 64
 int wq_int4_group_quant_pack_grouped(const wq_int4_pack_desc *descs, const int64_t *work_start, int n_desc,
                                      int64_t total_work, int group, void *stream);
+
+/* Asymmetric form of wq_int4_group_quant_pack (pack_layer(weight, group, sym=False),
+ * tools/convert_hf_to_int4_direct.py:123-153): codes rintf(x/scale) + zero with scale = max((max-min)/15, 1e-5)
+ * and zero = clamp(-rintf(min/scale), 0, 15) (fake_int4_quant_cuda.cu:61-75), passed through the reference's
+ * dequantise / re-quantise / clamp-to-uint8 chain and packed without masking, as pack_to_int32 does.
+ * Outputs: packed int32 [M,N/8], scale bf16 [M,N/group], zero bf16 [M,N/group] (the caller packs the zero points
+ * in AWQ order from it, :134-141).  x bf16, unit column stride, 16-byte aligned rows; group in {32, 64, 128}. */
+int wq_int4_group_quant_pack_asym(const void *x, int64_t M, int64_t N, int64_t sx_m, int group,
+                                  int32_t *packed, void *scale, void *zero, void *stream);
 
 /* INT4 pack-quantized -> bf16: y[i,j] = bf16((nibble(i,j) - 8) * f32(scale[i, j/group])), nibble j of word c at
  * bits [4j,4j+4).  packed int32 [M,N/8], scale bf16 [M,N/group], y bf16 [M,N], all contiguous; N % group == 0,

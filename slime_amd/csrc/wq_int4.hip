@@ -349,6 +349,82 @@ __global__ __launch_bounds__(256) void int4_fake_quant_vec_kernel(const uint16_t
     }
 }
 
+// Asymmetric quantise + pack for the same layout: codes rintf(x / scale) + zero, then what the reference's
+// pack_layer does to them before packing - dequantise to bf16, re-quantise, clamp to the uint8 range - and the
+// un-masked shift-add of pack_to_int32 (a code above 15 spills into the neighbouring nibbles there, and so it
+// does here).  That chain is the identity on every code in [0, 17] for every zero point and every bf16 scale below
+// 2^121 (checked by exhaustion in the CPU tests); lanes whose eight codes are all in that range skip it, the others
+// run it literally.
+__device__ __forceinline__ uint32_t code_literal_asym(float q, float z, float sb)
+{
+    const float qb = bf16_round(q);            // the fake-quant kernel stores the code as bf16
+    const float t = bf16_round(qb - z);
+    const float d = bf16_round(t * sb);
+    float r = bf16_round(d / sb);
+    r = bf16_round(r + z);
+    if (r == r) r = fminf(fmaxf(r, 0.0f), 255.0f);
+    return (uint32_t)(int)__builtin_rintf(r);
+}
+
+template <int L>
+__global__ __launch_bounds__(256) void int4_pack_asym_kernel(const uint16_t* __restrict__ x, int64_t sx_m,
+                                                            int groups_per_row, uint32_t* __restrict__ packed,
+                                                            uint16_t* __restrict__ scale_out,
+                                                            uint16_t* __restrict__ zero_out, int64_t n_groups,
+                                                            int64_t total_items)
+{
+    constexpr int CL = 256 / L;
+    constexpr int STEPS = kFakeGroupsPerWg / CL;
+    const int64_t slot = (int64_t)blockIdx.x + (int64_t)blockIdx.y * gridDim.x;
+    if (slot >= total_items) return;
+    const int64_t item = xcd_chunked_item(slot, total_items, kFakeItemsPerXcdRun);
+    const int cl = threadIdx.x / L, ll = threadIdx.x % L;
+    const int64_t g0 = item * kFakeGroupsPerWg + cl;
+    u32x4 v[STEPS];
+#pragma unroll
+    for (int i = 0; i < STEPS; ++i) {
+        const int64_t g = min(g0 + i * CL, n_groups - 1);
+        const int64_t row = g / groups_per_row, gc = g - row * groups_per_row;
+        v[i] = ldg_nt<u32x4>(x + row * sx_m + gc * (8 * L) + ll * 8);
+    }
+#pragma unroll
+    for (int i = 0; i < STEPS; ++i) {
+        const int64_t g = g0 + i * CL;
+        float xs[8];
+        unpack8(v[i], xs);
+        float vmax = fmaxf(fmaxf(fmaxf(xs[0], xs[1]), fmaxf(xs[2], xs[3])), fmaxf(fmaxf(xs[4], xs[5]), fmaxf(xs[6], xs[7])));
+        float vmin = fminf(fminf(fminf(xs[0], xs[1]), fminf(xs[2], xs[3])), fminf(fminf(xs[4], xs[5]), fminf(xs[6], xs[7])));
+        vmax = lanes_max_f32<L>(vmax);
+        vmin = lanes_min_f32<L>(vmin);
+        const float scale = fmaxf((vmax - vmin) * (1.0f / 15.0f), 1e-5f);
+        const float zero = fminf(fmaxf(-__builtin_rintf(vmin / scale), 0.0f), 15.0f) + 0.0f;
+        const uint32_t sb_bits = f32_to_bf16_bits(scale);
+        float q[8];
+        bool plain = sb_bits < kLiteralChainScaleBits;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            q[j] = __builtin_rintf(xs[j] / scale) + zero;
+            plain = plain && q[j] >= 0.0f && q[j] <= 17.0f;
+        }
+        uint32_t word = 0;
+        if (plain) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) word += (uint32_t)q[j] << (4 * j);
+        } else {
+            const float sb = u2f(sb_bits << 16);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) word += code_literal_asym(q[j], zero, sb) << (4 * j);
+        }
+        if (g < n_groups) {
+            stg_nt<uint32_t>(packed + g * L + ll, word);
+            if (ll == 0) {
+                stg<uint16_t>(scale_out + g, (uint16_t)sb_bits);
+                stg<uint16_t>(zero_out + g, (uint16_t)f32_to_bf16_bits(zero));
+            }
+        }
+    }
+}
+
 template <bool SYM>
 static bool launch_fake_vec(const uint16_t* x, int64_t M, int64_t N, int64_t sx_m, int bn, uint16_t* q, uint16_t* sc,
                             uint16_t* zp, hipStream_t st)
@@ -437,6 +513,30 @@ WQ_EXPORT int wq_int4_fake_quant(const void* x, int dtype, int64_t M, int64_t N,
     else
         int4_fake_quant_kernel<float><<<grid_for_items(cdiv64(groups, 4)), 256, 0, st>>>(
             (const float*)x, M, N, sx_m, sx_n, bm, bn, sym, (float*)q, (float*)scale, (float*)zero);
+    WQ_LAUNCH_CHECK();
+    return WQ_OK;
+}
+
+WQ_EXPORT int wq_int4_group_quant_pack_asym(const void* x, int64_t M, int64_t N, int64_t sx_m, int group,
+                                            int32_t* packed, void* scale, void* zero, void* stream)
+{
+    if (M < 0 || N < 0 || group <= 0 || N % group != 0) return WQ_ERR_SHAPE;
+    if (group != 32 && group != 64 && group != 128) return WQ_ERR_UNSUPPORTED;
+    if (M == 0 || N == 0) return WQ_OK;
+    if (!x || !packed || !scale || !zero) return WQ_ERR_NULL;
+    if (((uintptr_t)x & 15) || (sx_m & 7) || ((uintptr_t)packed & 3) || ((uintptr_t)scale & 1) || ((uintptr_t)zero & 1))
+        return WQ_ERR_ALIGN;
+    if (N / group >= (1ll << 31)) return WQ_ERR_TOO_LARGE;
+    const int64_t n_groups = M * (N / group);
+    const int64_t items = cdiv64(n_groups, kFakeGroupsPerWg);
+    const dim3 g = grid_for_items(items);
+    const int gpr = (int)(N / group);
+    hipStream_t st = (hipStream_t)stream;
+    const uint16_t* xp = (const uint16_t*)x;
+    uint32_t* pp = (uint32_t*)packed;
+    if (group == 32) int4_pack_asym_kernel<4><<<g, 256, kFakeOccupancyPadBytes, st>>>(xp, sx_m, gpr, pp, (uint16_t*)scale, (uint16_t*)zero, n_groups, items);
+    else if (group == 64) int4_pack_asym_kernel<8><<<g, 256, kFakeOccupancyPadBytes, st>>>(xp, sx_m, gpr, pp, (uint16_t*)scale, (uint16_t*)zero, n_groups, items);
+    else int4_pack_asym_kernel<16><<<g, 256, kFakeOccupancyPadBytes, st>>>(xp, sx_m, gpr, pp, (uint16_t*)scale, (uint16_t*)zero, n_groups, items);
     WQ_LAUNCH_CHECK();
     return WQ_OK;
 }

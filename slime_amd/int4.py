@@ -5,11 +5,12 @@ in slime/backends/megatron_utils/megatron_to_hf/processors/quantizer_compressed_
 the extension entry point fake_int4_quant_cuda(x, block_size, sym) of
 slime/backends/megatron_utils/kernels/int4_qat/fake_int4_quant_cuda.cu:327-378.
 
-``pack_layer`` with ``sym=True`` on a bf16 weight runs ONE fused HIP kernel (amax, scale, divide,
-round, nibble pack).  The reference's intermediate dequantise / re-quantise steps map every integer
+``pack_layer`` on a bf16 weight runs ONE fused HIP kernel (amax or min/max, scale, divide, round, nibble pack),
+symmetric or asymmetric.  The reference's intermediate dequantise / re-quantise steps map every integer
 code back to itself for all reachable (code, bf16 scale) pairs - the test-suite re-proves this by
-exhaustion - so they are not executed.  The asymmetric branch runs the HIP fake-quant kernel and then
-the reference's own chain of tensor ops on the GPU.
+exhaustion - so they are not executed there; where they are not the identity (scales of 2^121 and above,
+asymmetric codes above 17) the kernels run them literally.  Other dtypes, strides and group sizes run the HIP
+fake-quant kernel and then the reference's own chain of tensor ops on the GPU.
 """
 
 from __future__ import annotations
@@ -107,6 +108,14 @@ def _check_pack_input(weight: torch.Tensor, group_size: int, what: str) -> None:
         raise RuntimeError(f"block_m * block_n ({group_size}) must be divisible by 32. But got a 1x{group_size} block.")
 
 
+def _pack_zero_points_awq(zp: torch.Tensor) -> torch.Tensor:
+    """[M, G] zero points -> int32 [G, M/8]: transposed, eight row-consecutive values per word in the nibble
+    order 0,4,1,5,2,6,3,7 (convert_hf_to_int4_direct.py:134-141)."""
+    z = zp.t().contiguous().to(torch.float32).to(torch.int32)
+    awq_order = torch.tensor([0, 4, 1, 5, 2, 6, 3, 7], device=z.device) * 4
+    return (z.reshape(-1, z.shape[1] // 8, 8) << awq_order).sum(dim=-1).to(torch.int32)
+
+
 def pack_layer(weight: torch.Tensor, group_size: int, sym: bool = True):
     """-> (weight_packed int32 [M, N/8], weight_scale [M, N/group_size] in weight dtype,
     packed_zero_point int32 [N/group_size, M/8] or None).  convert_hf_to_int4_direct.py:123-153."""
@@ -123,6 +132,19 @@ def pack_layer(weight: torch.Tensor, group_size: int, sym: bool = True):
             _lib.check(rc, "pack_layer")
         return packed, scale, None
 
+    if (not sym and weight.dtype == torch.bfloat16 and weight.stride(1) == 1 and group_size in (32, 64, 128)
+            and weight.stride(0) % 8 == 0 and weight.data_ptr() % 16 == 0 and M and N):
+        # fused asymmetric quantise + pack; only the (small) zero-point tensor goes through tensor ops
+        packed = torch.empty((M, N // 8), dtype=torch.int32, device=weight.device)
+        scale = torch.empty((M, N // group_size), dtype=torch.bfloat16, device=weight.device)
+        zp = torch.empty_like(scale)
+        with torch.cuda.device(weight.device):
+            rc = _lib.load().wq_int4_group_quant_pack_asym(weight.data_ptr(), M, N, weight.stride(0), int(group_size),
+                                                           packed.data_ptr(), scale.data_ptr(), zp.data_ptr(),
+                                                           _lib.stream_ptr(weight.device))
+        _lib.check(rc, "pack_layer")
+        return packed, scale, _pack_zero_points_awq(zp)
+
     # general form: HIP fake-quant kernel, then the reference's tensor-op chain on the GPU
     G = N // group_size
     q, scale, zp = fake_int4_quant_cuda(weight, (1, group_size), sym)
@@ -135,9 +157,7 @@ def pack_layer(weight: torch.Tensor, group_size: int, sym: bool = True):
         zp = packed_zp = None
     else:
         zp = zp.view(M, -1)
-        z = zp.t().contiguous().to(torch.float32).to(torch.int32)
-        awq_order = torch.tensor([0, 4, 1, 5, 2, 6, 3, 7], device=z.device) * 4
-        packed_zp = (z.reshape(-1, z.shape[1] // 8, 8) << awq_order).sum(dim=-1).to(torch.int32)
+        packed_zp = _pack_zero_points_awq(zp)
     codes = quantize(deq, scale, zp, torch.int8 if sym else torch.uint8)
     return pack_to_int32(codes, 4, sym=sym), scale, packed_zp
 

@@ -158,6 +158,58 @@ def test_pack_layer_asym(cuda, shape, gs):
     assert torch.equal(p.cpu(), po) and I.same_bits(s.cpu(), so) and torch.equal(z.cpu(), zo)
 
 
+def _check_pack_asym(w, cuda, gs=128, view=None):
+    wg = w.to(cuda)
+    if view is not None:
+        wg, w = view(wg), view(w).contiguous()
+    p, s, z = slime_amd.pack_layer(wg, gs, False)
+    po, so, zo = C.int4_pack_layer(w, gs, False)
+    nbad = int((p.cpu() != po).sum())
+    assert nbad == 0, f"{nbad} packed-word mismatches"
+    assert I.same_bits(s.cpu(), so) and torch.equal(z.cpu(), zo)
+
+
+@pytest.mark.parametrize("shape,gs", [((768, 2048), 128), ((2048, 768), 128), ((40, 7168), 128), ((64, 96), 32),
+                                      ((336, 1024), 64), ((1000, 2560), 128)])
+def test_pack_layer_asym_fused(cuda, shape, gs):
+    w = I.weights(*shape, seed=shape[1] + 1, outlier_p=0.01)
+    w[0, :gs] = 0
+    _check_pack_asym(w, cuda, gs)
+
+
+def test_pack_layer_asym_one_sided_groups_and_extremes(cuda):
+    # all-positive / all-negative groups give codes far above 15 (the reference packs them unmasked), huge values
+    # give scales where the dequantise / re-quantise chain is not the identity, tiny ones hit the 1e-5 floor
+    rows = [I.weights(8, 1024, seed=1).abs() + 0.5, -(I.weights(8, 1024, seed=2).abs()) - 0.25,
+            I.near_max_block(8, 1024, seed=3, amax=3.0e38), I.near_max_block(8, 1024, seed=4, amax=1.0e37).abs(),
+            I.subnormal_block(8, 1024, seed=5), I.weights(8, 1024, seed=6, std=1e-6),
+            torch.zeros(8, 1024, dtype=torch.bfloat16), -torch.zeros(8, 1024, dtype=torch.bfloat16),
+            I.weights(8, 1024, seed=7) + 3.0]
+    _check_pack_asym(torch.cat(rows), cuda)
+
+
+def test_pack_layer_asym_every_bf16_value(cuda):
+    vals = I.finite_bf16_values()
+    g = I.gen(23)
+    rows = []
+    for ab in torch.randint(0x3000, 0x7F80, (12,), generator=g).tolist() + [0x3728, 0x7F7F, 0x7C80]:
+        amax = torch.tensor([ab], dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+        x = vals[vals.abs() <= amax]
+        x = torch.cat([x, torch.zeros((-x.numel()) % 1024, dtype=torch.bfloat16)]).view(-1, 128)
+        x[:, 0] = amax
+        x[:, 1] = -amax
+        rows.append(x.reshape(-1, 1024))
+    w = torch.cat(rows)
+    w = w[: w.shape[0] // 8 * 8]
+    _check_pack_asym(w, cuda)
+
+
+def test_pack_layer_asym_strided_rows(cuda):
+    w = I.weights(64, 1536, seed=9)
+    _check_pack_asym(w, cuda, 128, view=lambda t: t[:, 256:1280])
+    _check_pack_asym(w, cuda, 128, view=lambda t: t[::2])
+
+
 def test_pack_plan_moe_experts(cuda):
     # Qwen3-30B-A3B expert shapes: 8 experts x {gate, up [768,2048], down [2048,768]} in one launch
     ws = []

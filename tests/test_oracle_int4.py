@@ -187,6 +187,22 @@ def test_pack_layer_sym_equals_direct_formula():
     assert torch.equal(p, want) and I.same_bits(s, s2)
 
 
+def test_asym_dequant_requant_is_identity_on_small_codes():
+    # the asymmetric chain of pack_layer: bf16(q - z) * s -> / s -> + z -> clamp to uint8 -> round, all in bf16, over
+    # every code in [0, 17], every zero point and every positive bf16 scale below 2^121
+    bits = torch.arange(0x0001, 0x7C00, dtype=torch.int32)
+    sb = bits.to(torch.int16).view(torch.bfloat16)
+    for q in range(18):
+        for z in range(16):
+            qv, zv = torch.full_like(sb, float(q)), torch.full_like(sb, float(z))
+            r = ((qv - zv) * sb) / sb + zv
+            assert (torch.round(torch.clamp(r, 0, 255)).to(torch.uint8) == q).all(), (q, z)
+    # and it is not the identity everywhere above: the kernels must run the chain there
+    big = torch.tensor([0x7F00], dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+    r = ((torch.full_like(big, 15.0) - 0) * big) / big
+    assert not (torch.round(torch.clamp(r, 0, 255)) == 15).all()
+
+
 def test_pack_layer_extreme_scales_where_the_chain_is_not_the_identity():
     # bf16(7 * scale) overflows to infinity for scales near 2^125: the chain then yields code 127 and the
     # packing sum carries into neighbouring nibbles.  Both oracles must agree on that corner too.
