@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define WQ_ABI_VERSION 4
+#define WQ_ABI_VERSION 5
 
 enum {
     WQ_OK = 0,
@@ -42,7 +42,7 @@ enum {
 };
 
 /* element type selectors */
-enum { WQ_DTYPE_BF16 = 0, WQ_DTYPE_F32 = 1 };
+enum { WQ_DTYPE_BF16 = 0, WQ_DTYPE_F32 = 1, WQ_DTYPE_F16 = 2 };
 
 /* FP8 block quant arithmetic.
  * WQ_FP8_MODE_TORCH  : amax clamped at bf16(1e-12) in bf16, scale = f32(amax)/448, q = f32(x)/scale
@@ -94,6 +94,13 @@ typedef struct wq_fp8_quant_desc {
 
 int wq_fp8_block_quant_grouped(const wq_fp8_quant_desc *descs, const int64_t *tile_start, int n_desc,
                                int64_t total_tiles, int bm, int bn, int mode, void *stream);
+
+/* wq_fp8_block_quant for bf16, fp16 or fp32 weights (`dtype` = WQ_DTYPE_*): the reference functions take any
+ * floating dtype - block_fp8 computes amax and the 1e-12 floor in the weight dtype (the floor rounds to 0 in
+ * fp16), the Triton cast converts to fp32 on load (fp8_kernel.py:50).  A plain two-pass kernel: bf16 weights
+ * should go through wq_fp8_block_quant, which gives the same bytes several times faster. */
+int wq_fp8_block_quant_any(const void *x, int dtype, int64_t M, int64_t N, int64_t sx_m, int64_t sx_n,
+                           void *y, int64_t sy_m, float *s, int bm, int bn, int mode, void *stream);
 
 /* Per-row and per-tensor scaling: channel_fp8 / tensor_fp8, tools/convert_hf_to_fp8.py:78-91, and the
  * per-tensor branch of _quantize_param, quantizer_fp8.py:112-117.  s has M entries (row) or 1 (tensor).

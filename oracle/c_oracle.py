@@ -32,6 +32,7 @@ def lib() -> ctypes.CDLL:
             build()
         L = ctypes.CDLL(_SO)
         L.wqo_fp8_block_quant.argtypes = [_vp, _i64, _i64, _i64, _i64, _i64, _i64, _int, _vp, _vp]
+        L.wqo_fp8_block_quant_any.argtypes = [_vp, _int, _i64, _i64, _i64, _i64, _i64, _i64, _int, _vp, _vp]
         L.wqo_fp8_channel_quant.argtypes = [_vp, _i64, _i64, _i64, _i64, _int, _vp, _vp]
         L.wqo_fp8_tensor_quant.argtypes = [_vp, _i64, _i64, _i64, _i64, _int, _vp, _vp]
         L.wqo_fp8_block_dequant.argtypes = [_vp, _vp, _i64, _i64, _i64, _int, _vp]
@@ -85,11 +86,16 @@ def f32_to_bf16(x: torch.Tensor) -> torch.Tensor:
 
 def fp8_block_quant(w: torch.Tensor, block_size=(128, 128), mode: int = 0):
     """-> (uint8 [M,N] holding e4m3fn codes, float32 [cdiv(M,bm), cdiv(N,bn)])."""
-    assert _cpu(w).dtype == torch.bfloat16 and w.dim() == 2
+    assert _cpu(w).dim() == 2
     M, N = w.shape
     bm, bn = int(block_size[0]), int(block_size[1])
     y = torch.empty(M, N, dtype=torch.uint8)
     s = torch.empty(_cdiv(M, bm), _cdiv(N, bn), dtype=torch.float32)
+    if w.dtype != torch.bfloat16:
+        sel = {torch.float32: 1, torch.float16: 2}[w.dtype]
+        _check(lib().wqo_fp8_block_quant_any(w.data_ptr(), sel, M, N, w.stride(0), w.stride(1), bm, bn, mode,
+                                             y.data_ptr(), s.data_ptr()), "fp8_block_quant")
+        return y, s
     _check(lib().wqo_fp8_block_quant(w.data_ptr(), M, N, w.stride(0), w.stride(1), bm, bn, mode,
                                      y.data_ptr(), s.data_ptr()), "fp8_block_quant")
     return y, s

@@ -190,6 +190,64 @@ static inline uint8_t quant_elem_mode1(float x, float s_inv)
 /* x: bf16 bits, element (i,j) at x[i*sx_m + j*sx_n].  y: [M,N] contiguous bytes.
  * s: [cdiv(M,bm), cdiv(N,bn)] contiguous fp32.  Out-of-range elements of an edge block
  * count as +0.0 (F.pad value=0.0 / masked load other=0.0). */
+/* fp16 bits -> fp32 (exact) */
+WQO_API float wqo_f16_to_f32(uint16_t h)
+{
+    uint32_t sign = (uint32_t)(h & 0x8000u) << 16, e = (h >> 10) & 0x1Fu, m = h & 0x3FFu;
+    if (e == 0x1F) return u2f(sign | 0x7F800000u | (m << 13));
+    if (e == 0) {
+        float v = (float)m * 0x1p-24f;          /* subnormal: m * 2^-24, exact */
+        return sign ? -v : v;
+    }
+    return u2f(sign | ((e + 112u) << 23) | (m << 13));
+}
+
+/* element (any of the dtypes the reference functions take) -> fp32, exact.  dtype: 0 bf16, 1 fp32, 2 fp16 */
+static inline float load_any(const void *x, int dtype, int64_t off)
+{
+    if (dtype == 1) return ((const float *)x)[off];
+    if (dtype == 2) return wqo_f16_to_f32(((const uint16_t *)x)[off]);
+    return wqo_bf16_to_f32(((const uint16_t *)x)[off]);
+}
+
+/* clamp(min=1e-12) happens in the weight dtype: the bound is 1e-12 rounded to that dtype - 0x2B8D in bf16,
+ * 0 in fp16 (1e-12 is below half the smallest fp16 subnormal), 1e-12f in fp32. */
+static inline float torch_floor(int dtype)
+{ return dtype == 1 ? 1e-12f : dtype == 2 ? 0.0f : wqo_bf16_to_f32(BF16_1EM12_BITS); }
+
+WQO_API int wqo_fp8_block_quant_any(const void *x, int dtype, int64_t M, int64_t N, int64_t sx_m, int64_t sx_n,
+                                    int64_t bm, int64_t bn, int mode, uint8_t *y, float *s)
+{
+    if (M < 0 || N < 0 || bm <= 0 || bn <= 0 || mode < 0 || mode > 2 || dtype < 0 || dtype > 2) return 1;
+    int64_t nt = cdiv(M, bm), kt = cdiv(N, bn);
+    volatile float inv448 = 1.0f / FP8_MAX;
+#pragma omp parallel for schedule(static)
+    for (int64_t bi = 0; bi < nt; ++bi) {
+        for (int64_t bj = 0; bj < kt; ++bj) {
+            int64_t r0 = bi * bm, r1 = r0 + bm < M ? r0 + bm : M;
+            int64_t c0 = bj * bn, c1 = c0 + bn < N ? c0 + bn : N;
+            float amax = 0.0f;
+            for (int64_t i = r0; i < r1; ++i)
+                for (int64_t j = c0; j < c1; ++j)
+                    amax = max_nanprop(amax, fabsf(load_any(x, dtype, i * sx_m + j * sx_n)));
+            float scale, s_inv = 0.0f;
+            if (mode == 1) { scale = scale_from_amax_mode1(amax); s_inv = 1.0f / scale; }
+            else {
+                float a = amax;
+                if (a == a && a < torch_floor(dtype)) a = torch_floor(dtype);
+                scale = mode == 2 ? a * inv448 : a / FP8_MAX;
+            }
+            s[bi * kt + bj] = scale;
+            for (int64_t i = r0; i < r1; ++i)
+                for (int64_t j = c0; j < c1; ++j) {
+                    float v = load_any(x, dtype, i * sx_m + j * sx_n);
+                    y[i * N + j] = mode != 1 ? quant_elem_mode0(v, scale) : quant_elem_mode1(v, s_inv);
+                }
+        }
+    }
+    return 0;
+}
+
 WQO_API int wqo_fp8_block_quant(const uint16_t *x, int64_t M, int64_t N, int64_t sx_m, int64_t sx_n,
                                 int64_t bm, int64_t bn, int mode, uint8_t *y, float *s)
 {

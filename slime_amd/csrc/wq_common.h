@@ -159,6 +159,16 @@ __device__ __forceinline__ float row16_min_f32(float v)
     v = fminf(v, u2f(dpp_u32<0x140>(f2u(v))));
     return v;
 }
+// NaN-propagating fp32 maximum over the wavefront
+__device__ __forceinline__ float wave64_max_nanprop_f32(float v)
+{
+#pragma unroll
+    for (int m = 1; m < 64; m <<= 1) {
+        const float o = u2f((uint32_t)__shfl_xor((int)f2u(v), m));
+        v = (v != v || o != o) ? __builtin_nanf("") : fmaxf(v, o);
+    }
+    return v;
+}
 __device__ __forceinline__ uint32_t wave64_max_u32(uint32_t v)
 {
     v = row16_max_u32(v);

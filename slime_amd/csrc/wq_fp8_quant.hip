@@ -388,6 +388,87 @@ __global__ __launch_bounds__(256) void fp8_tensor_apply_vec_kernel(const uint16_
     }
 }
 
+// ---- block quant of fp16 / fp32 weights --------------------------------------------------------------
+// The reference functions take any floating dtype; checkpoints and weight-sync buckets are bf16, so these
+// dtypes get a plain two-pass tile kernel (second pass from L2) with the literal arithmetic: amax in the input
+// dtype, the 1e-12 floor rounded to that dtype (0 for fp16: an all-zero fp16 block divides 0 by 0 in the
+// reference, and here), fp32 from there on.
+template <typename T> __device__ __forceinline__ float load_any(const void* p, int64_t off);
+template <> __device__ __forceinline__ float load_any<float>(const void* p, int64_t off) { return ((const float*)p)[off]; }
+template <> __device__ __forceinline__ float load_any<_Float16>(const void* p, int64_t off)
+{
+    return (float)((const _Float16*)p)[off];
+}
+template <> __device__ __forceinline__ float load_any<uint16_t>(const void* p, int64_t off)
+{
+    return u2f((uint32_t)((const uint16_t*)p)[off] << 16);
+}
+template <typename T> __device__ __forceinline__ float torch_floor_1em12();
+template <> __device__ __forceinline__ float torch_floor_1em12<float>() { return 1e-12f; }
+template <> __device__ __forceinline__ float torch_floor_1em12<_Float16>() { return 0.0f; }
+template <> __device__ __forceinline__ float torch_floor_1em12<uint16_t>() { return u2f(kBf16Floor1em12 << 16); }
+
+template <typename T, int MODE>
+__global__ __launch_bounds__(256) void fp8_block_quant_any_kernel(const void* __restrict__ x, int64_t M, int64_t N,
+                                                                 int64_t sx_m, int64_t sx_n, uint8_t* __restrict__ y,
+                                                                 int64_t sy_m, float* __restrict__ s, int bm, int bn,
+                                                                 int64_t total_tiles)
+{
+    __shared__ float lds[4];
+    const int64_t tile = (int64_t)blockIdx.x + (int64_t)blockIdx.y * gridDim.x;
+    if (tile >= total_tiles) return;
+    const int64_t kt = (N + bn - 1) / bn;
+    const int64_t tm = tile / kt, tn = tile - tm * kt;
+    const int64_t r0 = tm * bm, c0 = tn * bn;
+    const int rows = (int)min((int64_t)bm, M - r0), cols = (int)min((int64_t)bn, N - c0);
+    const int n = rows * cols;
+    // NaN-propagating maximum of |x| (torch.max; the Triton reduction is not specified for NaN)
+    float m = 0.0f;
+    bool nan = false;
+    for (int e = threadIdx.x; e < n; e += 256) {
+        const int i = e / cols, j = e - i * cols;
+        const float v = fabsf(load_any<T>(x, (r0 + i) * sx_m + (c0 + j) * sx_n));
+        nan = nan || v != v;
+        m = fmaxf(m, v);
+    }
+    m = nan ? __builtin_nanf("") : m;
+    m = wave64_max_nanprop_f32(m);
+    if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6] = m;
+    __syncthreads();
+    m = lds[0];
+#pragma unroll
+    for (int w = 1; w < 4; ++w) m = (m != m || lds[w] != lds[w]) ? __builtin_nanf("") : fmaxf(m, lds[w]);
+    float scale, inv = 0.0f;
+    if (MODE == WQ_FP8_MODE_TRITON) {
+        scale = (m != m ? m : fmaxf(m, 1e-10f)) / kFp8Max;
+        inv = 1.0f / scale;
+    } else {
+        const float a = m != m ? m : fmaxf(m, torch_floor_1em12<T>());
+        scale = MODE == WQ_FP8_MODE_TORCH_DEVICE ? a * (1.0f / kFp8Max) : a / kFp8Max;
+    }
+    if (threadIdx.x == 0) s[tile] = scale;
+    for (int e = threadIdx.x; e < n; e += 256) {
+        const int i = e / cols, j = e - i * cols;
+        const float xv = load_any<T>(x, (r0 + i) * sx_m + (c0 + j) * sx_n);
+        y[(r0 + i) * sy_m + (c0 + j)] = (uint8_t)(MODE == WQ_FP8_MODE_TRITON ? fp8_elem_exact_triton(xv, inv)
+                                                                             : fp8_elem_exact_torch(xv, scale));
+    }
+}
+
+template <typename T>
+static void launch_block_quant_any(const void* x, int64_t M, int64_t N, int64_t sx_m, int64_t sx_n, uint8_t* y,
+                                   int64_t sy_m, float* s, int bm, int bn, int mode, hipStream_t st)
+{
+    const int64_t tiles = cdiv64(M, bm) * cdiv64(N, bn);
+    const dim3 g = grid_for_items(tiles);
+    if (mode == WQ_FP8_MODE_TORCH)
+        fp8_block_quant_any_kernel<T, WQ_FP8_MODE_TORCH><<<g, 256, 0, st>>>(x, M, N, sx_m, sx_n, y, sy_m, s, bm, bn, tiles);
+    else if (mode == WQ_FP8_MODE_TORCH_DEVICE)
+        fp8_block_quant_any_kernel<T, WQ_FP8_MODE_TORCH_DEVICE><<<g, 256, 0, st>>>(x, M, N, sx_m, sx_n, y, sy_m, s, bm, bn, tiles);
+    else
+        fp8_block_quant_any_kernel<T, WQ_FP8_MODE_TRITON><<<g, 256, 0, st>>>(x, M, N, sx_m, sx_n, y, sy_m, s, bm, bn, tiles);
+}
+
 static bool known_mode(int mode)
 {
     return mode == WQ_FP8_MODE_TORCH || mode == WQ_FP8_MODE_TRITON || mode == WQ_FP8_MODE_TORCH_DEVICE;
@@ -503,6 +584,21 @@ WQ_EXPORT int wq_fp8_tensor_quant(const void* x, int64_t M, int64_t N, int64_t s
     WQ_LAUNCH_CHECK();
     fp8_tensor_apply_kernel<<<blocks, 256, 0, st>>>((const uint16_t*)x, M, N, sx_m, sx_n, (uint8_t*)y, sy_m, s,
                                                    workspace, mode);
+    WQ_LAUNCH_CHECK();
+    return WQ_OK;
+}
+
+WQ_EXPORT int wq_fp8_block_quant_any(const void* x, int dtype, int64_t M, int64_t N, int64_t sx_m, int64_t sx_n, void* y,
+                                     int64_t sy_m, float* s, int bm, int bn, int mode, void* stream)
+{
+    if (dtype != WQ_DTYPE_BF16 && dtype != WQ_DTYPE_F32 && dtype != WQ_DTYPE_F16) return WQ_ERR_MODE;
+    int rc = check_desc_host(x, M, N, y, s, bm, bn, mode);
+    if (rc) return rc;
+    if (M == 0 || N == 0) return WQ_OK;
+    hipStream_t st = (hipStream_t)stream;
+    if (dtype == WQ_DTYPE_F32) launch_block_quant_any<float>(x, M, N, sx_m, sx_n, (uint8_t*)y, sy_m, s, bm, bn, mode, st);
+    else if (dtype == WQ_DTYPE_F16) launch_block_quant_any<_Float16>(x, M, N, sx_m, sx_n, (uint8_t*)y, sy_m, s, bm, bn, mode, st);
+    else launch_block_quant_any<uint16_t>(x, M, N, sx_m, sx_n, (uint8_t*)y, sy_m, s, bm, bn, mode, st);
     WQ_LAUNCH_CHECK();
     return WQ_OK;
 }

@@ -38,8 +38,18 @@ def _check_weight(w: torch.Tensor, what: str) -> None:
         raise TypeError(f"{what}: only bfloat16 weights are supported (got {w.dtype})")
 
 
+_OTHER_FLOAT_DTYPES = {torch.float16: _lib.DTYPE_F16, torch.float32: _lib.DTYPE_F32}
+
+
 def _block_quant(w: torch.Tensor, bm: int, bn: int, mode: int, what: str):
-    _check_weight(w, what)
+    """bf16 weights take the bandwidth-tuned kernel; fp16 / fp32 weights, which the reference functions also accept,
+    a plain one with the reference's arithmetic for that dtype."""
+    if w.dtype in _OTHER_FLOAT_DTYPES:
+        _lib.require_gpu(w, what)
+        if w.dim() != 2:
+            raise ValueError(f"{what}: expected a 2-D weight, got shape {tuple(w.shape)}")
+    else:
+        _check_weight(w, what)
     if bm <= 0 or bn <= 0:
         raise ValueError(f"{what}: block size must be positive, got {(bm, bn)}")
     M, N = w.shape
@@ -47,8 +57,13 @@ def _block_quant(w: torch.Tensor, bm: int, bn: int, mode: int, what: str):
     s = torch.empty((ceildiv(M, bm), ceildiv(N, bn)), dtype=torch.float32, device=w.device)
     if M and N:
         with torch.cuda.device(w.device):
-            rc = _lib.load().wq_fp8_block_quant(w.data_ptr(), M, N, w.stride(0), w.stride(1), q.data_ptr(), N,
-                                                s.data_ptr(), bm, bn, mode, _lib.stream_ptr(w.device))
+            if w.dtype == torch.bfloat16:
+                rc = _lib.load().wq_fp8_block_quant(w.data_ptr(), M, N, w.stride(0), w.stride(1), q.data_ptr(), N,
+                                                    s.data_ptr(), bm, bn, mode, _lib.stream_ptr(w.device))
+            else:
+                rc = _lib.load().wq_fp8_block_quant_any(w.data_ptr(), _OTHER_FLOAT_DTYPES[w.dtype], M, N, w.stride(0),
+                                                        w.stride(1), q.data_ptr(), N, s.data_ptr(), bm, bn, mode,
+                                                        _lib.stream_ptr(w.device))
         _lib.check(rc, what)
     return q, s
 

@@ -384,3 +384,41 @@ def test_channel_quant_every_bf16_value(cuda):
             q, s = slime_amd.channel_fp8(w.to(cuda))
         qo, so = C.fp8_channel_quant(w, mode)
         assert torch.equal(_codes(q), qo) and torch.equal(_bits32(s), _bits32(so))
+
+
+# ------------------------------------------------------------------ fp16 / fp32 weights
+
+@pytest.mark.parametrize("dt", [torch.float16, torch.float32])
+@pytest.mark.parametrize("mode", [0, 1, 2])
+def test_block_quant_other_dtypes(cuda, dt, mode):
+    g = torch.Generator().manual_seed(4)
+    for shape in ((256, 384), (300, 200), (7, 7168), (129, 127), (1024, 2560)):
+        w = I.zero_blocks(I.weights(*shape, seed=sum(shape)), 0.2, seed=1)
+        x = (w.float() * (1 + 1e-3 * torch.randn(shape, generator=g))).to(dt)
+        for view in (lambda t: t, lambda t: t.t(), lambda t: t[::2, 1:]):
+            xc, xg = view(x), view(x.to(cuda))
+            if mode == 1:
+                q, s = slime_amd.blockwise_cast_to_fp8_triton(xg, (128, 128))
+            else:
+                with slime_amd.torch_arithmetic(ARITH[mode]):
+                    q, s = slime_amd.block_fp8(xg, (128, 128))
+            qo, so = C.fp8_block_quant(xc, (128, 128), mode)
+            qc = _codes(q)
+            nan = (qo & 0x7F) == 0x7F
+            assert torch.equal((qc & 0x7F) == 0x7F, nan) and torch.equal(qc[~nan], qo[~nan])
+            assert torch.equal(_bits32(s), _bits32(so))
+
+
+@pytest.mark.parametrize("dt", [torch.float16, torch.float32])
+def test_block_quant_other_dtypes_match_torch_ops_on_the_gpu(cuda, dt):
+    g = torch.Generator().manual_seed(5)
+    w = I.weights(512, 640, seed=6)
+    x = (w.float() * (1 + 1e-3 * torch.randn(512, 640, generator=g))).to(dt).to(cuda)
+    q, s = slime_amd.block_fp8(x, (128, 128))
+    qr, sr = T.block_fp8_ref(x, (128, 128))
+    assert torch.equal(_bits32(s), _bits32(sr)) and torch.equal(_codes(q), _codes(qr))
+
+
+def test_int8_weights_are_refused(cuda):
+    with pytest.raises(TypeError):
+        slime_amd.block_fp8(torch.zeros(128, 128, dtype=torch.int8, device=cuda), (128, 128))

@@ -76,3 +76,12 @@ def test_weight_dequant_matches_triton_on_this_gpu(cuda, shape):
     assert I.same_bits(got.cpu(), T.weight_dequant_triton_ref(x, s).cpu())
     got32 = slime_amd.weight_dequant(x, s)
     assert I.same_bits(got32.cpu(), T.weight_dequant_triton_ref(x, s, out_dtype=torch.float32).cpu())
+
+
+@pytest.mark.parametrize("dt", [torch.float16, torch.float32])
+def test_blockwise_cast_other_dtypes_match_triton(cuda, dt):
+    T = _triton_ref()
+    g = torch.Generator().manual_seed(8)
+    w = I.zero_blocks(I.weights(300, 1000, seed=9), 0.2, seed=1)
+    x = (w.float() * (1 + 1e-3 * torch.randn(300, 1000, generator=g))).to(dt).to(cuda)
+    _same(*slime_amd.blockwise_cast_to_fp8_triton(x, (128, 128)), *T.blockwise_cast_triton_ref(x, (128, 128)))

@@ -325,3 +325,49 @@ def test_tensor_fp8_rounds_quotient_to_bf16_first():
             twice += want != e4m3_code(rn_e4m3(min(max(q32, Fraction(-448)), Fraction(448))), negative_zero=v < 0)
     # the double rounding is observable on this sample (otherwise the test would not pin it)
     assert twice > 0
+
+
+# ------------------------------------------------------------------ fp16 / fp32 weights
+
+def _as_dtype(w, dt, seed):
+    g = torch.Generator().manual_seed(seed)
+    return (w.float() * (1 + 1e-3 * torch.randn(w.shape, generator=g))).to(dt)
+
+
+@pytest.mark.parametrize("dt", [torch.float16, torch.float32])
+@pytest.mark.parametrize("mode", [0, 1, 2])
+@pytest.mark.parametrize("shape", [(256, 384), (300, 200), (7, 7168), (129, 127)])
+def test_c_equals_torch_block_quant_other_dtypes(dt, mode, shape):
+    x = _as_dtype(I.zero_blocks(I.weights(*shape, seed=sum(shape)), 0.2, seed=1), dt, 3)
+    for view in (lambda t: t, lambda t: t.t()):
+        q, s = C.fp8_block_quant(view(x), (128, 128), mode)
+        qr, sr = T.blockwise_cast_ref(view(x), (128, 128)) if mode == 1 else T.block_fp8_ref(view(x), (128, 128), mode == 2)
+        qr = _codes(qr)
+        nan = (qr & 0x7F) == 0x7F
+        assert torch.equal((q & 0x7F) == 0x7F, nan) and torch.equal(q[~nan], qr[~nan])
+        assert torch.equal(_bits32(s), _bits32(sr))
+        # an all-zero fp16 block divides 0 by 0 in the torch formulation (its 1e-12 floor rounds to 0 in fp16)
+        if not (dt == torch.float16 and mode != 1):
+            assert not nan.any()
+        elif shape == (300, 200):
+            assert nan.any()
+
+
+def test_fp16_conversion_is_exact_for_every_value():
+    bits = torch.arange(65536, dtype=torch.int32).to(torch.int16)
+    x = bits.view(torch.float16).view(-1, 64)
+    finite = x.float().abs() < float("inf")
+    x = torch.where(finite, x, torch.zeros_like(x))
+    # mode 1 with a huge block: scale = amax / 448 with amax = 65504, codes = e4m3(x * (1 / scale))
+    q, s = C.fp8_block_quant(x, (1024, 64), 1)
+    qr, sr = T.blockwise_cast_ref(x, (1024, 64))
+    assert torch.equal(q, _codes(qr)) and torch.equal(_bits32(s), _bits32(sr))
+
+
+def test_fp32_floor_is_fp32_1e_12():
+    w = torch.zeros(4, 4, dtype=torch.float32)
+    w[0, 0] = 3e-13
+    _, s0 = C.fp8_block_quant(w, (4, 4), 0)
+    assert Fraction(s0.item()) == rn_f32(rn_f32(Fraction(1, 10 ** 12)) / 448)
+    _, s2 = C.fp8_block_quant(w, (4, 4), 2)
+    assert Fraction(s2.item()) == rn_f32(rn_f32(Fraction(1, 10 ** 12)) * rn_f32(Fraction(1, 448)))
