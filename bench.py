@@ -113,6 +113,41 @@ def bench_fp8_quant(dev, steps, warmup):
     }
 
 
+def bench_fp8_quant_moe(dev, steps, warmup, layers):
+    """Block-FP8 quant of every linear weight of a Qwen3-30B-A3B-shaped state dict (48 layers: 128 experts x
+    gate/up [768,2048], down [2048,768]; attention q [4096,2048], k/v [512,2048], o [2048,4096]), one grouped launch."""
+    import torch
+
+    import slime_amd
+    from oracle import c_oracle
+
+    experts = 128
+    weights = []
+    for _ in range(layers):
+        gate = _gen_bf16((experts, 768, 2048), dev, outliers=True)
+        up = _gen_bf16((experts, 768, 2048), dev, outliers=True)
+        down = _gen_bf16((experts, 2048, 768), dev, outliers=True)
+        for e in range(experts):
+            weights += [gate[e], up[e], down[e]]
+        weights += [_gen_bf16(sh, dev) for sh in ((4096, 2048), (512, 2048), (512, 2048), (2048, 4096))]
+    plan = slime_amd.Fp8QuantPlan(weights, (128, 128))
+    wall_ms, ev_ms, ev_min = _time_launches(plan.run, steps, warmup)
+    elements = sum(w.numel() for w in weights)
+    algo_bytes = 3 * elements + 4 * plan.total_tiles
+    for idx in (0, 2, 385, len(weights) - 1):
+        q, s = plan.outputs[idx]
+        qo, so = c_oracle.fp8_block_quant(weights[idx].cpu().contiguous(), (128, 128), plan.mode)
+        assert torch.equal(q.cpu().view(torch.uint8), qo) and torch.equal(s.cpu().view(torch.int32), so.view(torch.int32))
+    out = {"workload": f"Qwen3-30B-A3B-shaped state dict, {layers} layers x (128 experts x gate, up [768,2048], down "
+                       "[2048,768] + q, k, v, o), block-FP8 128x128, one grouped launch",
+           "tensors": len(weights), "bf16_GB": 2 * elements / 1e9, "kernel_ms": ev_ms, "wall_ms": wall_ms,
+           "bf16_GBps": 2 * elements / ev_ms / 1e6, "algo_GBps": algo_bytes / ev_ms / 1e6,
+           "hbm_frac": algo_bytes / ev_ms / 1e6 / HBM_PEAK_GBS, "parity_tensors_checked": 4}
+    del plan, weights
+    torch.cuda.empty_cache()
+    return out
+
+
 def bench_int4_pack(dev, steps, warmup, layers):
     import torch
 
@@ -393,7 +428,7 @@ def main():
     ap.add_argument("--dequant-experts", type=int, default=256)
     ap.add_argument("--no-extras", action="store_true", help="headline workload only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
-    ap.add_argument("--only", choices=["int4", "dequant", "int4deq", "ste", "delta", "forms", "copy", "stream"], default=None,
+    ap.add_argument("--only", choices=["fp8moe", "int4", "dequant", "int4deq", "ste", "delta", "forms", "copy", "stream"], default=None,
                     help="run just one of the other legs and print its record: a kernel for profiling, the plain copy "
                          "kernel that hardware counters are calibrated against, or the host-resident streaming run "
                          "(64 x 1 GiB buckets, PCIe-bound)")
@@ -414,6 +449,9 @@ def main():
     dev = torch.device("cuda:0")
     torch.manual_seed(0)
 
+    if args.only == "fp8moe":
+        print(json.dumps(bench_fp8_quant_moe(dev, args.steps, args.warmup, args.int4_layers)))
+        return
     if args.only == "int4":
         print(json.dumps(bench_int4_pack(dev, args.steps, args.warmup, args.int4_layers)))
         return
@@ -466,6 +504,7 @@ def main():
     if not args.no_extras:
         extras = {}
         if args.int4_layers > 0:
+            extras["fp8_block_quant_moe"] = bench_fp8_quant_moe(dev, args.steps, args.warmup, args.int4_layers)
             extras["int4_group_quant_pack"] = bench_int4_pack(dev, args.steps, args.warmup, args.int4_layers)
         if args.dequant_experts > 0:
             extras["fp8_block_dequant"] = bench_fp8_dequant(dev, args.steps, args.warmup, args.dequant_experts)
