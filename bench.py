@@ -494,7 +494,7 @@ def main():
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS,
                      "traffic": _traffic_from_profile("fp8_block_quant_qwen3_4b_pmc.txt"),
-                     "kernel": "fp8_block_quant_kernel<TORCH_DEVICE, grouped>", "kernel_ms": r["kernel_ms"],
+                     "kernel": "fp8_block_quant_kernel<TORCH_DEVICE, per-tile descriptors>", "kernel_ms": r["kernel_ms"],
                      "kernel_ms_min": r["kernel_ms_min"], "algorithmic_bytes_per_launch": r["algo_bytes"]},
     }
     if not args.no_cpu:

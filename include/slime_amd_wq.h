@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define WQ_ABI_VERSION 5
+#define WQ_ABI_VERSION 7
 
 enum {
     WQ_OK = 0,
@@ -94,6 +94,13 @@ typedef struct wq_fp8_quant_desc {
 
 int wq_fp8_block_quant_grouped(const wq_fp8_quant_desc *descs, const int64_t *tile_start, int n_desc,
                                int64_t total_tiles, int bm, int bn, int mode, void *stream);
+
+/* The same launch with every tile resolved beforehand: `tiles` is a DEVICE array with one descriptor per
+ * (bm x bn) tile, moved to the tile's origin - x and y point at the tile's first element, s at the tile's scale,
+ * M and N are the rows and columns of the tensor from there on (the kernel uses min(bm, M) x min(bn, N)), strides
+ * as in the tensor.  Costs 64 bytes of table per tile and saves the per-workgroup search; meant for plans that
+ * are built once and run every weight sync. */
+int wq_fp8_block_quant_tiles(const wq_fp8_quant_desc *tiles, int64_t n_tiles, int bm, int bn, int mode, void *stream);
 
 /* wq_fp8_block_quant for bf16, fp16 or fp32 weights (`dtype` = WQ_DTYPE_*): the reference functions take any
  * floating dtype - block_fp8 computes amax and the 1e-12 floor in the weight dtype (the floor rounds to 0 in
@@ -166,6 +173,13 @@ typedef struct wq_int4_pack_desc {
 #define WQ_INT4_GROUPS_PER_WG 64
 int wq_int4_group_quant_pack_grouped(const wq_int4_pack_desc *descs, const int64_t *work_start, int n_desc,
                                      int64_t total_work, int group, void *stream);
+
+/* The same launch with the owner of every work item resolved beforehand: `items` is a DEVICE array with one
+ * descriptor per work item - x, packed and scale pointing at the item's first group, n_groups = the groups of the
+ * item (at most WQ_INT4_GROUPS_PER_WG; every item but a tensor's last has exactly that many).  Costs 32 bytes of
+ * table per 16 KiB of weights and saves the per-workgroup search; meant for plans that are built once and run
+ * every weight sync. */
+int wq_int4_group_quant_pack_items(const wq_int4_pack_desc *items, int64_t n_items, int group, void *stream);
 
 /* Asymmetric form of wq_int4_group_quant_pack (pack_layer(weight, group, sym=False),
  * tools/convert_hf_to_int4_direct.py:123-153): codes rintf(x/scale) + zero with scale = max((max-min)/15, 1e-5)

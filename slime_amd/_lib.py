@@ -15,7 +15,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libslime_amd_wq.so")
 
-ABI_VERSION = 5
+ABI_VERSION = 7
 
 # selectors (mirrors of the header's enums)
 DTYPE_BF16, DTYPE_F32, DTYPE_F16 = 0, 1, 2
@@ -33,6 +33,7 @@ SIGNATURES = {
     "wq_error_string": [_int],
     "wq_fp8_block_quant": [_vp, _i64, _i64, _i64, _i64, _vp, _i64, _vp, _int, _int, _int, _vp],
     "wq_fp8_block_quant_grouped": [_vp, _vp, _int, _i64, _int, _int, _int, _vp],
+    "wq_fp8_block_quant_tiles": [_vp, _i64, _int, _int, _int, _vp],
     "wq_fp8_block_quant_any": [_vp, _int, _i64, _i64, _i64, _i64, _vp, _i64, _vp, _int, _int, _int, _vp],
     "wq_fp8_row_quant": [_vp, _i64, _i64, _i64, _i64, _vp, _i64, _vp, _int, _vp],
     "wq_fp8_tensor_quant": [_vp, _i64, _i64, _i64, _i64, _vp, _i64, _vp, _vp, _int, _vp],
@@ -41,6 +42,7 @@ SIGNATURES = {
     "wq_int4_fake_quant": [_vp, _int, _i64, _i64, _i64, _i64, _int, _int, _int, _vp, _vp, _vp, _vp],
     "wq_int4_group_quant_pack": [_vp, _i64, _i64, _i64, _int, _vp, _vp, _vp],
     "wq_int4_group_quant_pack_grouped": [_vp, _vp, _int, _i64, _int, _vp],
+    "wq_int4_group_quant_pack_items": [_vp, _i64, _int, _vp],
     "wq_int4_group_quant_pack_asym": [_vp, _i64, _i64, _i64, _int, _vp, _vp, _vp, _vp],
     "wq_int4_dequant": [_vp, _vp, _vp, _i64, _i64, _int, _vp],
     "wq_int4_fake_quant_ste": [_vp, _vp, _i64, _i64, _int, _int, _vp],

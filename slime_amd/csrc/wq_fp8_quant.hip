@@ -150,7 +150,9 @@ __device__ __forceinline__ void quant_tile_generic(const wq_fp8_quant_desc& d, i
     }
 }
 
-template <int MODE, bool GROUPED>
+// GROUPED: 0 = one tensor in the kernel arguments, 1 = descriptor array + prefix sums (the owner of a tile is
+// searched), 2 = one descriptor per tile, already moved to the tile's origin (a single scalar load, no search)
+template <int MODE, int GROUPED>
 __global__ __launch_bounds__(kTileThreads) void fp8_block_quant_kernel(const Fp8QuantArgs a, const int64_t total_tiles)
 {
     __shared__ __attribute__((aligned(16))) uint32_t lds[kRowSlots];
@@ -160,14 +162,17 @@ __global__ __launch_bounds__(kTileThreads) void fp8_block_quant_kernel(const Fp8
 
     wq_fp8_quant_desc d;
     int64_t local = tile;
-    if (GROUPED) {
+    if (GROUPED == 1) {
         const int di = find_owner(a.tile_start, a.n_desc, tile, total_tiles);
         d = a.descs[di];
         local = tile - a.tile_start[di];
+    } else if (GROUPED == 2) {
+        d = a.descs[tile];      // M, N: what is left of the tensor from this tile's origin; s: this tile's slot
+        local = 0;
     } else {
         d = a.d;
     }
-    const int kt = (int)((d.N + a.bn - 1) / a.bn);
+    const int kt = GROUPED == 2 ? 1 : (int)((d.N + a.bn - 1) / a.bn);
     const int64_t tm = local / kt, tn = local - tm * kt;
     if (a.bm == 128 && a.bn == 128 && desc_vector_ok(d))
         quant_tile_vec128<MODE>(d, tm, tn, kt, lds);
@@ -474,7 +479,7 @@ static bool known_mode(int mode)
     return mode == WQ_FP8_MODE_TORCH || mode == WQ_FP8_MODE_TRITON || mode == WQ_FP8_MODE_TORCH_DEVICE;
 }
 
-template <bool GROUPED>
+template <int GROUPED>
 static void launch_block_quant(const Fp8QuantArgs& a, int64_t tiles, int mode, hipStream_t st)
 {
     const dim3 g = grid_for_items(tiles);
@@ -511,7 +516,7 @@ WQ_EXPORT int wq_fp8_block_quant(const void* x, int64_t M, int64_t N, int64_t sx
     a.bn = bn;
     const int64_t tiles = cdiv64(M, bm) * cdiv64(N, bn);
     hipStream_t st = (hipStream_t)stream;
-    launch_block_quant<false>(a, tiles, mode, st);
+    launch_block_quant<0>(a, tiles, mode, st);
     WQ_LAUNCH_CHECK();
     return WQ_OK;
 }
@@ -531,7 +536,7 @@ WQ_EXPORT int wq_fp8_block_quant_grouped(const wq_fp8_quant_desc* descs, const i
     a.bm = bm;
     a.bn = bn;
     hipStream_t st = (hipStream_t)stream;
-    launch_block_quant<true>(a, total_tiles, mode, st);
+    launch_block_quant<1>(a, total_tiles, mode, st);
     WQ_LAUNCH_CHECK();
     return WQ_OK;
 }
@@ -599,6 +604,23 @@ WQ_EXPORT int wq_fp8_block_quant_any(const void* x, int dtype, int64_t M, int64_
     if (dtype == WQ_DTYPE_F32) launch_block_quant_any<float>(x, M, N, sx_m, sx_n, (uint8_t*)y, sy_m, s, bm, bn, mode, st);
     else if (dtype == WQ_DTYPE_F16) launch_block_quant_any<_Float16>(x, M, N, sx_m, sx_n, (uint8_t*)y, sy_m, s, bm, bn, mode, st);
     else launch_block_quant_any<uint16_t>(x, M, N, sx_m, sx_n, (uint8_t*)y, sy_m, s, bm, bn, mode, st);
+    WQ_LAUNCH_CHECK();
+    return WQ_OK;
+}
+
+WQ_EXPORT int wq_fp8_block_quant_tiles(const wq_fp8_quant_desc* tiles, int64_t n_tiles, int bm, int bn, int mode,
+                                       void* stream)
+{
+    if (n_tiles < 0 || bm <= 0 || bn <= 0) return WQ_ERR_SHAPE;
+    if (!known_mode(mode)) return WQ_ERR_MODE;
+    if (n_tiles == 0) return WQ_OK;
+    if (!tiles) return WQ_ERR_NULL;
+    if ((int64_t)bm * bn > (1 << 30)) return WQ_ERR_TOO_LARGE;
+    Fp8QuantArgs a{};
+    a.descs = tiles;
+    a.bm = bm;
+    a.bn = bn;
+    launch_block_quant<2>(a, n_tiles, mode, (hipStream_t)stream);
     WQ_LAUNCH_CHECK();
     return WQ_OK;
 }

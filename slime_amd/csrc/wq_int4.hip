@@ -101,7 +101,9 @@ __device__ __forceinline__ uint32_t pack8_literal(const float (&x)[8], float sca
 
 // Contiguous tensors only: group g of the tensor starts at x + g*G, its packed words at
 // packed + g*L, its scale at scale[g].
-template <int L, bool GROUPED>
+// GROUPED: 0 = one tensor in the kernel arguments, 1 = descriptor array + prefix sums (the owner of a work item is
+// searched), 2 = one pre-resolved descriptor per work item (a single scalar load, no search)
+template <int L, int GROUPED>
 __global__ __launch_bounds__(256) void int4_pack_kernel(const Int4PackArgs a, const int64_t total_work)
 {
     constexpr int CL = 256 / L;              // groups per step of the workgroup
@@ -112,10 +114,13 @@ __global__ __launch_bounds__(256) void int4_pack_kernel(const Int4PackArgs a, co
     const int64_t item = xcd_chunked_item(slot, total_work, kPackItemsPerXcdRun);
     wq_int4_pack_desc d;
     int64_t local = item;
-    if (GROUPED) {
+    if (GROUPED == 1) {
         const int di = find_owner(a.work_start, a.n_desc, item, total_work);
         d = a.descs[di];
         local = item - a.work_start[di];
+    } else if (GROUPED == 2) {
+        d = a.descs[item];
+        local = 0;
     } else {
         d = a.d;
     }
@@ -439,7 +444,7 @@ static bool launch_fake_vec(const uint16_t* x, int64_t M, int64_t N, int64_t sx_
     return true;
 }
 
-template <bool GROUPED>
+template <int GROUPED>
 static int launch_pack(const Int4PackArgs& a, int64_t work, int group, hipStream_t st)
 {
     switch (group) {
@@ -468,7 +473,7 @@ WQ_EXPORT int wq_int4_group_quant_pack(const void* x, int64_t M, int64_t N, int6
     if (fast) {
         Int4PackArgs a{};
         a.d = wq_int4_pack_desc{x, packed, scale, n_groups};
-        return launch_pack<false>(a, cdiv64(n_groups, kGroupsPerWg), group, st);
+        return launch_pack<0>(a, cdiv64(n_groups, kGroupsPerWg), group, st);
     }
     int4_pack_generic_kernel<<<grid_for_items(cdiv64(n_groups, 16)), 256, 0, st>>>(
         (const uint16_t*)x, M, N, sx_m, group, (uint32_t*)packed, (uint16_t*)scale);
@@ -487,7 +492,7 @@ WQ_EXPORT int wq_int4_group_quant_pack_grouped(const wq_int4_pack_desc* descs, c
     a.descs = descs;
     a.work_start = work_start;
     a.n_desc = n_desc;
-    return launch_pack<true>(a, total_work, group, (hipStream_t)stream);
+    return launch_pack<1>(a, total_work, group, (hipStream_t)stream);
 }
 
 WQ_EXPORT int wq_int4_fake_quant(const void* x, int dtype, int64_t M, int64_t N, int64_t sx_m, int64_t sx_n, int bm,
@@ -539,4 +544,15 @@ WQ_EXPORT int wq_int4_group_quant_pack_asym(const void* x, int64_t M, int64_t N,
     else int4_pack_asym_kernel<16><<<g, 256, kFakeOccupancyPadBytes, st>>>(xp, sx_m, gpr, pp, (uint16_t*)scale, (uint16_t*)zero, n_groups, items);
     WQ_LAUNCH_CHECK();
     return WQ_OK;
+}
+
+WQ_EXPORT int wq_int4_group_quant_pack_items(const wq_int4_pack_desc* items, int64_t n_items, int group, void* stream)
+{
+    if (n_items < 0) return WQ_ERR_SHAPE;
+    if (group != 32 && group != 64 && group != 128) return WQ_ERR_UNSUPPORTED;
+    if (n_items == 0) return WQ_OK;
+    if (!items) return WQ_ERR_NULL;
+    Int4PackArgs a{};
+    a.descs = items;
+    return launch_pack<2>(a, n_items, group, (hipStream_t)stream);
 }

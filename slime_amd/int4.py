@@ -201,14 +201,23 @@ class Int4PackPlan:
             starts.append(work)
         self.total_work = work
         self.bf16_bytes = sum(2 * w.numel() for w in self.weights)
-        self._descs = torch.tensor(rows, dtype=torch.int64).to(self.device)
-        self._starts = torch.tensor(starts, dtype=torch.int64).to(self.device)
+        # one pre-resolved descriptor per work item (32 bytes per 16 KiB of weights): the kernel then needs a single
+        # scalar load instead of a search through the per-tensor prefix sums
+        per = _lib.INT4_GROUPS_PER_WG
+        desc = torch.tensor(rows, dtype=torch.int64)
+        start = torch.tensor(starts, dtype=torch.int64)
+        owner = torch.repeat_interleave(torch.arange(len(rows)), start[1:] - start[:-1])
+        local = torch.arange(work, dtype=torch.int64) - start[owner]
+        items = torch.stack([desc[owner, 0] + local * (per * self.group * 2),
+                             desc[owner, 1] + local * (per * self.group // 8 * 4),
+                             desc[owner, 2] + local * (per * 2),
+                             torch.clamp(desc[owner, 3] - local * per, max=per)], dim=1)
+        self._items = items.contiguous().to(self.device)
 
     def run(self):
         with torch.cuda.device(self.device):
-            rc = _lib.load().wq_int4_group_quant_pack_grouped(self._descs.data_ptr(), self._starts.data_ptr(),
-                                                              len(self.weights), self.total_work, self.group,
-                                                              _lib.stream_ptr(self.device))
+            rc = _lib.load().wq_int4_group_quant_pack_items(self._items.data_ptr(), self.total_work, self.group,
+                                                            _lib.stream_ptr(self.device))
         _lib.check(rc, "Int4PackPlan.run")
         return self.outputs
 

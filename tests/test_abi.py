@@ -47,6 +47,9 @@ def test_argument_validation_without_launch():
     assert lib.wq_fp8_block_quant(None, 0, 4, 4, 1, None, 4, None, 128, 128, 0, None) == 0      # empty: no-op
     assert lib.wq_fp8_block_quant_grouped(None, None, 3, 10, 128, 128, 0, None) == N_
     assert lib.wq_fp8_block_quant_grouped(None, None, 0, 0, 128, 128, 0, None) == 0
+    assert lib.wq_fp8_block_quant_tiles(None, 4, 128, 128, 0, None) == N_
+    assert lib.wq_fp8_block_quant_tiles(None, 4, 128, 128, 9, None) == M_
+    assert lib.wq_fp8_block_quant_tiles(None, 0, 128, 128, 0, None) == 0
     assert lib.wq_fp8_block_quant(None, 4, 4, 4, 1, None, 4, None, 128, 128, 2, None) == N_
     assert lib.wq_fp8_row_quant(None, -1, 4, 4, 1, None, 4, None, 0, None) == S
     assert lib.wq_fp8_row_quant(None, 4, 4, 4, 1, None, 4, None, 1, None) == M_         # no Triton row form
@@ -62,6 +65,9 @@ def test_argument_validation_without_launch():
     assert lib.wq_int4_group_quant_pack(None, 4, 100, 100, 128, None, None, None) == S
     assert lib.wq_int4_group_quant_pack(None, 4, 128, 128, 128, None, None, None) == N_
     assert lib.wq_int4_group_quant_pack_grouped(None, None, 1, 1, 96, None) == U
+    assert lib.wq_int4_group_quant_pack_items(None, 5, 128, None) == N_
+    assert lib.wq_int4_group_quant_pack_items(None, 5, 96, None) == U
+    assert lib.wq_int4_group_quant_pack_items(None, 0, 128, None) == 0
     assert lib.wq_int4_dequant(None, None, None, 4, 100, 128, None) == S
     assert lib.wq_int4_dequant(None, None, None, 4, 128, 12, None) == S
     assert lib.wq_int4_dequant(None, None, None, 4, 128, 128, None) == N_

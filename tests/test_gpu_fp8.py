@@ -422,3 +422,31 @@ def test_block_quant_other_dtypes_match_torch_ops_on_the_gpu(cuda, dt):
 def test_int8_weights_are_refused(cuda):
     with pytest.raises(TypeError):
         slime_amd.block_fp8(torch.zeros(128, 128, dtype=torch.int8, device=cuda), (128, 128))
+
+
+def test_grouped_search_entry_point(cuda):
+    # Fp8QuantPlan uses the per-tile table; the descriptor-array + prefix-sum form stays part of the C ABI
+    from slime_amd import _lib
+
+    shapes = [(4096, 2560), (300, 200), (7, 7168), (129, 127), (1024, 2560)]
+    ws = [I.zero_blocks(I.weights(*sh, seed=60 + i), 0.1, seed=i) for i, sh in enumerate(shapes)]
+    wg = [w.to(cuda) for w in ws]
+    wg[1] = wg[1].t().contiguous().t()
+    outs, rows, starts, tiles = [], [], [0], 0
+    for w in wg:
+        M, N = w.shape
+        q = torch.empty(M, N, dtype=torch.uint8, device=cuda)
+        sc = torch.empty(-(-M // 128), -(-N // 128), dtype=torch.float32, device=cuda)
+        outs.append((q, sc))
+        rows.append([w.data_ptr(), q.data_ptr(), sc.data_ptr(), M, N, w.stride(0), w.stride(1), N])
+        tiles += sc.numel()
+        starts.append(tiles)
+    descs = torch.tensor(rows, dtype=torch.int64).to(cuda)
+    st = torch.tensor(starts, dtype=torch.int64).to(cuda)
+    for mode in (0, 1, 2):
+        rc = _lib.load().wq_fp8_block_quant_grouped(descs.data_ptr(), st.data_ptr(), len(ws), tiles, 128, 128, mode,
+                                                    _lib.stream_ptr(cuda))
+        _lib.check(rc, "grouped")
+        for w, (q, sc) in zip(ws, outs):
+            qo, so = C.fp8_block_quant(w, (128, 128), mode)
+            assert torch.equal(q.cpu(), qo) and torch.equal(_bits32(sc), _bits32(so))

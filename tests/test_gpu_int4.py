@@ -376,3 +376,29 @@ def test_fake_ste_ragged_and_gradient(cuda):
     gy = torch.randn(16, 256, device=cuda).to(torch.bfloat16)
     y.backward(gy)
     assert torch.equal(x.grad, gy)                                            # straight-through: identity
+
+
+def test_grouped_search_entry_point(cuda):
+    # Int4PackPlan uses the per-item table; the descriptor-array + prefix-sum form stays part of the C ABI
+    from slime_amd import _lib
+
+    shapes = [(768, 2048), (33, 768), (1, 128), (2048, 768), (7, 7168)]
+    ws = [I.weights(*sh, seed=50 + i) for i, sh in enumerate(shapes)]
+    wg = [w.to(cuda) for w in ws]
+    outs, rows, starts, work = [], [], [0], 0
+    for w in wg:
+        M, N = w.shape
+        p = torch.empty(M, N // 8, dtype=torch.int32, device=cuda)
+        sc = torch.empty(M, N // 128, dtype=torch.bfloat16, device=cuda)
+        outs.append((p, sc))
+        rows.append([w.data_ptr(), p.data_ptr(), sc.data_ptr(), M * N // 128])
+        work += -(-(M * N // 128) // _lib.INT4_GROUPS_PER_WG)
+        starts.append(work)
+    descs = torch.tensor(rows, dtype=torch.int64).to(cuda)
+    st = torch.tensor(starts, dtype=torch.int64).to(cuda)
+    rc = _lib.load().wq_int4_group_quant_pack_grouped(descs.data_ptr(), st.data_ptr(), len(ws), work, 128,
+                                                      _lib.stream_ptr(cuda))
+    _lib.check(rc, "grouped")
+    for w, (p, sc) in zip(ws, outs):
+        po, so, _ = C.int4_pack_layer(w, 128, True)
+        assert torch.equal(p.cpu(), po) and I.same_bits(sc.cpu(), so)
