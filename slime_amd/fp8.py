@@ -166,6 +166,9 @@ def _align(n: int, a: int = 256) -> int:
     return (n + a - 1) // a * a
 
 
+_ITEM_TABLE_MIN_TENSORS = 64     # plans with at least this many tensors pre-resolve every work item on the host
+
+
 def _to_device_i64(rows, device) -> torch.Tensor:
     return torch.tensor(rows, dtype=torch.int64).to(device)
 
@@ -213,24 +216,37 @@ class Fp8QuantPlan:
             starts.append(tiles)
         self.total_tiles = tiles
         self.bf16_bytes = sum(2 * w.numel() for w in self.weights)
-        # one descriptor per tile, moved to the tile's origin (64 bytes per 48 KiB of traffic): the kernel then needs
-        # a single scalar load instead of a search through the per-tensor prefix sums
-        desc = torch.tensor(rows, dtype=torch.int64)             # x, y, s, M, N, sx_m, sx_n, sy_m
-        start = torch.tensor(starts, dtype=torch.int64)
-        owner = torch.repeat_interleave(torch.arange(len(rows)), start[1:] - start[:-1])
-        local = torch.arange(tiles, dtype=torch.int64) - start[owner]
-        d = desc[owner]
-        kt = (d[:, 4] + self.bn - 1) // self.bn
-        tm, tn = local // kt, local % kt
-        r0, c0 = tm * self.bm, tn * self.bn
-        table = torch.stack([d[:, 0] + (r0 * d[:, 5] + c0 * d[:, 6]) * 2, d[:, 1] + r0 * d[:, 7] + c0,
-                             d[:, 2] + local * 4, d[:, 3] - r0, d[:, 4] - c0, d[:, 5], d[:, 6], d[:, 7]], dim=1)
-        self._tiles = table.contiguous().to(self.device)
+        # Many small tensors: one descriptor per tile, moved to the tile's origin (64 bytes per 48 KiB of traffic), so
+        # that the kernel needs a single scalar load instead of a search through the per-tensor prefix sums.  A
+        # handful of tensors (the q/k/v or gate/up group of one weight-sync call) keeps the search: it is short
+        # there and the table would cost more host time to build than it saves.
+        self._tiles = None
+        if len(rows) >= _ITEM_TABLE_MIN_TENSORS:
+            desc = torch.tensor(rows, dtype=torch.int64)             # x, y, s, M, N, sx_m, sx_n, sy_m
+            start = torch.tensor(starts, dtype=torch.int64)
+            owner = torch.repeat_interleave(torch.arange(len(rows)), start[1:] - start[:-1])
+            local = torch.arange(tiles, dtype=torch.int64) - start[owner]
+            d = desc[owner]
+            kt = (d[:, 4] + self.bn - 1) // self.bn
+            tm, tn = local // kt, local % kt
+            r0, c0 = tm * self.bm, tn * self.bn
+            table = torch.stack([d[:, 0] + (r0 * d[:, 5] + c0 * d[:, 6]) * 2, d[:, 1] + r0 * d[:, 7] + c0,
+                                 d[:, 2] + local * 4, d[:, 3] - r0, d[:, 4] - c0, d[:, 5], d[:, 6], d[:, 7]], dim=1)
+            self._tiles = table.contiguous().to(self.device)
+        else:
+            self._descs = _to_device_i64(rows, self.device)
+            self._starts = _to_device_i64(starts, self.device)
 
     def run(self):
+        lib = _lib.load()
         with torch.cuda.device(self.device):
-            rc = _lib.load().wq_fp8_block_quant_tiles(self._tiles.data_ptr(), self.total_tiles, self.bm, self.bn,
-                                                      self.mode, _lib.stream_ptr(self.device))
+            if self._tiles is not None:
+                rc = lib.wq_fp8_block_quant_tiles(self._tiles.data_ptr(), self.total_tiles, self.bm, self.bn, self.mode,
+                                                  _lib.stream_ptr(self.device))
+            else:
+                rc = lib.wq_fp8_block_quant_grouped(self._descs.data_ptr(), self._starts.data_ptr(), len(self.weights),
+                                                    self.total_tiles, self.bm, self.bn, self.mode,
+                                                    _lib.stream_ptr(self.device))
         _lib.check(rc, "Fp8QuantPlan.run")
         return self.outputs
 

@@ -162,6 +162,9 @@ def pack_layer(weight: torch.Tensor, group_size: int, sym: bool = True):
     return pack_to_int32(codes, 4, sym=sym), scale, packed_zp
 
 
+_ITEM_TABLE_MIN_TENSORS = 64     # plans with at least this many tensors pre-resolve every work item on the host
+
+
 class Int4PackPlan:
     """Symmetric quantise+pack of a fixed list of contiguous bf16 weights with one launch per ``run()``.
 
@@ -201,23 +204,35 @@ class Int4PackPlan:
             starts.append(work)
         self.total_work = work
         self.bf16_bytes = sum(2 * w.numel() for w in self.weights)
-        # one pre-resolved descriptor per work item (32 bytes per 16 KiB of weights): the kernel then needs a single
-        # scalar load instead of a search through the per-tensor prefix sums
-        per = _lib.INT4_GROUPS_PER_WG
-        desc = torch.tensor(rows, dtype=torch.int64)
-        start = torch.tensor(starts, dtype=torch.int64)
-        owner = torch.repeat_interleave(torch.arange(len(rows)), start[1:] - start[:-1])
-        local = torch.arange(work, dtype=torch.int64) - start[owner]
-        items = torch.stack([desc[owner, 0] + local * (per * self.group * 2),
-                             desc[owner, 1] + local * (per * self.group // 8 * 4),
-                             desc[owner, 2] + local * (per * 2),
-                             torch.clamp(desc[owner, 3] - local * per, max=per)], dim=1)
-        self._items = items.contiguous().to(self.device)
+        # Many small tensors (the experts of a model): one pre-resolved descriptor per work item (32 bytes per 16 KiB of
+        # weights), so that the kernel needs a single scalar load instead of a search through the per-tensor prefix
+        # sums.  A handful of tensors keeps the search.
+        self._items = None
+        if len(rows) >= _ITEM_TABLE_MIN_TENSORS:
+            per = _lib.INT4_GROUPS_PER_WG
+            desc = torch.tensor(rows, dtype=torch.int64)
+            start = torch.tensor(starts, dtype=torch.int64)
+            owner = torch.repeat_interleave(torch.arange(len(rows)), start[1:] - start[:-1])
+            local = torch.arange(work, dtype=torch.int64) - start[owner]
+            items = torch.stack([desc[owner, 0] + local * (per * self.group * 2),
+                                 desc[owner, 1] + local * (per * self.group // 8 * 4),
+                                 desc[owner, 2] + local * (per * 2),
+                                 torch.clamp(desc[owner, 3] - local * per, max=per)], dim=1)
+            self._items = items.contiguous().to(self.device)
+        else:
+            self._descs = torch.tensor(rows, dtype=torch.int64).to(self.device)
+            self._starts = torch.tensor(starts, dtype=torch.int64).to(self.device)
 
     def run(self):
+        lib = _lib.load()
         with torch.cuda.device(self.device):
-            rc = _lib.load().wq_int4_group_quant_pack_items(self._items.data_ptr(), self.total_work, self.group,
-                                                            _lib.stream_ptr(self.device))
+            if self._items is not None:
+                rc = lib.wq_int4_group_quant_pack_items(self._items.data_ptr(), self.total_work, self.group,
+                                                        _lib.stream_ptr(self.device))
+            else:
+                rc = lib.wq_int4_group_quant_pack_grouped(self._descs.data_ptr(), self._starts.data_ptr(),
+                                                          len(self.weights), self.total_work, self.group,
+                                                          _lib.stream_ptr(self.device))
         _lib.check(rc, "Int4PackPlan.run")
         return self.outputs
 

@@ -252,6 +252,25 @@ def test_quant_plan_equals_single_calls(cuda):
         wg[0].div_(2)
 
 
+def test_quant_plan_many_tensors_uses_tile_table(cuda):
+    # 8 tensors keep the searched launch (above); 72 mixed tensors get one pre-resolved descriptor per tile
+    shapes = [(256, 384), (300, 200), (7, 7168), (129, 127), (128, 128), (1, 1), (640, 128), (100, 1000), (384, 2560)] * 8
+    ws = [I.zero_blocks(I.weights(*sh, seed=300 + i), 0.1, seed=i) for i, sh in enumerate(shapes)]
+    wg = [w.to(cuda) for w in ws]
+    wg[1] = wg[1].t().contiguous().t()              # strided members: generic path behind a tile descriptor
+    wg[12] = wg[12].t().contiguous().t()
+    for mode in (0, 1, 2):
+        plan = slime_amd.Fp8QuantPlan(wg, (128, 128), mode)
+        assert plan._tiles is not None and plan._tiles.shape == (plan.total_tiles, 8)
+        for w, (q, s) in zip(ws, plan.run()):
+            qo, so = C.fp8_block_quant(w, (128, 128), mode)
+            assert torch.equal(_codes(q), qo) and torch.equal(_bits32(s), _bits32(so))
+    plan = slime_amd.Fp8QuantPlan(wg, (64, 32), 2)   # other block sizes through the same table
+    for w, (q, s) in zip(ws, plan.run()):
+        qo, so = C.fp8_block_quant(w, (64, 32), 2)
+        assert torch.equal(_codes(q), qo) and torch.equal(_bits32(s), _bits32(so))
+
+
 def test_dequant_plan_equals_single_calls(cuda):
     shapes = [(2048, 7168), (7168, 2048), (300, 200), (16, 1024), (5, 1000)]
     xs = [I.fp8_codes(*sh, seed=i) for i, sh in enumerate(shapes)]

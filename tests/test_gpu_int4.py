@@ -226,6 +226,21 @@ def test_pack_plan_moe_experts(cuda):
     assert ((nib * sf - ws[0].to(cuda).float()).abs() <= sf * (0.5 + 7 * 2 ** -8)).all()
 
 
+def test_pack_plan_many_small_tensors_uses_item_table(cuda):
+    # 24 tensors keep the searched launch (above); 90 mixed tensors get one pre-resolved descriptor per work item
+    shapes = [(96, 256), (33, 768), (1, 128), (64, 128), (7, 7168), (128, 2048), (5, 384), (200, 1024), (63, 128)] * 10
+    ws = [I.weights(*sh, seed=200 + i) for i, sh in enumerate(shapes)]
+    plan = slime_amd.Int4PackPlan([w.to(cuda) for w in ws], 128)
+    assert plan._items is not None and plan._items.shape == (plan.total_work, 4)
+    for w, (p, s) in zip(ws, plan.run()):
+        po, so, _ = C.int4_pack_layer(w, 128, True)
+        assert torch.equal(p.cpu(), po) and I.same_bits(s.cpu(), so)
+    plan32 = slime_amd.Int4PackPlan([w.to(cuda) for w in ws[:70]], 32)
+    for w, (p, s) in zip(ws, plan32.run()):
+        po, so, _ = C.int4_pack_layer(w, 32, True)
+        assert torch.equal(p.cpu(), po) and I.same_bits(s.cpu(), so)
+
+
 def test_int4_golden(cuda):
     from safetensors.torch import load_file
 
