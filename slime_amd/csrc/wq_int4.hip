@@ -338,8 +338,18 @@ __global__ __launch_bounds__(256) void int4_fake_quant_vec_kernel(const uint16_t
             vmin = lanes_min_f32<L>(vmin);
             scale = fmaxf((vmax - vmin) * (1.0f / 15.0f), 1e-5f);
             zero = fminf(fmaxf(-__builtin_rintf(vmin / scale), 0.0f), 15.0f) + 0.0f;
+            // x / scale by the correctly rounded reciprocal (one division per lane) and the two-FMA correction, which
+            // yields the correctly rounded quotient for any fp32 divisor as long as the reciprocal is a normal number and
+            // nothing overflows (Markstein's theorem); groups holding huge or non-finite values divide element by element.
+            const float r = 1.0f / scale;
+            const bool safe = scale < 0x1p100f && fmaxf(fabsf(vmax), fabsf(vmin)) * r < 0x1p60f;
+            if (__builtin_amdgcn_ballot_w64(!safe) == 0) {
 #pragma unroll
-            for (int j = 0; j < 8; ++j) o[j] = __builtin_rintf(xs[j] / scale) + zero;
+                for (int j = 0; j < 8; ++j) o[j] = __builtin_rintf(div_by_scale(xs[j], scale, r)) + zero;
+            } else {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) o[j] = __builtin_rintf(xs[j] / scale) + zero;
+            }
         }
         if (g < n_groups) {
             u32x4 r = {pack2_bf16_hw(o[0], o[1]), pack2_bf16_hw(o[2], o[3]), pack2_bf16_hw(o[4], o[5]),
@@ -405,12 +415,19 @@ __global__ __launch_bounds__(256) void int4_pack_asym_kernel(const uint16_t* __r
         const float zero = fminf(fmaxf(-__builtin_rintf(vmin / scale), 0.0f), 15.0f) + 0.0f;
         const uint32_t sb_bits = f32_to_bf16_bits(scale);
         float q[8];
+        // x / scale by the correctly rounded reciprocal and the two-FMA correction (see int4_fake_quant_vec_kernel)
+        const float r = 1.0f / scale;
+        const bool safe = scale < 0x1p100f && fmaxf(fabsf(vmax), fabsf(vmin)) * r < 0x1p60f;
+        if (__builtin_amdgcn_ballot_w64(!safe) == 0) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) q[j] = __builtin_rintf(div_by_scale(xs[j], scale, r)) + zero;
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) q[j] = __builtin_rintf(xs[j] / scale) + zero;
+        }
         bool plain = sb_bits < kLiteralChainScaleBits;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            q[j] = __builtin_rintf(xs[j] / scale) + zero;
-            plain = plain && q[j] >= 0.0f && q[j] <= 17.0f;
-        }
+        for (int j = 0; j < 8; ++j) plain = plain && q[j] >= 0.0f && q[j] <= 17.0f;
         uint32_t word = 0;
         if (plain) {
 #pragma unroll

@@ -130,6 +130,22 @@ def test_fake_quant_every_bf16_value(cuda, sym):
     _fake_quant_same(q.cpu(), s.cpu(), z.cpu(), *C.int4_fake_quant(w, (1, 128), sym))
 
 
+def test_fake_quant_asym_many_scales(cuda):
+    # the asymmetric quotients use a reciprocal and a two-FMA correction: 4M elements under ~32k different scales,
+    # with offsets (one-sided groups), tiny ranges (1e-5 floor) and ties (bf16 data makes x / scale land on .5 often)
+    g = I.gen(77)
+    base = torch.randn(4096, 1024, generator=g)
+    scale = torch.exp(torch.empty(4096, 8, 1).uniform_(-12.0, 6.0, generator=g))
+    shift = torch.randn(4096, 8, 1, generator=g) * (torch.rand(4096, 8, 1, generator=g) < 0.3)
+    w = ((base.view(4096, 8, 128) + shift) * scale).view(4096, 1024).to(torch.bfloat16)
+    q, s, z = slime_amd.fake_int4_quant_cuda(w.to(cuda), (1, 128), False)
+    _fake_quant_same(q.cpu(), s.cpu(), z.cpu(), *C.int4_fake_quant(w, (1, 128), False))
+    w8 = w[:, :512].contiguous()
+    p, sc, pz = slime_amd.pack_layer(w8.to(cuda), 128, False)
+    po, so, pzo = C.int4_pack_layer(w8, 128, False)
+    assert torch.equal(p.cpu(), po) and I.same_bits(sc.cpu(), so) and torch.equal(pz.cpu(), pzo)
+
+
 def test_fake_quant_ragged_big(cuda):
     w = I.weights(4100, 3000, seed=2)
     q, s, z = slime_amd.fake_int4_quant_cuda(w.to(cuda), (1, 128), True)
