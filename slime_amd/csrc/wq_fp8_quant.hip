@@ -352,12 +352,22 @@ typedef float f32x2q __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2q __attribute__((ext_vector_type(2)));
 
 // Two elements of the per-tensor form: IEEE quotient, rounded to bf16 (the reference's bf16 tensor), NaN-propagating
-// clamp, e4m3fn.  Returns the two codes in the low 16 bits.
-__device__ __forceinline__ uint32_t tensor_quant2(uint32_t w, float divisor)
+// clamp, e4m3fn.  Returns the two codes in the low 16 bits.  FAST: the tensor's amax is finite, so |x / divisor| stays
+// near 448 and the quotient comes from the correctly rounded reciprocal and two FMAs (exact for any divisor); that
+// form turns -0 into +0, so the sign of x is put back on the code.
+template <bool FAST>
+__device__ __forceinline__ uint32_t tensor_quant2(uint32_t w, float divisor, float rcp)
 {
-    f32x2q q = {bf16lo(w) / divisor, bf16hi(w) / divisor};
+    const float x0 = bf16lo(w), x1 = bf16hi(w);
+    f32x2q q = {FAST ? div_by_scale(x0, divisor, rcp) : x0 / divisor, FAST ? div_by_scale(x1, divisor, rcp) : x1 / divisor};
     const uint32_t b = __builtin_bit_cast(uint32_t, __builtin_convertvector(q, bf16x2q));
     float q0 = bf16lo(b), q1 = bf16hi(b);
+    if (FAST) {
+        q0 = fminf(fmaxf(q0, -kFp8Max), kFp8Max);
+        q1 = fminf(fmaxf(q1, -kFp8Max), kFp8Max);
+        const uint32_t r = cvt_pk_fp8_lo(q0, q1, 0u) & 0x7F7Fu;
+        return r | ((w >> 8) & 0x80u) | ((w >> 16) & 0x8000u);
+    }
     const bool nan0 = q0 != q0, nan1 = q1 != q1;
     q0 = fminf(fmaxf(q0, -kFp8Max), kFp8Max);
     q1 = fminf(fmaxf(q1, -kFp8Max), kFp8Max);
@@ -383,13 +393,25 @@ __global__ __launch_bounds__(256) void fp8_tensor_apply_vec_kernel(const uint16_
     u32x4 v[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) v[i] = ldg_nt<u32x4>(xb + min(p0 + i * 256, n_pieces - 1) * 16);
+    const float rcp = 1.0f / divisor;
+    if (p.fast && divisor > 0x1p-100f) {      // finite amax, reciprocal a normal number
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int64_t piece = p0 + i * 256;
-        u32x2 o;
-        o.x = tensor_quant2(v[i].x, divisor) | (tensor_quant2(v[i].y, divisor) << 16);
-        o.y = tensor_quant2(v[i].z, divisor) | (tensor_quant2(v[i].w, divisor) << 16);
-        if (piece < n_pieces) stg_nt<u32x2>(y + piece * 8, o);
+        for (int i = 0; i < 4; ++i) {
+            const int64_t piece = p0 + i * 256;
+            u32x2 o;
+            o.x = tensor_quant2<true>(v[i].x, divisor, rcp) | (tensor_quant2<true>(v[i].y, divisor, rcp) << 16);
+            o.y = tensor_quant2<true>(v[i].z, divisor, rcp) | (tensor_quant2<true>(v[i].w, divisor, rcp) << 16);
+            if (piece < n_pieces) stg_nt<u32x2>(y + piece * 8, o);
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int64_t piece = p0 + i * 256;
+            u32x2 o;
+            o.x = tensor_quant2<false>(v[i].x, divisor, rcp) | (tensor_quant2<false>(v[i].y, divisor, rcp) << 16);
+            o.y = tensor_quant2<false>(v[i].z, divisor, rcp) | (tensor_quant2<false>(v[i].w, divisor, rcp) << 16);
+            if (piece < n_pieces) stg_nt<u32x2>(y + piece * 8, o);
+        }
     }
 }
 

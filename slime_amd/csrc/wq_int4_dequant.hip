@@ -115,14 +115,16 @@ __global__ __launch_bounds__(256) void int4_fake_ste_kernel(const uint16_t* __re
         float s = div7 == WQ_DIV7_DEVICE ? u2f(mb << 16) * (1.0f / 7.0f) : u2f(mb << 16) / 7.0f;
         s = (s != s) ? s : fmaxf(s, 1e-5f);           // clamp(min=1e-5) keeps NaN
         float o[8];
-        // Finite amax under the reciprocal-multiply rule: s is the scale of the pack kernel, for which
+        // Finite amax.  Under the reciprocal-multiply rule s is the scale of the pack kernel, for which
         // q0 = x*r, q = fma(fma(-q0, s, x), r, q0) rounds to the same integer as the IEEE quotient for every bf16 x
         // of the group (the exhaustive check of the pack function covers exactly these pairs).  |q| <= 7 there, so
         // the clamp is a no-op; adding and subtracting 1.5 * 2^23 rounds half to even.  The result carries the
         // sign of x, zero included (round and clamp keep it, s is positive); it is restored on the bf16 pairs.
-        const bool fast = div7 == WQ_DIV7_DEVICE && mb < kBf16Inf;
+        const bool fast = mb < kBf16Inf;
         if (fast) {
-            const float r = rcp_refined(s);
+            // under the division rule s is an arbitrary fp32 number: the correctly rounded reciprocal (one division
+            // per lane) keeps the two-FMA quotient exact for any divisor
+            const float r = div7 == WQ_DIV7_DEVICE ? rcp_refined(s) : 1.0f / s;
 #pragma unroll
             for (int j = 0; j < 8; ++j) o[j] = ((div_by_scale(xs[j], s, r) + 12582912.0f) - 12582912.0f) * s;
         } else {

@@ -433,3 +433,14 @@ def test_grouped_search_entry_point(cuda):
     for w, (p, sc) in zip(ws, outs):
         po, so, _ = C.int4_pack_layer(w, 128, True)
         assert torch.equal(p.cpu(), po) and I.same_bits(sc.cpu(), so)
+
+
+def test_fake_ste_many_scales_both_rules(cuda):
+    g = I.gen(78)
+    base = torch.randn(4096, 1024, generator=g)
+    scale = torch.exp(torch.empty(4096, 8, 1).uniform_(-12.0, 6.0, generator=g))
+    w = (base.view(4096, 8, 128) * scale).view(4096, 1024).to(torch.bfloat16)
+    for div7, arith in ARITH.items():
+        with slime_amd.torch_arithmetic(arith):
+            y = slime_amd.fake_int4_quantization_ste(w.to(cuda), 128)
+        assert I.same_bits(y.cpu(), C.int4_fake_ste(w, 128, div7)), arith
