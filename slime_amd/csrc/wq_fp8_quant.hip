@@ -321,6 +321,63 @@ __global__ __launch_bounds__(256) void fp8_row_quant_vec_kernel(const uint16_t* 
     }
 }
 
+// Rows of up to 8192 elements: one wavefront per row (four rows per workgroup), so that short rows still put
+// 16 - 64 KiB per workgroup in flight; no LDS, no barrier.
+constexpr int kWaveRowMaxSteps = 16;
+__global__ __launch_bounds__(256) void fp8_row_quant_wave_kernel(const uint16_t* __restrict__ x, int64_t M, int64_t N,
+                                                                int64_t sx_m, uint8_t* __restrict__ y, int64_t sy_m,
+                                                                float* __restrict__ s, int mode, int64_t items)
+{
+    const int64_t slot = (int64_t)blockIdx.x + (int64_t)blockIdx.y * gridDim.x;
+    if (slot >= items) return;
+    const int64_t item = xcd_chunked_item(slot, items, kRowsPerXcdRun);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const int64_t row = item * 4 + wave;
+    if (row >= M) return;                                  // uniform per wavefront
+    const char* xr = (const char*)(x + row * sx_m);
+    char* yr = (char*)(y + row * sy_m);
+    const int n_pieces = (int)(N / 8);
+    const int steps = (n_pieces + 63) / 64;
+    u32x4 v[kWaveRowMaxSteps];
+#pragma unroll
+    for (int i = 0; i < kWaveRowMaxSteps; ++i)
+        if (i < steps) v[i] = ldg_nt<u32x4>(xr + (uint32_t)min(i * 64 + lane, n_pieces - 1) * 16u);
+    uint32_t m = 0;
+#pragma unroll
+    for (int i = 0; i < kWaveRowMaxSteps; ++i) {
+        if (i < steps) {
+            if (i * 64 + lane >= n_pieces) v[i] = (u32x4){0u, 0u, 0u, 0u};
+            m = pk_absmax(m, v[i].x);
+            m = pk_absmax(m, v[i].y);
+            m = pk_absmax(m, v[i].z);
+            m = pk_absmax(m, v[i].w);
+        }
+    }
+    m = wave64_max_u32(pk_fold(m));
+    const Fp8BlockParams p = torch_params(m, mode);
+    if (lane == 0) stg<float>(s + row, p.scale);
+    if (p.fast) {
+#pragma unroll
+        for (int i = 0; i < kWaveRowMaxSteps; ++i) {
+            if (i < steps) {
+                const int piece = i * 64 + lane;
+                u32x2 o;
+                o.x = fp8_quant4_fast<WQ_FP8_MODE_TORCH>(v[i].x, v[i].y, p);
+                o.y = fp8_quant4_fast<WQ_FP8_MODE_TORCH>(v[i].z, v[i].w, p);
+                if (piece < n_pieces) stg_nt<u32x2>(yr + (uint32_t)piece * 8u, o);
+            }
+        }
+    } else {
+        for (int piece = lane; piece < n_pieces; piece += 64) {
+            const u32x4 w = ldg<u32x4>(xr + (uint32_t)piece * 16u);
+            u32x2 o;
+            o.x = fp8_quant4_exact<WQ_FP8_MODE_TORCH>(w.x, w.y, p);
+            o.y = fp8_quant4_exact<WQ_FP8_MODE_TORCH>(w.z, w.w, p);
+            stg<u32x2>(yr + (uint32_t)piece * 8u, o);
+        }
+    }
+}
+
 // Per-tensor amax of a contiguous tensor: a bounded grid, four 16-byte pieces per lane in flight, one atomic per
 // workgroup.
 __global__ __launch_bounds__(256) void fp8_tensor_amax_vec_kernel(const uint16_t* __restrict__ x, int64_t n_pieces,
@@ -577,6 +634,10 @@ WQ_EXPORT int wq_fp8_row_quant(const void* x, int64_t M, int64_t N, int64_t sx_m
     uint8_t* yp = (uint8_t*)y;
     const dim3 g = grid_for_items(M);
     if (!vec) fp8_row_quant_kernel<<<g, 256, 0, st>>>(xp, M, N, sx_m, sx_n, yp, sy_m, s, mode);
+    else if (N <= 8 * 64 * kWaveRowMaxSteps) {
+        const int64_t items = cdiv64(M, 4);
+        fp8_row_quant_wave_kernel<<<grid_for_items(items), 256, 0, st>>>(xp, M, N, sx_m, yp, sy_m, s, mode, items);
+    }
     else if (N <= kRowPieceElems) fp8_row_quant_vec_kernel<1><<<g, 256, 0, st>>>(xp, M, N, sx_m, yp, sy_m, s, mode);
     else if (N <= 2 * kRowPieceElems) fp8_row_quant_vec_kernel<2><<<g, 256, 0, st>>>(xp, M, N, sx_m, yp, sy_m, s, mode);
     else if (N <= 4 * kRowPieceElems) fp8_row_quant_vec_kernel<4><<<g, 256, 0, st>>>(xp, M, N, sx_m, yp, sy_m, s, mode);
