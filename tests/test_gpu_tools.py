@@ -11,6 +11,7 @@ from safetensors.torch import load_file, save_file
 from oracle import c_oracle as C
 from slime_amd.tools import convert_hf_to_fp8 as F8
 from slime_amd.tools import convert_hf_to_int4_direct as I4
+from slime_amd.tools import convert_k2_thinking_int4_to_bf16 as K2
 from slime_amd.tools import fp8_cast_bf16 as CAST
 from tests import wq_inputs as I
 
@@ -144,3 +145,46 @@ def test_convert_hf_to_int4_direct(ckpt, tmp_path, cuda, group, sym):
             assert I.same_bits(got[k], w), k
     idx = json.load(open(out / "model.safetensors.index.json"))
     assert set(idx["weight_map"]) == set(got) and idx["metadata"]["total_size"] == sum(len(v) for v in got.values())
+
+
+def test_convert_int4_experts_to_bf16(tmp_path, cuda):
+    # a pack-quantized checkpoint as convert_hf_to_int4_direct writes it -> bf16, tool against the oracle
+    src = tmp_path / "int4"
+    src.mkdir()
+    w = {"model.layers.0.mlp.experts.0.gate_proj": I.weights(64, 256, seed=1),
+         "model.layers.0.mlp.experts.0.down_proj": I.weights(256, 128, seed=2),
+         "model.layers.0.mlp.experts.1.up_proj": I.weights(40, 384, seed=3)}
+    shard = {"model.embed_tokens.weight": I.weights(16, 64, seed=4),
+             "model.layers.0.mlp.shared_experts.gate_proj.weight_packed": torch.zeros(4, 8, dtype=torch.int32),
+             "model.layers.0.mlp.experts.2.up_proj.weight_packed": torch.ones(4, 8, dtype=torch.int32)}   # incomplete
+    want = {}
+    for name, t in w.items():
+        p, s, _ = C.int4_pack_layer(t, 64, True)
+        shard[f"{name}.weight_packed"], shard[f"{name}.weight_scale"] = p, s
+        shard[f"{name}.weight_shape"] = torch.tensor(list(t.shape), dtype=torch.int32)
+        want[f"{name}.weight"] = C.int4_dequant(p, s, tuple(t.shape), 64)
+    save_file(shard, str(src / "model-00001-of-00001.safetensors"))
+    cfg = {"hidden_size": 256, "moe_intermediate_size": 64,
+           "quantization_config": {"config_groups": {"group_0": {"weights": {"group_size": 64}}}}}
+    json.dump(cfg, open(src / "config.json", "w"))
+    (src / "tokenizer.json").write_text("{}")
+    (src / "modeling.py").write_text("# code")
+    (src / "notes.txt").write_text("not copied")
+    out = tmp_path / "bf16"
+    assert K2._load_config(str(src), None) == (256, 64, 64)
+    K2.main(["--model-dir", str(src), "--output-dir", str(out)])
+    got = load_file(str(out / "model-00001-of-00001.safetensors"))
+    for name, t in want.items():
+        assert got[name].dtype == torch.bfloat16 and I.same_bits(got[name], t), name
+    assert not any(k.endswith((".weight_scale", ".weight_shape")) for k in got)
+    assert torch.equal(got["model.embed_tokens.weight"], shard["model.embed_tokens.weight"])
+    assert "model.layers.0.mlp.shared_experts.gate_proj.weight_packed" in got            # shared experts are not touched
+    assert "model.layers.0.mlp.experts.2.up_proj.weight_packed" in got                   # incomplete triple is kept
+    index = json.load(open(out / "model.safetensors.index.json"))
+    assert index["metadata"] == {} and set(index["weight_map"]) == set(got)
+    assert sorted(os.listdir(out)) == ["config.json", "model-00001-of-00001.safetensors", "model.safetensors.index.json",
+                                       "modeling.py", "tokenizer.json"]
+    # skip_existing: a second run leaves the file alone; --overwrite rewrites it
+    before = os.path.getmtime(out / "model-00001-of-00001.safetensors")
+    K2.main(["--model-dir", str(src), "--output-dir", str(out)])
+    assert os.path.getmtime(out / "model-00001-of-00001.safetensors") == before

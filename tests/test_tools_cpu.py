@@ -59,3 +59,16 @@ def test_index_total_size_is_sum_of_first_dims(tmp_path):
     idx = json.load(open(tmp_path / "model.safetensors.index.json"))
     assert idx == {"weight_map": {"a": "s1.safetensors", "b": "s1.safetensors", "c": "s2.safetensors"},
                    "metadata": {"total_size": 14}}
+
+
+def test_int4_to_bf16_key_rule():
+    from slime_amd.tools import convert_k2_thinking_int4_to_bf16 as K2
+
+    yes = ["model.layers.3.mlp.experts.17.gate_proj.weight_packed", "model.layers.3.mlp.experts.0.down_proj.weight_scale",
+           "model.layers.60.mlp.experts.383.up_proj.weight_shape"]
+    no = ["model.layers.3.mlp.shared_experts.gate_proj.weight_packed", "model.layers.3.mlp.experts.17.gate_proj.weight",
+          "model.layers.3.self_attn.q_proj.weight_packed", "model.layers.3.mlp.experts.17.gate_proj.weight_zero_point",
+          "model.layers.3.mlp.gate.weight"]
+    assert all(K2._is_quantized_weight_key(k) for k in yes) and not any(K2._is_quantized_weight_key(k) for k in no)
+    args = K2.parse_args(["--model-dir", "m", "--files", "a.safetensors", "b.safetensors", "--overwrite"])
+    assert args.files == ["a.safetensors", "b.safetensors"] and args.overwrite and args.output_dir is None
