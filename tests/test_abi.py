@@ -104,3 +104,15 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "nope.so"))
     with pytest.raises(_lib.WqLibraryError, match="no CPU or pure-torch fallback"):
         _lib.load()
+
+
+def test_shim_module_does_not_shadow_the_function():
+    import slime_amd
+    import slime_amd.fake_int4_quant_cuda as shim
+
+    # after the import the package attribute is the module; it must still be callable like the function
+    assert callable(slime_amd.fake_int4_quant_cuda) and callable(shim.fake_int4_quant_cuda)
+    import torch
+
+    with pytest.raises(RuntimeError):
+        slime_amd.fake_int4_quant_cuda(torch.zeros(4, 32), (1, 32), True)      # reaches the function: CPU input refused
