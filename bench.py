@@ -201,12 +201,22 @@ def bench_int4_inverse(dev, steps, warmup, layers, which):
             else:
                 tensors.append(w)
     outs = [None] * len(tensors)
+    if which == "int4deq":
+        # every expert its own tensor (views of the layer's packed buffer), all of them in one launch
+        per_expert = []
+        for p, sc, (rows, cols) in tensors:
+            r = rows // 128
+            per_expert += [(p[e * r:(e + 1) * r], sc[e * r:(e + 1) * r], (r, cols)) for e in range(128)]
+        plan = slime_amd.Int4DequantPlan([t[0] for t in per_expert], [t[1] for t in per_expert],
+                                         [t[2] for t in per_expert], 128)
 
-    def run():
-        for i, t in enumerate(tensors):
-            outs[i] = None          # free the previous output first: the allocator reuses the block
-            outs[i] = (slime_amd.dequantize_int4(t[0], t[1], t[2], 128) if which == "int4deq"
-                       else slime_amd.fake_int4_quantization_ste(t, 128))
+        def run():
+            plan.run()
+    else:
+        def run():
+            for i, t in enumerate(tensors):
+                outs[i] = None          # free the previous output first: the allocator reuses the block
+                outs[i] = slime_amd.fake_int4_quantization_ste(t, 128)
 
     wall_ms, ev_ms, ev_min = _time_launches(run, steps, warmup)
     elements = sum((t[2][0] * t[2][1]) if which == "int4deq" else t.numel() for t in tensors)
@@ -215,13 +225,18 @@ def bench_int4_inverse(dev, steps, warmup, layers, which):
         if which == "int4deq":
             p, sc, shape = tensors[idx]
             want = c_oracle.int4_dequant(p[:1024].cpu(), sc[:1024].cpu(), (1024, shape[1]), 128)
+            r = shape[0] // 128
+            got = torch.cat([plan.outputs[idx * 128 + e] for e in range(-(-1024 // r))])[:1024]
         else:
             want = c_oracle.int4_fake_ste(tensors[idx][:1024].cpu(), 128, 1)
-        assert torch.equal(outs[idx][:1024].cpu().view(torch.int16), want.view(torch.int16))
+            got = outs[idx][:1024]
+        assert torch.equal(got.cpu().view(torch.int16), want.view(torch.int16))
+    launches = 1 if which == "int4deq" else len(tensors)
     out = {"workload": f"Qwen3-30B-A3B experts, {layers} layers x (gate, up [128x768,2048], down [128x2048,768]), "
                        + ("INT4 group 128 -> bf16" if which == "int4deq" else "INT4 QAT quantise-dequantise forward")
-                       + f", {len(tensors)} launches per step",
-           "launches": len(tensors), "bf16_GB": 2 * elements / 1e9, "kernel_ms": ev_ms, "wall_ms": wall_ms,
+                       + (f", {len(tensors) * 128} expert tensors in one launch" if which == "int4deq"
+                          else f", {len(tensors)} launches per step"),
+           "launches": launches, "bf16_GB": 2 * elements / 1e9, "kernel_ms": ev_ms, "wall_ms": wall_ms,
            "bf16_GBps": 2 * elements / ev_ms / 1e6, "algo_GBps": algo_bytes / ev_ms / 1e6,
            "hbm_frac": algo_bytes / ev_ms / 1e6 / HBM_PEAK_GBS, "parity_tensors_checked": 2}
     del tensors, outs

@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define WQ_ABI_VERSION 7
+#define WQ_ABI_VERSION 8
 
 enum {
     WQ_OK = 0,
@@ -195,6 +195,20 @@ int wq_int4_group_quant_pack_asym(const void *x, int64_t M, int64_t N, int64_t s
  * group % 8 == 0.  Replaces _dequantize_tensor, tools/convert_k2_thinking_int4_to_bf16.py:55-84 (whose unpacking
  * is compressed_tensors.unpack_from_int32). */
 int wq_int4_dequant(const int32_t *packed, const void *scale, void *y, int64_t M, int64_t N, int group, void *stream);
+
+/* wq_int4_dequant over a bucket of tensors in one launch.  `items` is a DEVICE array with one entry per work item
+ * of WQ_INT4_DEQ_WORDS_PER_ITEM packed words (a tensor's last item may be shorter): pointers to the item's first
+ * packed word, to the scale of its first element and to its first output element, and its number of words.
+ * `group` must be a power of two between 8 and 8 * WQ_INT4_DEQ_WORDS_PER_ITEM, so that an item starts on a group
+ * boundary; y pointers 16-byte aligned. */
+#define WQ_INT4_DEQ_WORDS_PER_ITEM 2048
+typedef struct wq_int4_dequant_item {
+    const int32_t *packed;
+    const void *scale;   /* bf16 */
+    void *y;             /* bf16 */
+    int64_t n_words;
+} wq_int4_dequant_item;
+int wq_int4_dequant_items(const wq_int4_dequant_item *items, int64_t n_items, int group, void *stream);
 
 /* Forward of the INT4 QAT straight-through estimator: per (1 x group) group of a contiguous bf16 [M,N],
  * s = max(f32(amax) / 7, 1e-5), y = bf16(clamp(round_half_even(f32(x) / s), -7, 7) * s); N % group == 0 and

@@ -21,6 +21,7 @@ from .fp8 import (
     weight_dequant_bf16_scale,
 )
 from .int4 import (
+    Int4DequantPlan,
     Int4PackPlan,
     dequantize_int4,
     fake_int4_quant_cuda,
@@ -41,7 +42,7 @@ from .processors import (
 quantize_weight = blockwise_cast_to_fp8_triton
 
 __all__ = [
-    "Fp8DequantPlan", "Fp8QuantPlan", "Int4PackPlan", "block_fp8", "block_fp8_many",
+    "Fp8DequantPlan", "Fp8QuantPlan", "Int4DequantPlan", "Int4PackPlan", "block_fp8", "block_fp8_many",
     "blockwise_cast_to_fp8_triton", "channel_fp8", "dequantize_int4", "fake_int4_quant_cuda",
     "fake_int4_quantization_ste", "get_torch_arithmetic", "set_torch_arithmetic", "torch_arithmetic",
     "pack_layer", "pack_to_int32",

@@ -15,7 +15,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libslime_amd_wq.so")
 
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 # selectors (mirrors of the header's enums)
 DTYPE_BF16, DTYPE_F32, DTYPE_F16 = 0, 1, 2
@@ -24,6 +24,7 @@ DIV7_IEEE, DIV7_DEVICE = 0, 1
 DEQ_MODE_F32SCALE, DEQ_MODE_BF16SCALE = 0, 1
 DEQ_SEG, DEQ_SEGS_PER_WG = 512, 16
 INT4_GROUPS_PER_WG = 64
+INT4_DEQ_WORDS_PER_ITEM = 2048
 
 _i64, _int, _vp, _u32, _u64 = ctypes.c_int64, ctypes.c_int, ctypes.c_void_p, ctypes.c_uint32, ctypes.c_uint64
 
@@ -45,6 +46,7 @@ SIGNATURES = {
     "wq_int4_group_quant_pack_items": [_vp, _i64, _int, _vp],
     "wq_int4_group_quant_pack_asym": [_vp, _i64, _i64, _i64, _int, _vp, _vp, _vp, _vp],
     "wq_int4_dequant": [_vp, _vp, _vp, _i64, _i64, _int, _vp],
+    "wq_int4_dequant_items": [_vp, _i64, _int, _vp],
     "wq_int4_fake_quant_ste": [_vp, _vp, _i64, _i64, _int, _int, _vp],
     "wq_delta_workspace_bytes": [_i64],
     "wq_delta_xor": [_vp, _vp, _vp, _i64, _int, _vp, _vp, _vp],

@@ -19,7 +19,8 @@ typedef float f32x2d __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2d __attribute__((ext_vector_type(2)));
 
 constexpr int kDqSteps = 8;                       // packed words per lane
-constexpr int kDqWordsPerWg = 256 * kDqSteps;     // 8 KiB of packed input, 32 KiB of bf16 output
+constexpr int kDqWordsPerWg = 256 * kDqSteps;     // 8 KiB of packed input, 64 KiB of bf16 output
+static_assert(kDqWordsPerWg == WQ_INT4_DEQ_WORDS_PER_ITEM, "work item size is part of the C ABI");
 constexpr int kDqItemsPerXcdRun = 32;
 constexpr int kDqOccupancyPadBytes = 45 * 1024;           // unused dynamic LDS that caps workgroups per CU
 
@@ -29,15 +30,27 @@ __device__ __forceinline__ uint32_t pack2_bf16(float a, float b)
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2d));
 }
 
+// ITEMS: one pre-resolved descriptor per work item (a bucket of tensors in one launch) instead of one tensor in the
+// kernel arguments; the descriptor points at the item's first word, its first scale and its first output element.
+template <bool ITEMS>
 __global__ __launch_bounds__(256) void int4_dequant_kernel(const uint32_t* __restrict__ packed,
                                                           const uint16_t* __restrict__ scale,
                                                           uint16_t* __restrict__ y, int64_t n_words, int group,
+                                                          const wq_int4_dequant_item* __restrict__ items,
                                                           int64_t total_items)
 {
     const int64_t slot = (int64_t)blockIdx.x + (int64_t)blockIdx.y * gridDim.x;
     if (slot >= total_items) return;
     const int64_t item = xcd_chunked_item(slot, total_items, kDqItemsPerXcdRun);
-    const int64_t w0 = item * kDqWordsPerWg + threadIdx.x;
+    int64_t w0 = item * kDqWordsPerWg + threadIdx.x;
+    if (ITEMS) {
+        const wq_int4_dequant_item it = items[item];
+        packed = (const uint32_t*)it.packed;
+        scale = (const uint16_t*)it.scale;
+        y = (uint16_t*)it.y;
+        n_words = it.n_words;
+        w0 = threadIdx.x;
+    }
     const int gshift = (group & (group - 1)) == 0 ? __builtin_ctz((unsigned)group) : -1;
     uint32_t w[kDqSteps];
     uint32_t sb[kDqSteps];
@@ -156,8 +169,19 @@ WQ_EXPORT int wq_int4_dequant(const int32_t* packed, const void* scale, void* y,
     if (((uintptr_t)y & 15) || ((uintptr_t)packed & 3) || ((uintptr_t)scale & 1)) return WQ_ERR_ALIGN;
     const int64_t n_words = M * (N / 8);
     const int64_t items = cdiv64(n_words, kDqWordsPerWg);
-    int4_dequant_kernel<<<grid_for_items(items), 256, kDqOccupancyPadBytes, (hipStream_t)stream>>>(
-        (const uint32_t*)packed, (const uint16_t*)scale, (uint16_t*)y, n_words, group, items);
+    int4_dequant_kernel<false><<<grid_for_items(items), 256, kDqOccupancyPadBytes, (hipStream_t)stream>>>(
+        (const uint32_t*)packed, (const uint16_t*)scale, (uint16_t*)y, n_words, group, nullptr, items);
+    WQ_LAUNCH_CHECK();
+    return WQ_OK;
+}
+
+WQ_EXPORT int wq_int4_dequant_items(const wq_int4_dequant_item* items, int64_t n_items, int group, void* stream)
+{
+    if (n_items < 0 || group < 8 || (group & (group - 1)) != 0 || group > WQ_INT4_DEQ_WORDS_PER_ITEM * 8) return WQ_ERR_SHAPE;
+    if (n_items == 0) return WQ_OK;
+    if (!items) return WQ_ERR_NULL;
+    int4_dequant_kernel<true><<<grid_for_items(n_items), 256, kDqOccupancyPadBytes, (hipStream_t)stream>>>(
+        nullptr, nullptr, nullptr, 0, group, items, n_items);
     WQ_LAUNCH_CHECK();
     return WQ_OK;
 }

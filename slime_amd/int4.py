@@ -269,6 +269,56 @@ def dequantize_int4(weight_packed: torch.Tensor, weight_scale: torch.Tensor, wei
     return y
 
 
+class Int4DequantPlan:
+    """``dequantize_int4`` over a fixed list of (weight_packed, weight_scale, shape) triples with one launch per
+    ``run()``; ``outputs`` holds bf16 ``[M, N]`` views into one flat buffer (``flat_y``), in input order.  The group
+    size must be a power of two (32, 64, 128 ...)."""
+
+    def __init__(self, packeds: Sequence[torch.Tensor], scales: Sequence[torch.Tensor], shapes, group_size: int):
+        if not packeds or len(packeds) != len(scales) or len(packeds) != len(shapes):
+            raise ValueError("Int4DequantPlan: need equally many packed tensors, scales and shapes")
+        per = _lib.INT4_DEQ_WORDS_PER_ITEM
+        if group_size < 8 or group_size & (group_size - 1) or group_size > 8 * per:
+            raise ValueError(f"Int4DequantPlan: group_size {group_size} must be a power of two in [8, {8 * per}]")
+        self.group = int(group_size)
+        self.device = packeds[0].device
+        self.packeds, self.scales = [], []
+        y_off, total = [], 0
+        shapes = [tuple(int(v) for v in (sh.view(-1).tolist() if isinstance(sh, torch.Tensor) else sh)) for sh in shapes]
+        for p, sc, (M, N) in zip(packeds, scales, shapes):
+            _lib.require_gpu(p, "Int4DequantPlan")
+            if p.dtype != torch.int32 or tuple(p.shape) != (M, N // 8) or N % self.group or sc.dtype != torch.bfloat16 \
+                    or sc.numel() != M * (N // self.group) or p.device != self.device or sc.device != self.device:
+                raise ValueError(f"Int4DequantPlan: packed {tuple(p.shape)} {p.dtype} / scale {tuple(sc.shape)} {sc.dtype} "
+                                 f"do not describe a [{M}, {N}] weight with groups of {self.group}")
+            self.packeds.append(p.contiguous())
+            self.scales.append(sc.contiguous())
+            y_off.append(total)
+            total += (M * N + 127) // 128 * 128
+        self.flat_y = torch.empty(max(total, 1), dtype=torch.bfloat16, device=self.device)
+        self.outputs = [self.flat_y[o:o + M * N].view(M, N) for o, (M, N) in zip(y_off, shapes)]
+        n_words = torch.tensor([M * N // 8 for M, N in shapes], dtype=torch.int64)
+        counts = (n_words + per - 1) // per
+        start = torch.cat([torch.zeros(1, dtype=torch.int64), torch.cumsum(counts, 0)])
+        owner = torch.repeat_interleave(torch.arange(len(shapes)), counts)
+        local = torch.arange(int(start[-1]), dtype=torch.int64) - start[owner]
+        pbase = torch.tensor([p.data_ptr() for p in self.packeds], dtype=torch.int64)
+        sbase = torch.tensor([sc.data_ptr() for sc in self.scales], dtype=torch.int64)
+        ybase = torch.tensor([y.data_ptr() for y in self.outputs], dtype=torch.int64)
+        items = torch.stack([pbase[owner] + local * (per * 4), sbase[owner] + local * (per * 8 // self.group * 2),
+                             ybase[owner] + local * (per * 16), torch.clamp(n_words[owner] - local * per, max=per)], dim=1)
+        self.total_items = int(start[-1])
+        self._items = items.contiguous().to(self.device)
+        self.bf16_bytes = 2 * sum(M * N for M, N in shapes)
+
+    def run(self):
+        with torch.cuda.device(self.device):
+            rc = _lib.load().wq_int4_dequant_items(self._items.data_ptr(), self.total_items, self.group,
+                                                   _lib.stream_ptr(self.device))
+        _lib.check(rc, "Int4DequantPlan.run")
+        return self.outputs
+
+
 class _FakeInt4QuantizationSTE(torch.autograd.Function):
     """Quantise-dequantise forward, identity backward (docker/patch/latest/megatron.patch:212-255)."""
 

@@ -21,7 +21,7 @@ from collections import defaultdict
 import torch
 from safetensors import safe_open
 
-from ..int4 import dequantize_int4
+from ..int4 import Int4DequantPlan, dequantize_int4
 from . import _shards
 
 _PROJECTIONS = ("gate_proj", "up_proj", "down_proj")
@@ -65,6 +65,7 @@ def convert_file(input_path: str, output_path: str, group_size: int, skip_existi
             continue
         at = parts.index("experts")
         experts[".".join(parts[:at + 2])][parts[-2]][parts[-1]] = tensor
+    names, packeds, scales, shapes = [], [], [], []
     for prefix, components in experts.items():
         for proj in _PROJECTIONS:
             data = components.get(proj, {})
@@ -72,9 +73,26 @@ def convert_file(input_path: str, output_path: str, group_size: int, skip_existi
                 for suffix, value in data.items():          # incomplete: stays quantized
                     tensors[f"{prefix}.{proj}.{suffix}"] = value
                 continue
-            weight = _dequantize_tensor(_shards.to_device(data["weight_packed"], dev),
-                                        _shards.to_device(data["weight_scale"], dev), data["weight_shape"], group_size)
-            tensors[f"{prefix}.{proj}.weight"] = weight.cpu()
+            if data["weight_scale"].dtype != torch.bfloat16:
+                raise TypeError(f"{prefix}.{proj}.weight_scale must be bfloat16 (what pack-quantized checkpoints store), "
+                                f"got {data['weight_scale'].dtype}")
+            names.append(f"{prefix}.{proj}.weight")
+            packeds.append(_shards.to_device(data["weight_packed"].to(torch.int32), dev))
+            scales.append(_shards.to_device(data["weight_scale"], dev))
+            shapes.append(data["weight_shape"])
+    if names:
+        if group_size <= 0 or group_size & (group_size - 1):
+            # not a power of two: one kernel launch per tensor
+            for name, p, sc, sh in zip(names, packeds, scales, shapes):
+                tensors[name] = _dequantize_tensor(p, sc, sh, group_size).cpu()
+        else:
+            plan = Int4DequantPlan(packeds, scales, shapes, group_size)     # one launch and one copy for the shard
+            plan.run()
+            flat = plan.flat_y.cpu()
+            base = plan.flat_y.data_ptr()
+            for name, y in zip(names, plan.outputs):
+                off = (y.data_ptr() - base) // 2
+                tensors[name] = flat[off:off + y.numel()].view(y.shape)
     os.makedirs(os.path.dirname(output_path), exist_ok=True)
     _shards.write_shard(tensors, output_path, with_format_tag=False)
 

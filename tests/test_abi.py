@@ -72,6 +72,9 @@ def test_argument_validation_without_launch():
     assert lib.wq_int4_dequant(None, None, None, 4, 128, 12, None) == S
     assert lib.wq_int4_dequant(None, None, None, 4, 128, 128, None) == N_
     assert lib.wq_int4_dequant(None, None, None, 0, 128, 128, None) == 0
+    assert lib.wq_int4_dequant_items(None, 3, 128, None) == N_
+    assert lib.wq_int4_dequant_items(None, 3, 96, None) == S
+    assert lib.wq_int4_dequant_items(None, 0, 128, None) == 0
     assert lib.wq_int4_fake_quant_ste(None, None, 4, 100, 128, 0, None) == S
     assert lib.wq_int4_fake_quant_ste(None, None, 4, 96, 96, 0, None) == U
     assert lib.wq_int4_fake_quant_ste(None, None, 4, 128, 128, 5, None) == M_

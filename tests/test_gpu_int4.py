@@ -444,3 +444,17 @@ def test_fake_ste_many_scales_both_rules(cuda):
         with slime_amd.torch_arithmetic(arith):
             y = slime_amd.fake_int4_quantization_ste(w.to(cuda), 128)
         assert I.same_bits(y.cpu(), C.int4_fake_ste(w, 128, div7)), arith
+
+
+def test_int4_dequant_plan(cuda):
+    shapes = [(96, 256), (33, 768), (1, 128), (64, 128), (7, 7168), (128, 2048), (5, 384), (200, 1024), (63, 128), (768, 2048)]
+    for gs in (128, 32):
+        trip = [C.int4_pack_layer(I.weights(*sh, seed=400 + i), gs, True)[:2] for i, sh in enumerate(shapes)]
+        plan = slime_amd.Int4DequantPlan([p.to(cuda) for p, _ in trip], [s.to(cuda) for _, s in trip],
+                                         [torch.tensor(sh) for sh in shapes], gs)
+        for (p, s), sh, y in zip(trip, shapes, plan.run()):
+            assert tuple(y.shape) == sh and I.same_bits(y.cpu(), C.int4_dequant(p, s, sh, gs))
+    with pytest.raises(ValueError):
+        slime_amd.Int4DequantPlan([trip[0][0].to(cuda)], [trip[0][1].to(cuda)], [shapes[0]], 96)
+    with pytest.raises(ValueError):
+        slime_amd.Int4DequantPlan([trip[0][0].to(cuda)], [trip[0][1].to(cuda)], [(96, 512)], 32)
