@@ -28,8 +28,14 @@ class BucketPipeline:
 
     ``process(buckets)`` takes an iterable of CPU tensors (any dtype, contiguous) and yields, in order, tuples of
     CPU tensors holding the kernel's outputs.  Input buckets must not exceed ``max_in_bytes``; each output must
-    not exceed ``max_out_bytes``.  The yielded tensors are views of pinned staging buffers that are reused
-    ``depth`` buckets later: consume (or copy) them before advancing the iterator ``depth`` more times.
+    not exceed ``max_out_bytes``.
+
+    Buffer lifetimes.  The yielded tensors are views of pinned staging buffers, of which there are ``depth + 1``
+    sets: a result stays intact while the iterator is advanced ONCE more (so the previous result may be held while
+    the current one is worked on) and is overwritten, asynchronously, from the second advance on - copy what has to
+    live longer.  Input staging: ``staging_buffer(slot)`` of bucket ``i`` is ``slot = i % depth``; ``process`` pulls
+    bucket ``i`` from the iterable only after bucket ``i - depth`` (the previous user of that slot) has completely
+    left the GPU, so a generator may refill the buffer right before yielding it.
     """
 
     def __init__(self, device: torch.device, kernel: Callable[[torch.Tensor], tuple], max_in_bytes: int,
@@ -40,13 +46,15 @@ class BucketPipeline:
         self.max_in_bytes, self.max_out_bytes = int(max_in_bytes), int(max_out_bytes)
         self.h_in = [torch.empty(self.max_in_bytes, dtype=torch.uint8, pin_memory=True) for _ in range(depth)]
         self.d_in = [torch.empty(self.max_in_bytes, dtype=torch.uint8, device=device) for _ in range(depth)]
+        # one more set of output buffers than buckets in flight: the set of the result handed out last is not the
+        # one the next bucket downloads into
         self.h_out = [[torch.empty(self.max_out_bytes, dtype=torch.uint8, pin_memory=True) for _ in range(n_outputs)]
-                      for _ in range(depth)] if download else None
+                      for _ in range(depth + 1)] if download else None
         self.up = torch.cuda.Stream(device)
         self.down = torch.cuda.Stream(device)
         self.ev_uploaded = [torch.cuda.Event() for _ in range(depth)]
         self.ev_computed = [torch.cuda.Event() for _ in range(depth)]
-        self.ev_downloaded = [torch.cuda.Event() for _ in range(depth)]
+        self.ev_downloaded = [torch.cuda.Event() for _ in range(depth + 1)]
         self.kernel_events = []   # (start, end) pairs when time_kernels is set
         self.time_kernels = False
 
@@ -68,18 +76,19 @@ class BucketPipeline:
 
     def process(self, buckets: Iterable[torch.Tensor]) -> Iterator[tuple]:
         compute = torch.cuda.current_stream(self.device)
-        pending = []  # (slot, outputs on device, shapes/dtypes)
+        pending = []  # (input slot, output slot, outputs on device, their pinned host views)
         it = iter(buckets)
         i = 0
         while True:
+            slot = i % self.depth
+            if i >= self.depth:
+                # the slot is reused: its previous bucket must have left the GPU (uploaded, computed, downloaded) before
+                # the iterable is asked for the next bucket - it may refill this slot's staging buffer
+                yield self._finish(pending.pop(0))
             try:
                 bucket = next(it)
             except StopIteration:
                 break
-            slot = i % self.depth
-            if i >= self.depth:
-                # the slot is reused: its previous bucket must be fully consumed (downloaded or at least computed)
-                yield self._finish(pending.pop(0))
             staged = self._stage(slot, bucket)
             if i >= self.depth:
                 # d_in[slot] may be overwritten only after the kernel of its previous bucket has read it
@@ -101,26 +110,27 @@ class BucketPipeline:
             host_outs = None
             if self.download:
                 self.down.wait_event(self.ev_computed[slot])
+                oslot = i % (self.depth + 1)
                 host_outs = []
                 with torch.cuda.stream(self.down):
                     for k, o in enumerate(outs):
                         nbytes = o.numel() * o.element_size()
                         if nbytes > self.max_out_bytes:
                             raise ValueError(f"output of {nbytes} bytes exceeds the pipeline's {self.max_out_bytes}")
-                        h = self.h_out[slot][k][:nbytes]
+                        h = self.h_out[oslot][k][:nbytes]
                         h.copy_(o.contiguous().view(-1).view(torch.uint8), non_blocking=True)
                         o.record_stream(self.down)
                         host_outs.append(h.view(o.dtype).view(o.shape))
-                    self.ev_downloaded[slot].record(self.down)
-            pending.append((slot, outs, host_outs))
+                    self.ev_downloaded[oslot].record(self.down)
+            pending.append((slot, oslot if self.download else None, outs, host_outs))
             i += 1
         while pending:
             yield self._finish(pending.pop(0))
 
     def _finish(self, item):
-        slot, outs, host_outs = item
+        slot, oslot, outs, host_outs = item
         if self.download:
-            self.ev_downloaded[slot].synchronize()
+            self.ev_downloaded[oslot].synchronize()
             return tuple(host_outs)
         self.ev_computed[slot].synchronize()
         return tuple(outs)

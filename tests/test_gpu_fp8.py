@@ -70,10 +70,15 @@ def test_block_quant_config1_roundtrip(cuda, mode):
     assert ((d.cpu().float() - w.float()).abs() <= step / 2 * 1.01 + w.float().abs() * 2.0 ** -7).all()
 
 
-def test_block_quant_tall_ragged(cuda):
+@pytest.fixture(scope="module")
+def tall_ragged():
     # [151937, 2560]: vocabulary-sized, 1-row remainder block row
-    w = I.weights(151937, 2560, seed=5, outlier_p=0)
-    _check_block(w, w.to(cuda), mode=DEFAULT_MODE)
+    return I.zero_blocks(I.weights(151937, 2560, seed=5), 0.2, seed=6)
+
+
+@pytest.mark.parametrize("mode", [0, 1, 2])
+def test_block_quant_tall_ragged(cuda, tall_ragged, mode):
+    _check_block(tall_ragged, tall_ragged.to(cuda), mode=mode)
 
 
 @pytest.mark.parametrize("block", [(32, 32), (64, 128), (128, 64), (1, 128), (16, 48), (256, 256)])
@@ -132,14 +137,19 @@ def test_block_quant_every_bf16_value(cuda):
             _check_block(x, x.to(cuda), mode=mode)
 
 
-def test_block_quant_nan_inf(cuda):
+@pytest.mark.parametrize("mode", [0, 1, 2])
+def test_block_quant_nan_inf(cuda, mode):
     w = I.weights(128, 384, seed=6)
     w[5, 5] = float("nan")
     w[9, 130] = float("inf")
     w[10, 131] = -float("inf")
-    q, s = slime_amd.block_fp8(w.to(cuda), (128, 128))
+    if mode == 1:
+        q, s = slime_amd.blockwise_cast_to_fp8_triton(w.to(cuda), (128, 128))
+    else:
+        with slime_amd.torch_arithmetic(ARITH[mode]):
+            q, s = slime_amd.block_fp8(w.to(cuda), (128, 128))
     q, s = _codes(q), s.cpu()
-    qo, so = C.fp8_block_quant(w, (128, 128), DEFAULT_MODE)
+    qo, so = C.fp8_block_quant(w, (128, 128), mode)
     assert s[0, 0].isnan() and ((q[:, :128] & 0x7F) == 0x7F).all()
     assert s[0, 1].isinf()
     nan_o = (qo & 0x7F) == 0x7F
@@ -197,7 +207,7 @@ def test_dequant_all_codes(cuda):
 
 
 @pytest.mark.parametrize("shape", [(256, 256), (300, 200), (7, 7168), (129, 1), (2048, 7168), (7168, 2048), (16, 1024),
-                                   (17, 1040), (5, 1000)])
+                                   (17, 1040), (5, 1000), (4100, 3000), (151937, 2560)])
 def test_dequant_shapes(cuda, shape):
     x = I.fp8_codes(*shape, seed=shape[0])
     s = I.log_uniform_scales(-(-shape[0] // 128), -(-shape[1] // 128), seed=shape[1])

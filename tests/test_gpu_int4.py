@@ -65,6 +65,38 @@ def test_pack_layer_strided_rows(cuda):
         assert torch.equal(p.cpu(), po) and I.same_bits(s.cpu(), so)
 
 
+@pytest.fixture(scope="module")
+def vocab_ragged():
+    # [151937, 2560]: N is a multiple of 128, so the reference accepts it; M is not a multiple of 8
+    w = I.weights(151937, 2560, seed=11)
+    w[::1000, :128] = 0
+    return w
+
+
+def test_pack_layer_vocab_ragged_sym(cuda, vocab_ragged):
+    _check_pack(vocab_ragged, cuda)
+
+
+@pytest.mark.parametrize("sym", [True, False])
+def test_fake_quant_vocab_ragged(cuda, vocab_ragged, sym):
+    q, s, z = slime_amd.fake_int4_quant_cuda(vocab_ragged.to(cuda), (1, 128), sym)
+    assert s.shape == (151937, 20)
+    qo, so, zo = C.int4_fake_quant(vocab_ragged, (1, 128), sym)
+    assert I.same_bits(q.cpu(), qo) and I.same_bits(s.cpu(), so) and I.same_bits(z.cpu(), zo)
+
+
+def test_pack_layer_vocab_ragged_asym(cuda, vocab_ragged):
+    # asymmetric: the zero points are packed eight ROWS to a word, and 151937 rows do not divide by 8 - the
+    # reference fails in zeros.reshape(-1, zeros.shape[1] // 8, 8) (convert_hf_to_int4_direct.py:137), and so does this
+    with pytest.raises(RuntimeError, match="invalid for input of size"):
+        slime_amd.pack_layer(vocab_ragged.to(cuda), 128, False)
+    # the largest multiple of 8 rows goes through, bit for bit
+    w = vocab_ragged[:151936]
+    p, s, z = slime_amd.pack_layer(w.to(cuda), 128, False)
+    po, so, zo = C.int4_pack_layer(w, 128, False)
+    assert torch.equal(p.cpu(), po) and I.same_bits(s.cpu(), so) and torch.equal(z.cpu(), zo)
+
+
 def test_pack_layer_ragged_n_fails_like_reference(cuda):
     w = I.weights(4100, 3000, seed=1).to(cuda)
     with pytest.raises(RuntimeError):
