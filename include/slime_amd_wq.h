@@ -8,7 +8,8 @@
  *     marked "host".  Sizes and strides are in ELEMENTS.  `stream` is a hipStream_t passed
  *     as void*; NULL selects the default stream.  Launches are asynchronous and are ordered
  *     on `stream` only; the library keeps no mutable global state and every entry point may
- *     be called concurrently from several host threads.
+ *     be called concurrently from several host threads (one exception, documented there:
+ *     wq_delta_xor_noalloc works in a device array owned by the library).
  *   - Return value: 0 on success, a negative WQ_ERR_* for rejected arguments (nothing was
  *     launched), or a positive hipError_t reported by the launch.  wq_error_string() names any
  *     of them.
@@ -29,7 +30,7 @@
 extern "C" {
 #endif
 
-#define WQ_ABI_VERSION 8
+#define WQ_ABI_VERSION 9
 
 enum {
     WQ_OK = 0,
@@ -243,6 +244,19 @@ int wq_delta_xor(const void *new_bytes, void *old_bytes, void *diff, int64_t n, 
                  void *workspace, uint64_t *result, void *stream);
 int wq_delta_overwrite_encode(const void *new_bytes, const void *old_bytes, int64_t n, void *workspace,
                               uint32_t count, void *out, void *stream);
+
+/* wq_delta_xor without the workspace argument, for callers that cannot allocate device memory (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.
+ * The per-chunk partial sums go to a device array inside the library (24 bytes per WQ_DELTA_CHUNK of input,
+ * 6 MiB per GPU, held until the process ends); the call allocates and frees nothing.  n may not exceed
+ * WQ_DELTA_NOALLOC_MAX_BYTES (WQ_ERR_TOO_LARGE otherwise; split larger tensors).  Arguments, alignment rules and
+ * results are those of wq_delta_xor.  All calls on one GPU share the array: calls that may overlap on one GPU
+ * (different streams, or several host threads) race - order them on one stream.  Nothing has to be cleared
+ * between calls.  The first call on a device looks up the array's address (no stream work); make that call
+ * outside a graph capture.  The array does not hold the scan slots of wq_delta_overwrite_encode. */
+#define WQ_DELTA_NOALLOC_MAX_BYTES (4294967296LL)
+int wq_delta_xor_noalloc(const void *new_bytes, void *old_bytes, void *diff, int64_t n, int update_old,
+                         uint64_t *result, void *stream);
 
 /* wq_delta_xor over a bucket of tensors with two launches in total (the shape a weight-sync bucket wants:
  * update_weight_from_disk_delta.py:252-270 walks the gathered tensors one by one).  `descs` is a DEVICE array

@@ -15,7 +15,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libslime_amd_wq.so")
 
-ABI_VERSION = 8
+ABI_VERSION = 9
 
 # selectors (mirrors of the header's enums)
 DTYPE_BF16, DTYPE_F32, DTYPE_F16 = 0, 1, 2
@@ -51,6 +51,7 @@ SIGNATURES = {
     "wq_delta_workspace_bytes": [_i64],
     "wq_delta_xor": [_vp, _vp, _vp, _i64, _int, _vp, _vp, _vp],
     "wq_delta_overwrite_encode": [_vp, _vp, _i64, _vp, ctypes.c_uint32, _vp, _vp],
+    "wq_delta_xor_noalloc": [_vp, _vp, _vp, _i64, _int, _vp, _vp],
     "wq_delta_xor_grouped": [_vp, _vp, _int, _i64, _int, _int, _vp],
     "wq_selftest_fp8_elem": [_u32, _u32, _int, _vp, _vp],
     "wq_selftest_int4_elem": [_u32, _u32, _vp, _vp],

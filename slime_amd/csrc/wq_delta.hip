@@ -14,6 +14,8 @@
 // as a three-step stream compaction: per-chunk counts (from the pass above), an exclusive scan of them,
 // and a scatter in which each lane ranks its changed bytes with a wave prefix sum.
 
+#include <atomic>
+
 #include "wq_common.h"
 
 namespace wq {
@@ -380,6 +382,49 @@ WQ_EXPORT int wq_delta_xor(const void* new_bytes, void* old_bytes, void* diff, i
     delta_fold_kernel<false><<<1, kFoldThreads, 0, st>>>(a);
     WQ_LAUNCH_CHECK();
     return WQ_OK;
+}
+
+// ---- the same pass for callers that cannot allocate ------------------------------------------------------
+// The per-chunk partial sums live in a file-scope device array instead of a caller workspace.  Every GPU has its
+// own copy of the array at its own address; the address is looked up once per device, with that device current,
+// and only that pointer is ever handed to kernels (the array's name is a host-side handle, not a device address).
+constexpr int64_t kStaticMaxBytes = WQ_DELTA_NOALLOC_MAX_BYTES;
+constexpr int64_t kStaticRows = kStaticMaxBytes / kDeltaChunk;
+static __device__ __align__(256) uint64_t scratch[kStaticRows * 3];
+
+constexpr int kMaxDevices = 64;
+static std::atomic<uint64_t*> g_scratch_ptr[kMaxDevices];
+
+static int static_scratch(uint64_t** out)
+{
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= kMaxDevices) return WQ_ERR_UNSUPPORTED;
+    uint64_t* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!p) {
+        void* sym = nullptr;
+        e = hipGetSymbolAddress(&sym, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return (int)e;
+        if (!sym) return WQ_ERR_NULL;
+        p = (uint64_t*)sym;
+        g_scratch_ptr[dev].store(p, std::memory_order_release);   // racing threads store the same value
+    }
+    *out = p;
+    return WQ_OK;
+}
+
+WQ_EXPORT int wq_delta_xor_noalloc(const void* new_bytes, void* old_bytes, void* diff, int64_t n, int update_old,
+                                   uint64_t* result, void* stream)
+{
+    if (n < 0) return WQ_ERR_SHAPE;
+    if (n > kStaticMaxBytes) return WQ_ERR_TOO_LARGE;
+    if (!result) return WQ_ERR_NULL;
+    uint64_t* ws = nullptr;
+    const int rc = static_scratch(&ws);
+    if (rc) return rc;
+    // every chunk row that the fold reads is written by this call's first kernel: nothing to clear
+    return wq_delta_xor(new_bytes, old_bytes, diff, n, update_old, ws, result, stream);
 }
 
 WQ_EXPORT int wq_delta_xor_grouped(const wq_delta_desc* descs, const int64_t* chunk_start, int n_desc,
