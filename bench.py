@@ -1,16 +1,15 @@
-"""Benchmark of the weight-conversion hot path on one MI355X.
+"""Benchmark of the low-precision weight-conversion path on one MI355X.
 
-Headline workload (the "step"): one full weight-sync quantisation pass over a Qwen3-4B-shaped bf16 state
-dict - 36 layers x {q [4096,2560], k, v [1024,2560], o [2560,4096], gate, up [9728,2560], down [2560,9728]},
-252 tensors, 7.27 GB of bf16 - block-FP8 (128x128, e4m3fn, fp32 scale_inv) with the arithmetic of the
-reference's block_fp8, as ONE grouped kernel launch writing into a flat output bucket.  Inputs are resident
-in HBM before the timed region; weights are synthetic N(0, 0.02) generated on the device.
-
-Prints ONE JSON line.  `roofline` prices the kernel against the 8 TB/s HBM peak from the algorithmic bytes
-(2 B read + 1 B written per element + 4 B of scale per 128x128 block) and the kernel duration measured with
-HIP events on the launch stream.  `cpu_baseline` times the CPU restatement of the reference's torch path on
-this box's host cores on a bounded sample (one layer's seven tensors, repeated).  `other_workloads` adds the
-INT4 pack (Qwen3-30B-A3B experts) and FP8 dequant (DeepSeek-V3 MoE layer) kernels, measured the same way.
+`python bench.py --gpus 1 --steps K --warmup W` prints ONE JSON line.  A step is one conversion pass over a
+Qwen3-30B-A3B-shaped bf16 state dict resident in HBM into BOTH rollout formats: block-FP8 128x128 of all 18 624 linear
+weights (one grouped launch), then symmetric group-128 INT4 pack of the 18 432 expert weights (one grouped launch).
+`value` = bf16 bytes quantised per second over the timed region (wall clock around K steps); `roofline` describes the
+kernel of the step with the LOWER fraction of the HBM peak (both are listed under `roofline_kernels`), from its
+algorithmic bytes and its mean launch time measured with HIP events on the launch stream.  `cpu_baseline` times the
+CPU restatement of the reference's torch path on this box's host cores on bounded samples of the same tensors (the
+mix of the step, and per leg).  `other_workloads` holds the remaining configurations (Qwen3-4B state dict, the
+[4096,4096] matrix, FP8 -> bf16 of a DeepSeek-V3 layer, INT4 -> bf16, the QAT forward, delta sync, single-tensor forms
+and the bucket-level weight-sync drop-in), measured the same way.
 """
 
 from __future__ import annotations
@@ -32,24 +31,32 @@ QWEN3_4B_LAYER = [("q_proj", 4096, 2560), ("k_proj", 1024, 2560), ("v_proj", 102
 QWEN3_4B_LAYERS = 36
 
 
-def _time_launches(run, steps: int, warmup: int):
-    """-> (wall ms per step over the whole timed region, mean per-launch ms from HIP events)."""
+def _time_step(runs, steps: int, warmup: int):
+    """A step = the callables of `runs` in order.  -> (wall ms per step over the whole timed region, [mean ms per run],
+    [min ms per run]); the per-run times come from HIP events recorded on the current stream around each run."""
     import torch
 
     for _ in range(warmup):
-        run()
+        for run in runs:
+            run()
     torch.cuda.synchronize()
-    starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
-    ends = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    marks = [[torch.cuda.Event(enable_timing=True) for _ in range(len(runs) + 1)] for _ in range(steps)]
     t0 = time.perf_counter()
     for i in range(steps):
-        starts[i].record()
-        run()
-        ends[i].record()
+        marks[i][0].record()
+        for k, run in enumerate(runs):
+            run()
+            marks[i][k + 1].record()
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / steps
-    ev = [s.elapsed_time(e) for s, e in zip(starts, ends)]
-    return wall_ms, sum(ev) / len(ev), min(ev)
+    per = [[m[k].elapsed_time(m[k + 1]) for m in marks] for k in range(len(runs))]
+    return wall_ms, [sum(v) / len(v) for v in per], [min(v) for v in per]
+
+
+def _time_launches(run, steps: int, warmup: int):
+    """-> (wall ms per step over the whole timed region, mean per-launch ms from HIP events, min)."""
+    wall_ms, mean, mn = _time_step([run], steps, warmup)
+    return wall_ms, mean[0], mn[0]
 
 
 def _gen_bf16(shape, device, std=0.02, outliers=False):
@@ -63,54 +70,195 @@ def _gen_bf16(shape, device, std=0.02, outliers=False):
     return w
 
 
-def _traffic_from_profile(name: str):
-    """HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, if a summary with a
-    `traffic_bytes_per_launch:` line has been committed under profiles/ for this kernel and workload."""
+def kernel_source_hash(*files: str) -> str:
+    """sha256 over the named files of slime_amd/csrc (a kernel's source and the shared header)."""
+    import hashlib
+
+    h = hashlib.sha256()
+    for f in files:
+        with open(os.path.join(ROOT, "slime_amd", "csrc", f), "rb") as fh:
+            h.update(fh.read())
+    return h.hexdigest()
+
+
+KERNEL_SOURCES = {
+    "fp8_block_quant": ("wq_fp8_quant.hip", "wq_common.h"),
+    "int4_pack": ("wq_int4.hip", "wq_common.h"),
+    "fp8_block_dequant": ("wq_fp8_dequant.hip", "wq_common.h"),
+    "int4_dequant": ("wq_int4_dequant.hip", "wq_common.h"),
+    "delta_xor": ("wq_delta.hip", "wq_common.h"),
+}
+
+
+def _traffic_from_profile(name: str, kernel: str):
+    """HBM bytes per launch that rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE measured for this kernel and workload, from
+    the summary committed under profiles/ - a separate run, not this one.  The summary records the sha256 of the
+    kernel's source; when the source has changed since, the figure is stale and is NOT reported.
+    -> (bytes or None, note)."""
     path = os.path.join(ROOT, "profiles", name)
+    traffic = recorded = None
     try:
         with open(path) as f:
             for line in f:
                 if line.startswith("traffic_bytes_per_launch:"):
-                    return float(line.split(":", 1)[1].split()[0])
+                    traffic = float(line.split(":", 1)[1].split()[0])
+                elif line.startswith("kernel_source_sha256:"):
+                    recorded = line.split(":", 1)[1].split()[0]
     except OSError:
-        pass
-    return None
+        return None, f"profiles/{name} not found"
+    if traffic is None:
+        return None, f"profiles/{name} holds no traffic figure"
+    current = kernel_source_hash(*KERNEL_SOURCES[kernel])
+    if recorded != current:
+        return None, (f"profiles/{name} was taken on another version of the kernel source "
+                      f"(recorded {str(recorded)[:12]}, now {current[:12]}): figure withheld")
+    return traffic, f"profiles/{name} (rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE, separate run; kernel source {current[:12]} unchanged since)"
 
 
-def bench_fp8_quant(dev, steps, warmup):
+def _moe_state_dict(dev, layers, experts=128):
+    """Qwen3-30B-A3B-shaped linear weights: per layer 128 experts x (gate, up [768,2048], down [2048,768]) as views of
+    one allocation per projection (the layout of a grouped-GEMM weight), plus q [4096,2048], k, v [512,2048],
+    o [2048,4096].  -> (all weights in state-dict order, the expert weights only)."""
+    weights, expert_weights = [], []
+    for _ in range(layers):
+        gate = _gen_bf16((experts, 768, 2048), dev, outliers=True)
+        up = _gen_bf16((experts, 768, 2048), dev, outliers=True)
+        down = _gen_bf16((experts, 2048, 768), dev, outliers=True)
+        for e in range(experts):
+            expert_weights += [gate[e], up[e], down[e]]
+            weights += [gate[e], up[e], down[e]]
+        weights += [_gen_bf16(sh, dev) for sh in ((4096, 2048), (512, 2048), (512, 2048), (2048, 4096))]
+    return weights, expert_weights
+
+
+def bench_north_star(dev, steps, warmup, layers):
+    """One conversion pass over the Qwen3-30B-A3B-shaped state dict into both formats: block-FP8 of every linear
+    weight, then INT4 pack of the expert weights.  Two grouped launches per step."""
     import torch
 
     import slime_amd
     from oracle import c_oracle
 
-    weights, names = [], []
-    for layer in range(QWEN3_4B_LAYERS):
-        for n, M, N in QWEN3_4B_LAYER:
-            weights.append(_gen_bf16((M, N), dev))
-            names.append(f"model.layers.{layer}.{n}.weight")
-    plan = slime_amd.Fp8QuantPlan(weights, (128, 128))
-    wall_ms, ev_ms, ev_min = _time_launches(plan.run, steps, warmup)
+    weights, expert_weights = _moe_state_dict(dev, layers)
+    fp8_plan = slime_amd.Fp8QuantPlan(weights, (128, 128))
+    int4_plan = slime_amd.Int4PackPlan(expert_weights, 128)
+    wall_ms, mean, mn = _time_step([fp8_plan.run, int4_plan.run], steps, warmup)
 
-    elements = sum(w.numel() for w in weights)
-    blocks = plan.total_tiles
-    algo_bytes = 3 * elements + 4 * blocks
-    bf16_bytes = 2 * elements
-
+    el_fp8 = sum(w.numel() for w in weights)
+    el_int4 = sum(w.numel() for w in expert_weights)
+    algo_fp8 = 3 * el_fp8 + 4 * fp8_plan.total_tiles
+    algo_int4 = 2 * el_int4 + el_int4 // 2 + el_int4 // 128 * 2
     # parity on a sample of the very tensors that were timed
     checked = 0
-    for idx in (0, 1, 3, 6, len(weights) - 1):
+    for idx in (0, 2, 385, len(weights) - 1):
+        q, s = fp8_plan.outputs[idx]
+        qo, so = c_oracle.fp8_block_quant(weights[idx].cpu().contiguous(), (128, 128), fp8_plan.mode)
+        assert torch.equal(q.cpu().view(torch.uint8), qo), f"FP8 parity failure on tensor {idx}"
+        assert torch.equal(s.cpu().view(torch.int32), so.view(torch.int32)), f"FP8 scale parity failure on tensor {idx}"
+        checked += 1
+    for idx in (0, 2, len(expert_weights) - 1):
+        p, s = int4_plan.outputs[idx]
+        po, so, _ = c_oracle.int4_pack_layer(expert_weights[idx].cpu().contiguous(), 128, True)
+        assert torch.equal(p.cpu(), po), f"INT4 parity failure on tensor {idx}"
+        assert torch.equal(s.cpu().view(torch.int16), so.view(torch.int16)), f"INT4 scale parity failure on tensor {idx}"
+        checked += 1
+    out = {"wall_ms": wall_ms, "layers": layers, "tensors_fp8": len(weights), "tensors_int4": len(expert_weights),
+           "bf16_bytes": 2 * (el_fp8 + el_int4), "parity_tensors_checked": checked,
+           "fp8": {"kernel_ms": mean[0], "kernel_ms_min": mn[0], "elements": el_fp8, "blocks": fp8_plan.total_tiles,
+                   "algo_bytes": algo_fp8, "mode": fp8_plan.mode},
+           "int4": {"kernel_ms": mean[1], "kernel_ms_min": mn[1], "elements": el_int4, "algo_bytes": algo_int4}}
+    del fp8_plan, int4_plan, weights, expert_weights
+    torch.cuda.empty_cache()
+    return out
+
+
+def bench_fp8_quant(dev, steps, warmup):
+    """Block-FP8 quant of every linear weight of a Qwen3-4B-shaped state dict (252 tensors, 7.27 GB), one launch."""
+    import torch
+
+    import slime_amd
+    from oracle import c_oracle
+
+    weights = [_gen_bf16((M, N), dev) for _ in range(QWEN3_4B_LAYERS) for _, M, N in QWEN3_4B_LAYER]
+    plan = slime_amd.Fp8QuantPlan(weights, (128, 128))
+    wall_ms, ev_ms, ev_min = _time_launches(plan.run, steps, warmup)
+    elements = sum(w.numel() for w in weights)
+    algo_bytes = 3 * elements + 4 * plan.total_tiles
+    for idx in (0, 1, 3, 6, len(weights) - 1):      # parity on a sample of the very tensors that were timed
         q, s = plan.outputs[idx]
         qo, so = c_oracle.fp8_block_quant(weights[idx].cpu(), (128, 128), plan.mode)
-        assert torch.equal(q.cpu().view(torch.uint8), qo), f"parity failure on {names[idx]}"
-        assert torch.equal(s.cpu().view(torch.int32), so.view(torch.int32)), f"scale parity failure on {names[idx]}"
-        checked += 1
-    sample = [w.cpu() for w in weights[:len(QWEN3_4B_LAYER)]]
+        assert torch.equal(q.cpu().view(torch.uint8), qo) and torch.equal(s.cpu().view(torch.int32), so.view(torch.int32))
+    traffic, note = _traffic_from_profile("fp8_block_quant_qwen3_4b_pmc.txt", "fp8_block_quant")
+    out = {"workload": "Qwen3-4B-shaped bf16 state dict, block-FP8 128x128 quant of all 252 linear weights (36 layers x "
+                       "q,k,v,o,gate,up,down), one grouped launch, block_fp8 arithmetic as torch evaluates it on GPU tensors",
+           "tensors": len(weights), "bf16_GB": 2 * elements / 1e9, "kernel_ms": ev_ms, "kernel_ms_min": ev_min,
+           "wall_ms": wall_ms, "bf16_GBps": 2 * elements / ev_ms / 1e6, "algo_GBps": algo_bytes / ev_ms / 1e6,
+           "hbm_frac": algo_bytes / ev_ms / 1e6 / HBM_PEAK_GBS, "algorithmic_bytes_per_launch": algo_bytes,
+           "traffic": traffic, "traffic_source": note, "parity_tensors_checked": 5}
     del plan, weights
     torch.cuda.empty_cache()
-    return {
-        "wall_ms": wall_ms, "kernel_ms": ev_ms, "kernel_ms_min": ev_min, "elements": elements, "blocks": blocks,
-        "algo_bytes": algo_bytes, "bf16_bytes": bf16_bytes, "parity_tensors_checked": checked, "cpu_sample": sample,
-    }
+    return out
+
+
+def bench_cfg1(dev, steps, warmup, n_buffers=8):
+    """The single [4096, 4096] matrix (N(0, 0.02), 0.1 % of entries x20): block-FP8 quant then dequant of its own
+    output.  One 100 MB round trip fits the last-level cache, so the timed loop cycles through `n_buffers` distinct
+    matrices (cold) and, separately, re-runs one (warm)."""
+    import torch
+
+    import slime_amd
+    from oracle import c_oracle
+    from slime_amd import _lib
+
+    lib = _lib.load()
+    M = N = 4096
+    g = torch.Generator().manual_seed(0)
+    w0 = torch.randn(M, N, generator=g) * 0.02
+    w0[torch.rand(M, N, generator=g) < 0.001] *= 20
+    w0 = w0.to(torch.bfloat16)
+    ws = [w0.to(dev)] + [_gen_bf16((M, N), dev, outliers=True) for _ in range(n_buffers - 1)]
+    qs = [torch.empty((M, N), dtype=torch.uint8, device=dev) for _ in ws]
+    ss = [torch.empty((M // 128, N // 128), dtype=torch.float32, device=dev) for _ in ws]
+    ys = [torch.empty((M, N), dtype=torch.bfloat16, device=dev) for _ in ws]
+    mode = slime_amd.arith.fp8_torch_mode()
+    st = _lib.stream_ptr(dev)
+    state = {"i": 0}
+
+    def quant(k):
+        _lib.check(lib.wq_fp8_block_quant(ws[k].data_ptr(), M, N, N, 1, qs[k].data_ptr(), N, ss[k].data_ptr(), 128, 128,
+                                          mode, st), "cfg1 quant")
+
+    def dequant(k):
+        _lib.check(lib.wq_fp8_block_dequant(qs[k].data_ptr(), ss[k].data_ptr(), ys[k].data_ptr(), _lib.DTYPE_BF16, M, N,
+                                            128, _lib.DEQ_MODE_F32SCALE, st), "cfg1 dequant")
+
+    def cold_quant():
+        state["i"] = (state["i"] + 1) % n_buffers
+        quant(state["i"])
+
+    def cold_dequant():
+        dequant(state["i"])
+
+    wall_c, mean_c, _ = _time_step([cold_quant, cold_dequant], max(steps, 2 * n_buffers), max(warmup, n_buffers))
+    wall_w, mean_w, _ = _time_step([lambda: quant(0), lambda: dequant(0)], max(steps, 2 * n_buffers), warmup)
+    qo, so = c_oracle.fp8_block_quant(w0, (128, 128), mode)
+    assert torch.equal(qs[0].cpu(), qo) and torch.equal(ss[0].cpu().view(torch.int32), so.view(torch.int32))
+    yo = c_oracle.fp8_block_dequant(qo, so, 128, 0)
+    assert torch.equal(ys[0].cpu().view(torch.int16), yo.view(torch.int16))
+    algo = 3 * M * N + 4 * (M // 128) * (N // 128)
+    out = {"workload": f"one bf16 [4096,4096] matrix, block-FP8 quant then dequant of its own output; cold = {n_buffers} "
+                       "distinct matrices cycled, warm = the same matrix every step; whole tensor checked against the oracle",
+           "quant_kernel_ms_cold": mean_c[0], "dequant_kernel_ms_cold": mean_c[1],
+           "quant_kernel_ms_warm": mean_w[0], "dequant_kernel_ms_warm": mean_w[1],
+           "quant_hbm_frac_cold": algo / mean_c[0] / 1e6 / HBM_PEAK_GBS,
+           "dequant_hbm_frac_cold": algo / mean_c[1] / 1e6 / HBM_PEAK_GBS,
+           "roundtrip_bf16_GBps_cold": 2 * M * N / (mean_c[0] + mean_c[1]) / 1e6,
+           "roundtrip_bf16_GBps_warm": 2 * M * N / (mean_w[0] + mean_w[1]) / 1e6,
+           "note": "32 MiB tensors: launch latency and the tail of 1024 workgroups over 256 CUs are visible; warm runs "
+                   "are served from the last-level cache, so their rate is not an HBM figure"}
+    del ws, qs, ss, ys
+    torch.cuda.empty_cache()
+    return out
 
 
 def bench_fp8_quant_moe(dev, steps, warmup, layers):
@@ -121,15 +269,7 @@ def bench_fp8_quant_moe(dev, steps, warmup, layers):
     import slime_amd
     from oracle import c_oracle
 
-    experts = 128
-    weights = []
-    for _ in range(layers):
-        gate = _gen_bf16((experts, 768, 2048), dev, outliers=True)
-        up = _gen_bf16((experts, 768, 2048), dev, outliers=True)
-        down = _gen_bf16((experts, 2048, 768), dev, outliers=True)
-        for e in range(experts):
-            weights += [gate[e], up[e], down[e]]
-        weights += [_gen_bf16(sh, dev) for sh in ((4096, 2048), (512, 2048), (512, 2048), (2048, 4096))]
+    weights, _ = _moe_state_dict(dev, layers)
     plan = slime_amd.Fp8QuantPlan(weights, (128, 128))
     wall_ms, ev_ms, ev_min = _time_launches(plan.run, steps, warmup)
     elements = sum(w.numel() for w in weights)
@@ -148,21 +288,87 @@ def bench_fp8_quant_moe(dev, steps, warmup, layers):
     return out
 
 
+def bench_bucket(dev, steps, warmup, layers):
+    """The weight-sync drop-in: the Qwen3-30B-A3B-shaped state dict after name conversion - per layer 128 experts
+    (gate/up as chunk views of one fc1 weight, down), q/k/v from one fused parameter, o, two norms and the router -
+    through BucketConverter, as ONE bucket (launches per sync = 1) and as one bucket per layer."""
+    import torch
+
+    from oracle import c_oracle
+    from slime_amd import bucket as B
+
+    cfg = {"quant_method": "fp8", "fmt": "e4m3", "activation_scheme": "dynamic", "weight_block_size": [128, 128]}
+    per_layer = []
+    for layer in range(layers):
+        L, hf = f"module.module.decoder.layers.{layer}.", f"model.layers.{layer}."
+        fc1 = _gen_bf16((128, 2 * 768, 2048), dev, outliers=True)
+        fc2 = _gen_bf16((128, 2048, 768), dev, outliers=True)
+        params = [(L + "self_attention.linear_qkv.layer_norm_weight", [(hf + "input_layernorm.weight", _gen_bf16((2048,), dev))]),
+                  (L + "self_attention.linear_qkv.weight", [(hf + "self_attn.q_proj.weight", _gen_bf16((4096, 2048), dev)),
+                                                          (hf + "self_attn.k_proj.weight", _gen_bf16((512, 2048), dev)),
+                                                          (hf + "self_attn.v_proj.weight", _gen_bf16((512, 2048), dev))]),
+                  (L + "self_attention.linear_proj.weight", [(hf + "self_attn.o_proj.weight", _gen_bf16((2048, 4096), dev))]),
+                  (L + "pre_mlp_layernorm.weight", [(hf + "post_attention_layernorm.weight", _gen_bf16((2048,), dev))]),
+                  (L + "mlp.router.weight", [(hf + "mlp.gate.weight", _gen_bf16((128, 2048), dev))])]
+        for e in range(128):
+            gate, up = fc1[e].chunk(2, dim=0)
+            params.append((L + f"mlp.experts.linear_fc1.weight{e}",
+                           [(hf + f"mlp.experts.{e}.gate_proj.weight", gate), (hf + f"mlp.experts.{e}.up_proj.weight", up)]))
+            params.append((L + f"mlp.experts.linear_fc2.weight{e}", [(hf + f"mlp.experts.{e}.down_proj.weight", fc2[e])]))
+        per_layer.append(params)
+    whole = [p for params in per_layer for p in params]
+    n_tensors = sum(len(cv) for _, cv in whole)
+    quantised = [(n, t) for _, cv in whole for n, t in cv if n.endswith("proj.weight")]
+    elements = sum(t.numel() for _, t in quantised)
+    algo_bytes = 3 * elements + 4 * sum((-(-t.shape[0] // 128)) * (-(-t.shape[1] // 128)) for _, t in quantised)
+    conv = B.BucketConverter(None, cfg)
+    state = {}
+
+    def one_bucket():
+        state["out"] = None                       # the previous sync's buffer goes back to the allocator first
+        state["out"] = conv.convert(whole, bucket_id="all")
+
+    def per_layer_buckets():
+        state["out"] = None
+        state["out"] = [conv.convert(params, bucket_id=i) for i, params in enumerate(per_layer)]
+
+    t0 = time.perf_counter()
+    one_bucket()
+    torch.cuda.synchronize()
+    first_ms = (time.perf_counter() - t0) * 1e3
+    wall1, ev1, _ = _time_launches(one_bucket, steps, warmup)
+    launches1 = state["out"].launches
+    named = dict(state["out"].reconstruct_tensors())
+    for n, t in (quantised[0], quantised[5], quantised[-1]):
+        qo, so = c_oracle.fp8_block_quant(t.cpu().contiguous(), (128, 128), 1)
+        assert torch.equal(named[n].cpu().view(torch.uint8), qo)
+        assert torch.equal(named[n.replace(".weight", ".weight_scale_inv")].cpu().view(torch.int32), so.view(torch.int32))
+    assert torch.equal(named["model.layers.0.mlp.gate.weight"], whole[4][1][0][1])
+    del named
+    wallL, evL, _ = _time_launches(per_layer_buckets, steps, warmup)
+    launchesL = sum(b.launches for b in state["out"])
+    out = {"workload": f"Qwen3-30B-A3B-shaped state dict after name conversion, {layers} layers, {n_tensors} tensors "
+                       f"({len(quantised)} quantised to block-FP8 with the weight-sync arithmetic, the rest copied), written "
+                       "into the one uint8 buffer + metadata a FlattenedTensorBucket consumer reads; fresh output buffer per sync",
+           "tensors": n_tensors, "bf16_GB": 2 * elements / 1e9,
+           "one_bucket": {"launches_per_sync": launches1, "ms_per_sync_gpu": ev1, "ms_per_sync_wall": wall1,
+                          "first_call_ms_table_build": first_ms, "hbm_frac": algo_bytes / ev1 / 1e6 / HBM_PEAK_GBS,
+                          "bf16_GBps": 2 * elements / ev1 / 1e6},
+           "bucket_per_layer": {"launches_per_sync": launchesL, "ms_per_sync_gpu": evL, "ms_per_sync_wall": wallL,
+                                "hbm_frac": algo_bytes / evL / 1e6 / HBM_PEAK_GBS, "bf16_GBps": 2 * elements / evL / 1e6},
+           "table_builds": conv.plan_builds, "parity_tensors_checked": 3}
+    del state, conv, whole, per_layer, quantised
+    torch.cuda.empty_cache()
+    return out
+
+
 def bench_int4_pack(dev, steps, warmup, layers):
     import torch
 
     import slime_amd
     from oracle import c_oracle
 
-    experts = 128
-    weights = []
-    for _ in range(layers):
-        # one allocation per layer and projection; experts are views, as in a grouped-GEMM weight
-        gate = _gen_bf16((experts, 768, 2048), dev, outliers=True)
-        up = _gen_bf16((experts, 768, 2048), dev, outliers=True)
-        down = _gen_bf16((experts, 2048, 768), dev, outliers=True)
-        for e in range(experts):
-            weights += [gate[e], up[e], down[e]]
+    _, weights = _moe_state_dict(dev, layers)
     plan = slime_amd.Int4PackPlan(weights, 128)
     wall_ms, ev_ms, ev_min = _time_launches(plan.run, steps, warmup)
     elements = sum(w.numel() for w in weights)
@@ -407,8 +613,34 @@ def bench_stream(dev, n_buckets=64, bucket_bytes=1 << 30, download=True):
             "kernel_only_GBps": total / (pipe.kernel_ms() / 1e3) / 1e9, "parity_buckets_checked": checked}
 
 
-def cpu_baseline(sample, budget_s: float):
-    """The CPU restatement of the reference torch path (block_fp8 op sequence) on one layer's tensors."""
+def _cpu_gen(shape, seed, outliers=True):
+    import torch
+
+    g = torch.Generator().manual_seed(seed)
+    w = torch.randn(shape, generator=g) * 0.02
+    if outliers:
+        w[torch.rand(shape, generator=g) < 1e-3] *= 20
+    return w.to(torch.bfloat16)
+
+
+def _cpu_rate(fn, nbytes, budget_s, max_reps=500):
+    """Runs fn (one pass over the sample) until the time budget is used.  -> (GB/s of bf16, passes, seconds)."""
+    fn()                                       # warm the allocator and the thread pool
+    reps, t0 = 0, time.perf_counter()
+    while True:
+        fn()
+        reps += 1
+        dt = time.perf_counter() - t0
+        if dt >= budget_s or reps >= max_reps:
+            break
+    return nbytes * reps / dt / 1e9, reps, dt
+
+
+def cpu_baselines(budget_s: float, north_star_bytes):
+    """The CPU restatements of the reference's torch path (oracle/torch_ref.py: the same op sequences as
+    convert_hf_to_fp8.block_fp8, convert_hf_to_int4_direct.pack_layer and fp8_cast_bf16.weight_dequant), timed on
+    this box's host cores on bounded samples of the benchmark's own tensor shapes.
+    -> (the `cpu_baseline` object of the headline step, {leg: record})."""
     import torch
 
     from oracle import torch_ref
@@ -416,21 +648,59 @@ def cpu_baseline(sample, budget_s: float):
     cores = os.cpu_count() or 1
     cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
     torch.set_num_threads(cores)
-    nbytes = sum(2 * w.numel() for w in sample)
-    for w in sample[1:3]:
-        torch_ref.block_fp8_ref(w, (128, 128))      # warm the allocator and thread pool
-    reps, t0 = 0, time.perf_counter()
-    while True:
-        for w in sample:
-            torch_ref.block_fp8_ref(w, (128, 128))
-        reps += 1
-        dt = time.perf_counter() - t0
-        if dt >= budget_s or reps >= 500:
-            break
-    return {"value": nbytes * reps / dt / 1e9, "unit": "GB/s of bf16 weights", "cores": torch.get_num_threads(),
-            "kind": "port",
-            "sample": f"layer 0 of the same state dict (7 tensors, {nbytes / 1e6:.0f} MB bf16) x {reps} passes, "
-                      f"{dt:.1f} s, torch CPU op-for-op restatement of block_fp8"}
+    cores = torch.get_num_threads()
+    unit = "GB/s of bf16 weights"
+    legs = {}
+
+    # Qwen3-30B-A3B: 8 experts of one layer (24 tensors) + the layer's q, k, v, o
+    experts = [_cpu_gen(sh, 10 + i) for i, sh in enumerate([(768, 2048), (768, 2048), (2048, 768)] * 8)]
+    attn = [_cpu_gen(sh, 50 + i, False) for i, sh in enumerate([(4096, 2048), (512, 2048), (512, 2048), (2048, 4096)])]
+    nb = sum(2 * w.numel() for w in experts + attn)
+    rate_fp8, reps, dt = _cpu_rate(lambda: [torch_ref.block_fp8_ref(w, (128, 128)) for w in experts + attn], nb, budget_s * 0.3)
+    legs["fp8_block_quant"] = {"value": rate_fp8, "unit": unit, "cores": cores, "kind": "port",
+                               "sample": f"8 experts (gate, up, down) + q, k, v, o of one Qwen3-30B-A3B-shaped layer "
+                                         f"({nb / 1e6:.0f} MB bf16) x {reps} passes in {dt:.1f} s, torch CPU restatement of block_fp8"}
+    nb = sum(2 * w.numel() for w in experts)
+    rate_int4, reps, dt = _cpu_rate(lambda: [torch_ref.pack_layer_ref(w, 128, True) for w in experts], nb, budget_s * 0.3)
+    legs["int4_group_quant_pack"] = {"value": rate_int4, "unit": unit, "cores": cores, "kind": "port",
+                                     "sample": f"8 experts (gate, up, down) of one Qwen3-30B-A3B-shaped layer ({nb / 1e6:.0f} MB "
+                                               f"bf16) x {reps} passes in {dt:.1f} s, torch CPU restatement of the "
+                                               "fake_int4_quant_cuda kernel + pack_layer"}
+    del experts, attn
+
+    # DeepSeek-V3: 8 experts (24 tensors) of e4m3 codes + scales -> bf16
+    g = torch.Generator().manual_seed(7)
+    xs, ss = [], []
+    for sh in [(2048, 7168), (2048, 7168), (7168, 2048)] * 8:
+        c = torch.randint(0, 254, sh, generator=g, dtype=torch.int32)
+        xs.append((c + (c >= 0x7F).int()).to(torch.uint8).view(torch.float8_e4m3fn))
+        ss.append(torch.exp(torch.empty(sh[0] // 128, sh[1] // 128).uniform_(-9.21034, -2.302585, generator=g)))
+    nb = sum(2 * x.numel() for x in xs)
+    rate, reps, dt = _cpu_rate(lambda: [torch_ref.weight_dequant_ref(x, sc) for x, sc in zip(xs, ss)], nb, budget_s * 0.2)
+    legs["fp8_block_dequant"] = {"value": rate, "unit": "GB/s of bf16 weights produced", "cores": cores, "kind": "port",
+                                 "sample": f"8 experts (gate, up, down) of the DeepSeek-V3-shaped layer ({nb / 1e6:.0f} MB bf16 "
+                                           f"out) x {reps} passes in {dt:.1f} s, torch CPU restatement of weight_dequant"}
+    del xs, ss
+
+    # the [4096, 4096] matrix in full: quant, then dequant of its own output
+    w = _cpu_gen((4096, 4096), 0)
+
+    def cfg1():
+        q, sc = torch_ref.block_fp8_ref(w, (128, 128))
+        torch_ref.weight_dequant_ref(q, sc)
+
+    rate, reps, dt = _cpu_rate(cfg1, 2 * w.numel(), budget_s * 0.2)
+    legs["cfg1_roundtrip"] = {"value": rate, "unit": "GB/s of bf16 weights through quant + dequant", "cores": cores,
+                              "kind": "port", "sample": f"the whole [4096,4096] matrix x {reps} round trips in {dt:.1f} s, "
+                                                        "torch CPU restatement of block_fp8 + weight_dequant"}
+
+    b_fp8, b_int4 = north_star_bytes
+    mixed = (b_fp8 + b_int4) / (b_fp8 / rate_fp8 + b_int4 / rate_int4)
+    head = {"value": mixed, "unit": unit, "cores": cores, "kind": "port",
+            "sample": "the step's mix of block-FP8 and INT4 work at the CPU rates measured on 8 experts + q, k, v, o of one "
+                      f"layer: FP8 {rate_fp8:.2f} GB/s, INT4 {rate_int4:.2f} GB/s (records under cpu_baseline_legs); torch CPU "
+                      "op-for-op restatements of block_fp8 and fake_int4_quant_cuda + pack_layer"}
+    return head, legs
 
 
 def main():
@@ -438,12 +708,12 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="time budget of the CPU baseline sample")
+    ap.add_argument("--cpu-seconds", type=float, default=24.0, help="time budget of the CPU baseline samples (all legs)")
     ap.add_argument("--int4-layers", type=int, default=48, help="layers of Qwen3-30B-A3B experts in the INT4 extra")
     ap.add_argument("--dequant-experts", type=int, default=256)
-    ap.add_argument("--no-extras", action="store_true", help="headline workload only")
+    ap.add_argument("--no-extras", action="store_true", help="headline step only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
-    ap.add_argument("--only", choices=["fp8moe", "int4", "dequant", "int4deq", "ste", "delta", "forms", "copy", "stream"], default=None,
+    ap.add_argument("--only", choices=["fp8", "cfg1", "bucket", "fp8moe", "int4", "dequant", "int4deq", "ste", "delta", "forms", "copy", "stream", "hashes"], default=None,
                     help="run just one of the other legs and print its record: a kernel for profiling, the plain copy "
                          "kernel that hardware counters are calibrated against, or the host-resident streaming run "
                          "(64 x 1 GiB buckets, PCIe-bound)")
@@ -456,6 +726,10 @@ def main():
               "launcher; run with --gpus 1", file=sys.stderr)
         sys.exit(2)
 
+    if args.only == "hashes":       # what the profile summaries record as kernel_source_sha256
+        print(json.dumps({k: kernel_source_hash(*v) for k, v in KERNEL_SOURCES.items()}))
+        return
+
     import torch
 
     if not torch.cuda.is_available():
@@ -464,6 +738,15 @@ def main():
     dev = torch.device("cuda:0")
     torch.manual_seed(0)
 
+    if args.only == "fp8":
+        print(json.dumps(bench_fp8_quant(dev, args.steps, args.warmup)))
+        return
+    if args.only == "cfg1":
+        print(json.dumps(bench_cfg1(dev, args.steps, args.warmup)))
+        return
+    if args.only == "bucket":
+        print(json.dumps(bench_bucket(dev, args.steps, args.warmup, args.int4_layers)))
+        return
     if args.only == "fp8moe":
         print(json.dumps(bench_fp8_quant_moe(dev, args.steps, args.warmup, args.int4_layers)))
         return
@@ -490,8 +773,20 @@ def main():
                                       not args.stream_no_download)))
         return
 
-    r = bench_fp8_quant(dev, args.steps, args.warmup)
-    achieved = r["algo_bytes"] / r["kernel_ms"] / 1e6      # GB/s
+    r = bench_north_star(dev, args.steps, args.warmup, args.int4_layers)
+    kernels = {}
+    for key, name, profile, src in (("fp8", "fp8_block_quant_kernel<TORCH_DEVICE, per-tile descriptors>",
+                                     "fp8_block_quant_qwen3_30b_a3b_state_dict.txt", "fp8_block_quant"),
+                                    ("int4", "int4_pack_kernel<128, per-item descriptors>",
+                                     "int4_pack_qwen3_30b_a3b_experts.txt", "int4_pack")):
+        k = r[key]
+        achieved = k["algo_bytes"] / k["kernel_ms"] / 1e6      # GB/s
+        traffic, note = _traffic_from_profile(profile, src)
+        kernels[key] = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                        "frac": achieved / HBM_PEAK_GBS, "traffic": traffic, "traffic_source": note, "kernel": name,
+                        "kernel_ms": k["kernel_ms"], "kernel_ms_min": k["kernel_ms_min"],
+                        "algorithmic_bytes_per_launch": k["algo_bytes"]}
+    lower = min(kernels.values(), key=lambda v: v["frac"])
     line = {
         "metric": "GB/s of bf16 weights quantized (FP8 & INT4) + % of HBM peak, 1x MI355X",
         "value": r["bf16_bytes"] / r["wall_ms"] / 1e6,
@@ -500,32 +795,33 @@ def main():
         "ms_per_step": r["wall_ms"],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "Qwen3-4B-shaped bf16 state dict, block-FP8 128x128 quant of all 252 linear weights "
-                               "(36 layers x q,k,v,o,gate,up,down; 7.27 GB bf16) = one weight-sync pass, one grouped "
-                               "launch, block_fp8 arithmetic as torch evaluates it on GPU tensors",
-                   "elements": r["elements"], "blocks": r["blocks"], "bf16_GB": r["bf16_bytes"] / 1e9,
+        "config": {"workload": f"Qwen3-30B-A3B-shaped bf16 state dict ({r['layers']} layers x (128 experts x gate, up "
+                               "[768,2048], down [2048,768] + q, k, v, o), N(0, 0.02) with rare x20 outliers), resident in "
+                               f"HBM: block-FP8 128x128 quant of all {r['tensors_fp8']} linear weights (block_fp8 arithmetic "
+                               f"as torch evaluates it on GPU tensors), then INT4 sym group-128 pack of the {r['tensors_int4']} "
+                               "expert weights; one grouped launch each",
+                   "launches_per_step": 2, "bf16_GB_fp8": 2 * r["fp8"]["elements"] / 1e9,
+                   "bf16_GB_int4": 2 * r["int4"]["elements"] / 1e9, "fp8_blocks": r["fp8"]["blocks"],
                    "parity_tensors_checked": r["parity_tensors_checked"]},
-        "pct_hbm_peak": 100.0 * achieved / HBM_PEAK_GBS,
-        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS,
-                     "traffic": _traffic_from_profile("fp8_block_quant_qwen3_4b_pmc.txt"),
-                     "kernel": "fp8_block_quant_kernel<TORCH_DEVICE, per-tile descriptors>", "kernel_ms": r["kernel_ms"],
-                     "kernel_ms_min": r["kernel_ms_min"], "algorithmic_bytes_per_launch": r["algo_bytes"]},
+        "pct_hbm_peak": 100.0 * lower["frac"],
+        "roofline": lower,
+        "roofline_kernels": kernels,
     }
     if not args.no_cpu:
-        line["cpu_baseline"] = cpu_baseline(r["cpu_sample"], args.cpu_seconds)
+        line["cpu_baseline"], line["cpu_baseline_legs"] = cpu_baselines(
+            args.cpu_seconds, (2 * r["fp8"]["elements"], 2 * r["int4"]["elements"]))
     else:
         line["cpu_baseline"] = None
     if not args.no_extras:
-        extras = {}
-        if args.int4_layers > 0:
-            extras["fp8_block_quant_moe"] = bench_fp8_quant_moe(dev, args.steps, args.warmup, args.int4_layers)
-            extras["int4_group_quant_pack"] = bench_int4_pack(dev, args.steps, args.warmup, args.int4_layers)
+        extras = {"fp8_block_quant_qwen3_4b": bench_fp8_quant(dev, args.steps, args.warmup),
+                  "cfg1_matrix_roundtrip": bench_cfg1(dev, args.steps, args.warmup)}
         if args.dequant_experts > 0:
             extras["fp8_block_dequant"] = bench_fp8_dequant(dev, args.steps, args.warmup, args.dequant_experts)
         if args.int4_layers > 0:
             extras["int4_dequant"] = bench_int4_inverse(dev, args.steps, args.warmup, min(args.int4_layers, 8), "int4deq")
             extras["int4_qat_forward"] = bench_int4_inverse(dev, args.steps, args.warmup, min(args.int4_layers, 8), "ste")
+        if args.int4_layers > 0:
+            extras["weight_sync_bucket"] = bench_bucket(dev, args.steps, args.warmup, args.int4_layers)
         extras["delta_xor"] = bench_delta(dev, args.steps, args.warmup)
         extras["single_tensor_forms"] = bench_single_tensor_forms(dev, args.steps, args.warmup)
         line["other_workloads"] = extras

@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define WQ_ABI_VERSION 9
+#define WQ_ABI_VERSION 11
 
 enum {
     WQ_OK = 0,
@@ -43,7 +43,7 @@ enum {
 };
 
 /* element type selectors */
-enum { WQ_DTYPE_BF16 = 0, WQ_DTYPE_F32 = 1, WQ_DTYPE_F16 = 2 };
+enum { WQ_DTYPE_BF16 = 0, WQ_DTYPE_F32 = 1, WQ_DTYPE_F16 = 2, WQ_DTYPE_F64 = 3 };
 
 /* FP8 block quant arithmetic.
  * WQ_FP8_MODE_TORCH  : amax clamped at bf16(1e-12) in bf16, scale = f32(amax)/448, q = f32(x)/scale
@@ -57,8 +57,13 @@ enum { WQ_DTYPE_BF16 = 0, WQ_DTYPE_F32 = 1, WQ_DTYPE_F16 = 2 };
  *                      (the IEEE x/scale, clamp, cast) is as in WQ_FP8_MODE_TORCH.
  * WQ_FP8_MODE_TRITON : fp32 amax floored at 1e-10f, scale = amax/448, q = f32(x)*(1.0f/scale).
  *                      Replaces _blockwise_cast_to_fp8_triton,
- *                      slime/backends/megatron_utils/kernels/fp8_kernel.py:24-58. */
-enum { WQ_FP8_MODE_TORCH = 0, WQ_FP8_MODE_TRITON = 1, WQ_FP8_MODE_TORCH_DEVICE = 2 };
+ *                      slime/backends/megatron_utils/kernels/fp8_kernel.py:24-58.
+ * WQ_FP8_MODE_UE8M0  : power-of-two scales: fp32 amax floored at 1e-4, scale = 2^ceil(log2(amax/448)),
+ *                      q = f32(x) * (1/scale) (exact), RNE to e4m3fn, no clamp (|q| <= 448 by construction).
+ *                      Replaces quant_weight_ue8m0 as called at quantizer_fp8.py:103-106 - a function of sglang
+ *                      (not vendored in the reference), so bit parity with it is unpinned; bf16 weights only
+ *                      (wq_fp8_block_quant and the grouped / tile / bucket forms), 128x128 blocks in the reference. */
+enum { WQ_FP8_MODE_TORCH = 0, WQ_FP8_MODE_TRITON = 1, WQ_FP8_MODE_TORCH_DEVICE = 2, WQ_FP8_MODE_UE8M0 = 3 };
 
 /* FP8 block dequant arithmetic.
  * WQ_DEQ_MODE_F32SCALE  : y = bf16(f32(x) * s).  Replaces weight_dequant, tools/fp8_cast_bf16.py:16-41.
@@ -102,6 +107,19 @@ int wq_fp8_block_quant_grouped(const wq_fp8_quant_desc *descs, const int64_t *ti
  * as in the tensor.  Costs 64 bytes of table per tile and saves the per-workgroup search; meant for plans that
  * are built once and run every weight sync. */
 int wq_fp8_block_quant_tiles(const wq_fp8_quant_desc *tiles, int64_t n_tiles, int bm, int bn, int mode, void *stream);
+
+/* A whole weight-sync bucket in ONE launch, written into ONE caller-owned byte buffer: the loop over
+ * convert_to_hf / quantize_params in HfWeightIteratorDirect._convert_to_hf_named_tensors
+ * (slime/backends/megatron_utils/update_weight/hf_weight_iterator_direct.py:50-67) followed by the flatten copy of
+ * FlattenedTensorBucket (update_weight_from_tensor.py:30-48).  `items` is a DEVICE array like the `tiles` of
+ * wq_fp8_block_quant_tiles, except that y and s hold BYTE OFFSETS from `out_base` (so a table built once serves a
+ * fresh output buffer on every sync), and that a descriptor with sx_m == WQ_BUCKET_COPY_MARK is a pass-through item:
+ * M bytes (at most WQ_BUCKET_COPY_BYTES) are copied from x to out_base + y, any alignment.  Quantised tiles need y
+ * 4-byte aligned for the vector kernel (other alignments take the generic one) and s 4-byte aligned. */
+#define WQ_BUCKET_COPY_MARK (-1)
+#define WQ_BUCKET_COPY_BYTES 32768
+int wq_fp8_bucket_convert(const wq_fp8_quant_desc *items, int64_t n_items, void *out_base, int bm, int bn, int mode,
+                          void *stream);
 
 /* wq_fp8_block_quant for bf16, fp16 or fp32 weights (`dtype` = WQ_DTYPE_*): the reference functions take any
  * floating dtype - block_fp8 computes amax and the 1e-12 floor in the weight dtype (the floor rounds to 0 in
@@ -149,7 +167,9 @@ int wq_fp8_block_dequant_grouped(const wq_fp8_dequant_desc *descs, const int64_t
  * dtype, plus scale and zero point [ceil(M/bm), ceil(N/bn)] in the input dtype.
  * Replaces fake_int4_quant_cuda(x, block_size, sym),
  * slime/backends/megatron_utils/kernels/int4_qat/fake_int4_quant_cuda.cu:327-378 (kernels :37-267).
- * dtype: WQ_DTYPE_BF16 or WQ_DTYPE_F32.  x has any strides; q/scale/zero are contiguous.
+ * dtype: WQ_DTYPE_BF16, WQ_DTYPE_F32 or WQ_DTYPE_F64 - the types the reference dispatches on (.cu:352-354); the
+ * arithmetic is fp32 for all of them (elements are converted on load, results on store).  x has any strides;
+ * q/scale/zero are contiguous.
  * Group shapes: (1, 32k), or bn dividing 32 with bm*bn a multiple of 32 (the shapes for which the
  * reference kernels are well defined); others return WQ_ERR_UNSUPPORTED. */
 int wq_int4_fake_quant(const void *x, int dtype, int64_t M, int64_t N, int64_t sx_m, int64_t sx_n,
@@ -182,6 +202,13 @@ int wq_int4_group_quant_pack_grouped(const wq_int4_pack_desc *descs, const int64
  * every weight sync. */
 int wq_int4_group_quant_pack_items(const wq_int4_pack_desc *items, int64_t n_items, int group, void *stream);
 
+/* The INT4 counterpart of wq_fp8_bucket_convert (the per-parameter loop it replaces calls
+ * quantize_params_compressed_tensors, quantizer_compressed_tensors.py:268-297, once per parameter): `items` as in
+ * wq_int4_group_quant_pack_items with packed and scale holding BYTE OFFSETS from `out_base`; an item with
+ * n_groups < 0 is a pass-through item that copies -n_groups bytes (at most WQ_BUCKET_COPY_BYTES) from x to
+ * out_base + packed, any alignment.  packed offsets 4-byte aligned, scale offsets 2-byte aligned. */
+int wq_int4_bucket_convert(const wq_int4_pack_desc *items, int64_t n_items, void *out_base, int group, void *stream);
+
 /* Asymmetric form of wq_int4_group_quant_pack (pack_layer(weight, group, sym=False),
  * tools/convert_hf_to_int4_direct.py:123-153): codes rintf(x/scale) + zero with scale = max((max-min)/15, 1e-5)
  * and zero = clamp(-rintf(min/scale), 0, 15) (fake_int4_quant_cuda.cu:61-75), passed through the reference's
@@ -196,6 +223,14 @@ int wq_int4_group_quant_pack_asym(const void *x, int64_t M, int64_t N, int64_t s
  * group % 8 == 0.  Replaces _dequantize_tensor, tools/convert_k2_thinking_int4_to_bf16.py:55-84 (whose unpacking
  * is compressed_tensors.unpack_from_int32). */
 int wq_int4_dequant(const int32_t *packed, const void *scale, void *y, int64_t M, int64_t N, int group, void *stream);
+
+/* wq_int4_dequant for the inputs the tuned kernel does not take: scales stored as WQ_DTYPE_BF16, WQ_DTYPE_F16 or
+ * WQ_DTYPE_F32 (the reference converts any dtype with .to(float32), convert_k2_thinking_int4_to_bf16.py:69), any
+ * group >= 1 dividing N (group 1 with one scale per element is the reference's group_size <= 0 branch, :74-75), and N
+ * that is not a multiple of 8 (packed is [M, ceil(N/8)]; unpack_from_int32 cuts the last word of a row).  With an fp32
+ * scale the product is rounded to fp32 and then to bf16, as in the reference.  A plain kernel. */
+int wq_int4_dequant_any(const int32_t *packed, const void *scale, int scale_dtype, void *y, int64_t M, int64_t N,
+                        int group, void *stream);
 
 /* wq_int4_dequant over a bucket of tensors in one launch.  `items` is a DEVICE array with one entry per work item
  * of WQ_INT4_DEQ_WORDS_PER_ITEM packed words (a tensor's last item may be shorter): pointers to the item's first

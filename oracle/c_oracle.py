@@ -39,6 +39,7 @@ def lib() -> ctypes.CDLL:
         L.wqo_int4_fake_quant.argtypes = [_vp, _int, _i64, _i64, _i64, _i64, _i64, _i64, _int, _vp, _vp, _vp]
         L.wqo_int4_pack_layer.argtypes = [_vp, _i64, _i64, _i64, _int, _vp, _vp, _vp]
         L.wqo_int4_dequant.argtypes = [_vp, _vp, _i64, _i64, _i64, _vp]
+        L.wqo_int4_dequant_any.argtypes = [_vp, _vp, _int, _i64, _i64, _i64, _vp]
         L.wqo_int4_fake_ste.argtypes = [_vp, _i64, _i64, _i64, _int, _vp]
         for n in ("wqo_f32_to_e4m3fn_n", "wqo_e4m3fn_to_f32_n", "wqo_f32_to_bf16_n"):
             getattr(L, n).argtypes = [_vp, _vp, _i64]
@@ -135,13 +136,14 @@ def fp8_block_dequant(x: torch.Tensor, s: torch.Tensor, block: int = 128, mode: 
 
 
 def int4_fake_quant(x: torch.Tensor, block_size, sym: bool):
-    assert _cpu(x).dim() == 2 and x.dtype in (torch.bfloat16, torch.float32)
+    assert _cpu(x).dim() == 2 and x.dtype in (torch.bfloat16, torch.float32, torch.float64)
     M, N = x.shape
     bm, bn = int(block_size[0]), int(block_size[1])
     q = torch.empty(M, N, dtype=x.dtype)
     sc = torch.empty(_cdiv(M, bm), _cdiv(N, bn), dtype=x.dtype)
     zp = torch.empty_like(sc)
-    _check(lib().wqo_int4_fake_quant(x.data_ptr(), 0 if x.dtype == torch.bfloat16 else 1, M, N, x.stride(0),
+    sel = {torch.bfloat16: 0, torch.float32: 1, torch.float64: 3}[x.dtype]
+    _check(lib().wqo_int4_fake_quant(x.data_ptr(), sel, M, N, x.stride(0),
                                      x.stride(1), bm, bn, int(sym), q.data_ptr(), sc.data_ptr(), zp.data_ptr()),
            "int4_fake_quant")
     return q, sc, zp
@@ -166,6 +168,19 @@ def int4_dequant(packed: torch.Tensor, scale: torch.Tensor, shape, group_size: i
     assert packed.dtype == torch.int32 and scale.dtype == torch.bfloat16
     y = torch.empty(M, N, dtype=torch.bfloat16)
     _check(lib().wqo_int4_dequant(packed.data_ptr(), scale.data_ptr(), M, N, group_size, y.data_ptr()), "int4_dequant")
+    return y
+
+
+def int4_dequant_any(packed: torch.Tensor, scale: torch.Tensor, shape, group_size: int) -> torch.Tensor:
+    """Scale in bf16, fp16 or fp32; group_size <= 0 means one scale per element; N need not be a multiple of 8."""
+    M, N = shape
+    packed = _cpu(packed).contiguous()
+    scale = _cpu(scale).contiguous()
+    sel = {torch.bfloat16: 0, torch.float32: 1, torch.float16: 2}[scale.dtype]
+    assert packed.dtype == torch.int32 and tuple(packed.shape) == (M, _cdiv(N, 8))
+    y = torch.empty(M, N, dtype=torch.bfloat16)
+    _check(lib().wqo_int4_dequant_any(packed.data_ptr(), scale.data_ptr(), sel, M, N, group_size if group_size > 0 else 1,
+                                      y.data_ptr()), "int4_dequant_any")
     return y
 
 

@@ -86,6 +86,25 @@ def blockwise_cast_ref(x: torch.Tensor, block_size=None, eps: float = 1e-10) -> 
 # ----------------------------------------------------------------------------- FP8 dequant
 
 
+def quant_weight_ue8m0_ref(w: torch.Tensor, weight_block_size=(128, 128)) -> tuple[torch.Tensor, torch.Tensor]:
+    """The UE8M0 branch of _quantize_param (megatron_to_hf/processors/quantizer_fp8.py:103-106) calls sglang's
+    ``quant_weight_ue8m0`` (sglang v0.5.15.post1, not vendored), which applies DeepGEMM's ``per_block_cast_to_fp8`` with
+    power-of-two scales.  PARITY UNPINNED: restated from that third-party source as published -
+    zero-pad to 128 multiples, ``amax = |x|.float().amax(block).clamp(1e-4)``, ``sf = 2 ** ceil(log2(amax / 448))``,
+    ``q = (x * (1 / sf)).to(e4m3fn)`` (no clamp), crop."""
+    assert list(weight_block_size) == [128, 128]
+    m, n = w.shape
+    pm, pn = _cdiv(m, 128) * 128, _cdiv(n, 128) * 128
+    padded = torch.zeros((pm, pn), dtype=w.dtype)
+    padded[:m, :n] = w
+    view = padded.view(-1, 128, pn // 128, 128)
+    amax = view.abs().float().amax(dim=(1, 3), keepdim=True).clamp(1e-4)
+    sf = amax / 448.0
+    sf = torch.pow(2.0, torch.ceil(torch.log2(sf.abs())))
+    q = (view * (1.0 / sf)).to(E4M3)
+    return q.view_as(padded)[:m, :n].contiguous(), sf.view(view.size(0), view.size(2))
+
+
 def _expand_scale(s: torch.Tensor, rows: int, cols: int, block: int) -> torch.Tensor:
     return s.repeat_interleave(block, dim=0)[:rows].repeat_interleave(block, dim=1)[:, :cols]
 
@@ -188,12 +207,25 @@ def pack_layer_ref(weight: torch.Tensor, group_size: int, sym: bool = True):
 
 def int4_dequant_ref(packed: torch.Tensor, scale: torch.Tensor, shape, group_size: int) -> torch.Tensor:
     """tools/convert_k2_thinking_int4_to_bf16.py:55-84 with the third-party unpack written out: nibble j of a word
-    at bits [4j, 4j+4), minus 8, as int8; then (int8.to(f32) * scale.to(f32) repeated per group).to(bf16)."""
+    at bits [4j, 4j+4), minus 8, as int8, rows cut to their length; then the reference's own lines: the scale of any
+    dtype ``.to(float32)``, repeated per group (``group_size > 0``) or taken as it is (``group_size <= 0``), reshaped
+    to the weight when only the element counts agree, ``(int8.to(f32) * scales).to(bf16)``."""
     rows, cols = shape
     shifts = torch.arange(8, dtype=torch.int32) * 4
     nib = ((packed.unsqueeze(-1) >> shifts) & 0xF).view(rows, -1)[:, :cols]
     q = (nib - 8).to(torch.int8)
-    s = torch.repeat_interleave(scale.to(torch.float32), repeats=group_size, dim=1)
+    if group_size > 0:
+        s = scale.to(torch.float32)
+        if s.dim() == 1:
+            s = s.unsqueeze(1)
+        s = torch.repeat_interleave(s, repeats=group_size, dim=1)
+    else:
+        s = scale.to(torch.float32)
+    if s.shape != q.shape:
+        if s.numel() == q.numel():
+            s = s.reshape_as(q)
+        else:
+            raise ValueError(f"Scale shape {s.shape} incompatible with weight shape {q.shape}")
     return (q.to(torch.float32) * s).to(torch.bfloat16).contiguous()
 
 

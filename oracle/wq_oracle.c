@@ -9,6 +9,11 @@
  *   wqo_fp8_block_quant   mode 0: tools/convert_hf_to_fp8.py:41-75 (block_fp8) as torch evaluates it on CPU tensors
  *                         mode 2: the same, as torch evaluates it on GPU tensors (scalar division = reciprocal multiply)
  *                         mode 1: slime/backends/megatron_utils/kernels/fp8_kernel.py:24-58
+ *                         mode 3: power-of-two (UE8M0) scales, the branch of _quantize_param at
+ *                                 megatron_to_hf/processors/quantizer_fp8.py:103-106 - its arithmetic is sglang's
+ *                                 quant_weight_ue8m0 (sglang v0.5.15.post1, NOT vendored in the reference; it wraps
+ *                                 DeepGEMM's per_block_cast_to_fp8 with use_ue8m0): fp32 amax floored at 1e-4,
+ *                                 sf = 2^ceil(log2(amax / 448)), y = e4m3(x * (1 / sf)), no clamp
  *   wqo_fp8_channel_quant tools/convert_hf_to_fp8.py:78-83 (channel_fp8)
  *   wqo_fp8_tensor_quant  tools/convert_hf_to_fp8.py:86-91 (tensor_fp8), same arithmetic as
  *                         megatron_to_hf/processors/quantizer_fp8.py:114-116
@@ -35,6 +40,11 @@
  *     Triton's "/" is not guaranteed IEEE-exact (PARITY UNPINNED there).  On MI355X it is
  *     pinned: oracle/triton_ref.py restates the kernel in Triton and the GPU tests find it
  *     bit-identical to this file's reading for every bf16 amax and every bf16 value.
+ *   - fp8 mode 3: PARITY UNPINNED.  The algorithm lives in a third-party dependency that is absent from the
+ *     reference checkout; it is restated from that library's published source as remembered, and pinned only by
+ *     what the mathematics fixes: the scale is the smallest power of two >= max(amax, 1e-4) / 448, the codes are one
+ *     RNE of an exactly scaled value and never exceed 448, and the literal log2 / ceil / pow chain in torch_ref.py
+ *     agrees with the exponent arithmetic used here for every bf16 amax.
  *   - fp8 mode 2 and the bf16 divisor of the per-tensor form: pinned by torch's own GPU
  *     kernels run on the same inputs (tests/test_gpu_fp8.py).
  *   - wqo_int4_fake_quant: the reference kernel is CUDA-only, has no test and cannot be
@@ -178,6 +188,24 @@ static inline float scale_from_amax_mode1(float amax)
     return a / FP8_MAX;
 }
 
+/* Smallest power of two >= v for a positive finite v (a power of two maps to itself); NaN and Inf pass through. */
+static inline float pow2_ceil(float v)
+{
+    uint32_t u = f2u(v);
+    if ((u & 0x7F800000u) == 0x7F800000u) return v;
+    if ((u & 0x7F800000u) == 0) {                       /* subnormal: scale up, recurse, scale down */
+        return pow2_ceil(v * 0x1p64f) * 0x1p-64f;
+    }
+    if ((u & 0x007FFFFFu) == 0) return v;
+    return u2f((u & 0x7F800000u) + 0x00800000u);
+}
+static inline float scale_from_amax_mode3(float amax)
+{
+    float a = amax < 1e-4f ? 1e-4f : amax;              /* .clamp(1e-4); NaN stays NaN */
+    return pow2_ceil(a / FP8_MAX);
+}
+static inline uint8_t quant_elem_mode3(float x, float s_inv) { return wqo_f32_to_e4m3fn(x * s_inv); }
+
 static inline uint8_t quant_elem_mode1(float x, float s_inv)
 {
     float q = x * s_inv;
@@ -251,7 +279,7 @@ WQO_API int wqo_fp8_block_quant_any(const void *x, int dtype, int64_t M, int64_t
 WQO_API int wqo_fp8_block_quant(const uint16_t *x, int64_t M, int64_t N, int64_t sx_m, int64_t sx_n,
                                 int64_t bm, int64_t bn, int mode, uint8_t *y, float *s)
 {
-    if (M < 0 || N < 0 || bm <= 0 || bn <= 0 || mode < 0 || mode > 2) return 1;
+    if (M < 0 || N < 0 || bm <= 0 || bn <= 0 || mode < 0 || mode > 3) return 1;
     int64_t nt = cdiv(M, bm), kt = cdiv(N, bn);
 #pragma omp parallel for schedule(static)
     for (int64_t bi = 0; bi < nt; ++bi) {
@@ -263,13 +291,15 @@ WQO_API int wqo_fp8_block_quant(const uint16_t *x, int64_t M, int64_t N, int64_t
                 for (int64_t j = c0; j < c1; ++j)
                     amax = max_nanprop(amax, fabsf(wqo_bf16_to_f32(x[i * sx_m + j * sx_n])));
             float scale, s_inv = 0.0f;
-            if (mode != 1) scale = scale_torch(amax, mode);
+            if (mode == 3) { scale = scale_from_amax_mode3(amax); s_inv = 1.0f / scale; }
+            else if (mode != 1) scale = scale_torch(amax, mode);
             else { scale = scale_from_amax_mode1(amax); s_inv = 1.0f / scale; }
             s[bi * kt + bj] = scale;
             for (int64_t i = r0; i < r1; ++i)
                 for (int64_t j = c0; j < c1; ++j) {
                     float v = wqo_bf16_to_f32(x[i * sx_m + j * sx_n]);
-                    y[i * N + j] = mode != 1 ? quant_elem_mode0(v, scale) : quant_elem_mode1(v, s_inv);
+                    y[i * N + j] = mode == 3 ? quant_elem_mode3(v, s_inv)
+                                   : mode != 1 ? quant_elem_mode0(v, scale) : quant_elem_mode1(v, s_inv);
                 }
         }
     }
@@ -350,11 +380,13 @@ WQO_API int wqo_fp8_block_dequant(const uint8_t *x, const float *s, int64_t M, i
 static inline float ld_elem(const void *x, int dtype, int64_t off)
 {
     if (dtype == 0) return wqo_bf16_to_f32(((const uint16_t *)x)[off]);
+    if (dtype == 3) return (float)((const double *)x)[off];      /* static_cast<float>(x[...]), .cu:70 */
     return ((const float *)x)[off];
 }
 static inline void st_elem(void *p, int dtype, int64_t off, float v)
 {
     if (dtype == 0) ((uint16_t *)p)[off] = wqo_f32_to_bf16(v);
+    else if (dtype == 3) ((double *)p)[off] = (double)v;         /* static_cast<scalar_t>(val), .cu:92 */
     else ((float *)p)[off] = v;
 }
 
@@ -363,13 +395,14 @@ static inline void st_elem(void *p, int dtype, int64_t off, float v)
  * (.cu:233-234,254).  asym: scale = fmaxf((max-min) * (1.0f/15.0f), 1e-5f);
  * zero = clamp(-rintf(min/scale), 0, 15); q = rintf(x/scale) + zero (.cu:235-240,255-257).
  * fmaxf/fminf drop NaN operands exactly as the device functions do.  Outputs q [M,N],
- * scale/zero [cdiv(M,bm), cdiv(N,bn)], all contiguous, in the input dtype (0 = bf16, 1 = fp32).
+ * scale/zero [cdiv(M,bm), cdiv(N,bn)], all contiguous, in the input dtype (0 = bf16, 1 = fp32, 3 = fp64: the
+ * three types of AT_DISPATCH_FLOATING_TYPES_AND(BFloat16), .cu:352; every type is converted to fp32 on load).
  * Supported group shapes are the ones for which the reference kernels are well defined:
  * (1, 32k) and (bm, bn) with bn dividing 32 and bm*bn a multiple of 32. */
 WQO_API int wqo_int4_fake_quant(const void *x, int dtype, int64_t M, int64_t N, int64_t sx_m, int64_t sx_n,
                                 int64_t bm, int64_t bn, int sym, void *q, void *scale, void *zero)
 {
-    if (M < 0 || N < 0 || bm <= 0 || bn <= 0 || (dtype != 0 && dtype != 1)) return 1;
+    if (M < 0 || N < 0 || bm <= 0 || bn <= 0 || (dtype != 0 && dtype != 1 && dtype != 3)) return 1;
     if ((bm * bn) % 32 != 0) return 2;
     if (!((bm == 1 && bn % 32 == 0) || (32 % bn == 0))) return 3;
     const float SYM_CONS = 1.0f / 7.0f, ASYM_CONS = 1.0f / 15.0f;
@@ -494,6 +527,26 @@ WQO_API int wqo_int4_dequant(const int32_t *packed, const uint16_t *scale, int64
             uint32_t w = (uint32_t)packed[i * (N / 8) + j / 8];
             int q = (int)((w >> (4 * (j % 8))) & 0xFu) - 8;
             float s = wqo_bf16_to_f32(scale[i * (N / gs) + j / gs]);
+            y[i * N + j] = wqo_f32_to_bf16((float)q * s);
+        }
+    return 0;
+}
+
+/* The same function for the other inputs the reference accepts: scale stored as bf16 (0), fp32 (1) or fp16 (2) and
+ * converted with .to(float32) (:69); group_size <= 0 (pass gs = 1: one scale per element, :74-75); N not a multiple
+ * of 8 (packed is [M, ceil(N/8)], the tail of a row's last word is cut).  (float)q * s is one fp32 rounding, the
+ * conversion to bf16 a second one. */
+WQO_API int wqo_int4_dequant_any(const int32_t *packed, const void *scale, int scale_dtype, int64_t M, int64_t N,
+                                 int64_t gs, uint16_t *y)
+{
+    if (M < 0 || N < 0 || gs <= 0 || N % gs != 0 || scale_dtype < 0 || scale_dtype > 2) return 1;
+    int64_t wpr = (N + 7) / 8;
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < M; ++i)
+        for (int64_t j = 0; j < N; ++j) {
+            uint32_t w = (uint32_t)packed[i * wpr + j / 8];
+            int q = (int)((w >> (4 * (j % 8))) & 0xFu) - 8;
+            float s = load_any(scale, scale_dtype, i * (N / gs) + j / gs);
             y[i * N + j] = wqo_f32_to_bf16((float)q * s);
         }
     return 0;

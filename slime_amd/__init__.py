@@ -7,6 +7,7 @@ of ``slime_amd/lib/libslime_amd_wq.so``; there is no CPU or pure-torch fallback.
 """
 
 from . import _lib, arith, delta
+from .bucket import BucketConverter, FlattenedBucket, FlattenedTensorMetadata, quantize_bucket
 from .arith import get_torch_arithmetic, set_torch_arithmetic, torch_arithmetic
 from .fp8 import (
     Fp8DequantPlan,
@@ -16,7 +17,9 @@ from .fp8 import (
     blockwise_cast_to_fp8_triton,
     channel_fp8,
     quant_fp8,
+    quant_weight_ue8m0,
     tensor_fp8,
+    transform_scale_ue8m0,
     weight_dequant,
     weight_dequant_bf16_scale,
 )
@@ -35,6 +38,7 @@ from .processors import (
     quantize_params,
     quantize_params_compressed_tensors,
     quantize_params_fp8,
+    set_ue8m0_requant,
 )
 
 # the injectable `quantize_weight(weight, (128, 128)) -> (qweight, scale)` hook of the reference's
@@ -42,6 +46,8 @@ from .processors import (
 quantize_weight = blockwise_cast_to_fp8_triton
 
 __all__ = [
+    "BucketConverter", "FlattenedBucket", "FlattenedTensorMetadata", "quantize_bucket", "quant_weight_ue8m0",
+    "set_ue8m0_requant", "transform_scale_ue8m0",
     "Fp8DequantPlan", "Fp8QuantPlan", "Int4DequantPlan", "Int4PackPlan", "block_fp8", "block_fp8_many",
     "blockwise_cast_to_fp8_triton", "channel_fp8", "dequantize_int4", "fake_int4_quant_cuda",
     "fake_int4_quantization_ste", "get_torch_arithmetic", "set_torch_arithmetic", "torch_arithmetic",

@@ -15,16 +15,17 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libslime_amd_wq.so")
 
-ABI_VERSION = 9
+ABI_VERSION = 11
 
 # selectors (mirrors of the header's enums)
-DTYPE_BF16, DTYPE_F32, DTYPE_F16 = 0, 1, 2
-FP8_MODE_TORCH, FP8_MODE_TRITON, FP8_MODE_TORCH_DEVICE = 0, 1, 2
+DTYPE_BF16, DTYPE_F32, DTYPE_F16, DTYPE_F64 = 0, 1, 2, 3
+FP8_MODE_TORCH, FP8_MODE_TRITON, FP8_MODE_TORCH_DEVICE, FP8_MODE_UE8M0 = 0, 1, 2, 3
 DIV7_IEEE, DIV7_DEVICE = 0, 1
 DEQ_MODE_F32SCALE, DEQ_MODE_BF16SCALE = 0, 1
 DEQ_SEG, DEQ_SEGS_PER_WG = 512, 16
 INT4_GROUPS_PER_WG = 64
 INT4_DEQ_WORDS_PER_ITEM = 2048
+BUCKET_COPY_MARK, BUCKET_COPY_BYTES = -1, 32768
 
 _i64, _int, _vp, _u32, _u64 = ctypes.c_int64, ctypes.c_int, ctypes.c_void_p, ctypes.c_uint32, ctypes.c_uint64
 
@@ -35,6 +36,8 @@ SIGNATURES = {
     "wq_fp8_block_quant": [_vp, _i64, _i64, _i64, _i64, _vp, _i64, _vp, _int, _int, _int, _vp],
     "wq_fp8_block_quant_grouped": [_vp, _vp, _int, _i64, _int, _int, _int, _vp],
     "wq_fp8_block_quant_tiles": [_vp, _i64, _int, _int, _int, _vp],
+    "wq_fp8_bucket_convert": [_vp, _i64, _vp, _int, _int, _int, _vp],
+    "wq_int4_bucket_convert": [_vp, _i64, _vp, _int, _vp],
     "wq_fp8_block_quant_any": [_vp, _int, _i64, _i64, _i64, _i64, _vp, _i64, _vp, _int, _int, _int, _vp],
     "wq_fp8_row_quant": [_vp, _i64, _i64, _i64, _i64, _vp, _i64, _vp, _int, _vp],
     "wq_fp8_tensor_quant": [_vp, _i64, _i64, _i64, _i64, _vp, _i64, _vp, _vp, _int, _vp],
@@ -46,6 +49,7 @@ SIGNATURES = {
     "wq_int4_group_quant_pack_items": [_vp, _i64, _int, _vp],
     "wq_int4_group_quant_pack_asym": [_vp, _i64, _i64, _i64, _int, _vp, _vp, _vp, _vp],
     "wq_int4_dequant": [_vp, _vp, _vp, _i64, _i64, _int, _vp],
+    "wq_int4_dequant_any": [_vp, _vp, _int, _vp, _i64, _i64, _int, _vp],
     "wq_int4_dequant_items": [_vp, _i64, _int, _vp],
     "wq_int4_fake_quant_ste": [_vp, _vp, _i64, _i64, _int, _int, _vp],
     "wq_delta_workspace_bytes": [_i64],

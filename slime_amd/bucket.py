@@ -1,0 +1,348 @@
+"""A whole weight-sync bucket converted, quantised and flattened by ONE kernel launch.
+
+The reference's hot loop is one ``convert_to_hf`` / ``quantize_params`` call per Megatron parameter
+(``HfWeightIteratorDirect._convert_to_hf_named_tensors``, slime/backends/megatron_utils/update_weight/
+hf_weight_iterator_direct.py:50-67) - a kernel launch or a dozen per tensor - followed by a second pass that copies
+every result into one uint8 buffer (``FlattenedTensorBucket(named_tensors=...)`` in ``_build_flattened_tensor_data``,
+update_weight_from_tensor.py:30-48).  ``BucketConverter.convert`` takes the bucket after name conversion - a list of
+``(megatron_name, [(hf_name, tensor), ...])`` - applies the routing of ``quantize_params`` (processors/__init__.py:6-22,
+quantizer_fp8.py:10-95, quantizer_compressed_tensors.py:268-297) and issues one launch whose work items either quantise
+a tile / a run of groups straight into its place in the flat buffer or copy a piece of a pass-through tensor there.  The
+result has the layout the bucket consumer reads: one uint8 tensor plus ``(name, shape, dtype, start_idx, end_idx, numel)``
+per tensor, names in the order the per-parameter loop produces them, tensors packed back to back.
+
+The per-item table is built once per bucket *identity* (names, shapes, strides and addresses of the inputs) and cached:
+a weight sync that presents the same tensors again does no host-side table work.  Destinations in the table are offsets,
+so every call can write into a fresh buffer (the reference warns against reusing the IPC-facing one,
+update_weight_from_tensor.py:39-43) or into ``out=``.
+"""
+
+from __future__ import annotations
+
+import dataclasses
+import json
+from collections import OrderedDict
+from typing import Sequence
+
+import torch
+
+from . import _lib
+from .fp8 import FP8_DTYPE, ceildiv, tile_table
+from .int4 import item_table
+from .processors import _fp8_route, _is_ignored, quantize_params
+
+_COPY = _lib.BUCKET_COPY_BYTES
+
+
+@dataclasses.dataclass(frozen=True)
+class FlattenedTensorMetadata:
+    """One entry of ``FlattenedTensorBucket.get_metadata()``: the tensor is
+    ``flattened_tensor[start_idx:end_idx].view(dtype).reshape(shape)``; ``numel`` counts bytes."""
+    name: str
+    shape: torch.Size
+    dtype: torch.dtype
+    start_idx: int
+    end_idx: int
+    numel: int
+
+
+class FlattenedBucket:
+    """The pair the bucket consumer receives (``{"flattened_tensor": ..., "metadata": ...}``,
+    update_weight_from_tensor.py:44-48), with ``FlattenedTensorBucket``'s accessors."""
+
+    supports_multi_dtypes = True
+
+    def __init__(self, flattened_tensor: torch.Tensor, metadata: Sequence[FlattenedTensorMetadata], launches: int = 0):
+        self.flattened_tensor = flattened_tensor
+        self.metadata = list(metadata)
+        self.launches = launches            # kernel launches this bucket cost (diagnostic)
+
+    def get_flattened_tensor(self) -> torch.Tensor:
+        return self.flattened_tensor
+
+    def get_metadata(self):
+        return self.metadata
+
+    def reconstruct_tensors(self):
+        """-> [(name, tensor)]: views into the flat buffer, in bucket order."""
+        return [(m.name, self.flattened_tensor[m.start_idx:m.end_idx].view(m.dtype).reshape(m.shape))
+                for m in self.metadata]
+
+
+def flatten_named_tensors(named_tensors) -> FlattenedBucket:
+    """What ``FlattenedTensorBucket(named_tensors=...)`` builds - every tensor flattened to bytes, concatenated in order -
+    with torch ops.  Used for buckets the one-launch path does not cover, and by the tests as the expected layout."""
+    if not named_tensors:
+        return FlattenedBucket(torch.empty(0, dtype=torch.uint8, device=torch.device("cuda", torch.cuda.current_device())), [])
+    meta, parts, off = [], [], 0
+    for name, t in named_tensors:
+        b = t.detach().contiguous().flatten().view(torch.uint8)
+        meta.append(FlattenedTensorMetadata(name, t.shape, t.dtype, off, off + b.numel(), b.numel()))
+        parts.append(b)
+        off += b.numel()
+    return FlattenedBucket(torch.cat(parts, dim=0), meta, launches=len(parts) + 1)
+
+
+class _Plan:
+    __slots__ = ("kind", "items", "n_items", "total_bytes", "metadata", "keepalive", "late_copies", "group", "block", "device")
+
+
+class BucketConverter:
+    """Converts buckets of one model under one ``quantization_config``; see the module docstring.
+
+    ``convert(params)`` -> ``FlattenedBucket``.  ``params`` is ``[(megatron_name, [(hf_name, tensor), ...]), ...]`` -
+    what ``_convert_to_hf_core`` yields per Megatron parameter.  Tensors the one-launch kernels do not take
+    (FP8: not 2-D bf16 on the GPU; INT4: not contiguous 16-byte aligned bf16 with 32 / 64 / 128 groups, or asymmetric;
+    per-tensor FP8 configurations) go through the per-tensor functions first and are copied in by the same launch, so
+    the result is always what the per-parameter loop gives.
+    """
+
+    def __init__(self, args=None, quantization_config=None, transform_ue8m0: bool = True, max_cached_plans: int = 256):
+        self.args = args
+        self.config = quantization_config
+        self.transform_ue8m0 = transform_ue8m0
+        self._config_key = json.dumps(quantization_config, sort_keys=True, default=str)
+        self._plans: OrderedDict = OrderedDict()
+        self._max = int(max_cached_plans)
+        self.plan_builds = 0
+        method = None if quantization_config is None else quantization_config["quant_method"]
+        self._method = method if method in ("fp8", "compressed-tensors") else None
+        if self._method == "fp8":
+            assert quantization_config.get("fmt", "e4m3") == "e4m3", f"Unsupported FP8 format: {quantization_config.get('fmt')}"
+            assert quantization_config["activation_scheme"] == "dynamic"
+            self._block = quantization_config.get("weight_block_size", None)
+        elif self._method == "compressed-tensors":
+            w_cfg = quantization_config["config_groups"]["group_0"]["weights"]
+            self._group, self._sym = w_cfg["group_size"], w_cfg["symmetric"]
+            self._ignore = quantization_config.get("ignore", [])
+
+    # ------------------------------------------------------------------ routing (what the per-parameter loop decides)
+
+    def _route(self, megatron_name, converted):
+        """-> list of ("quant" | "pass" | "loop", hf_name, tensor, index in `converted`).  "loop": quantised, but by the
+        per-tensor function."""
+        from . import processors
+
+        if self._method == "fp8":
+            route = _fp8_route(megatron_name)
+            if route is None:
+                return [("pass", n, t, ci) for ci, (n, t) in enumerate(converted)]
+            ops = []
+            for ci, (n, t) in enumerate(converted):
+                if route == "skip_scales" and n.endswith("_scale"):
+                    continue
+                assert n.endswith(".weight"), f"Expected weight parameter, got {n}"
+                one_launch = (self._block is not None and not processors.ue8m0_requant_enabled() and t.is_cuda
+                              and t.dim() == 2 and t.dtype == torch.bfloat16 and t.numel() > 0)
+                ops.append(("quant" if one_launch else "loop", n, t, ci))
+            return ops
+        if self._method == "compressed-tensors":
+            ops = []
+            for ci, (n, t) in enumerate(converted):
+                if _is_ignored(n, self._ignore) or not n.endswith(".weight") or t.dim() < 2:
+                    ops.append(("pass", n, t, ci))
+                    continue
+                one_launch = (self._sym and t.is_cuda and t.dim() == 2 and t.dtype == torch.bfloat16 and t.is_contiguous()
+                              and t.data_ptr() % 16 == 0 and self._group in (32, 64, 128) and t.numel() > 0
+                              and t.shape[1] % self._group == 0)
+                ops.append(("quant" if one_launch else "loop", n, t, ci))
+            return ops
+        return [("pass", n, t, ci) for ci, (n, t) in enumerate(converted)]
+
+    # ------------------------------------------------------------------ plan
+
+    @staticmethod
+    def _key(params):
+        return tuple((mn, tuple((n, t.data_ptr(), tuple(t.shape), t.stride(), t.dtype) for n, t in conv)) for mn, conv in params)
+
+    def _build(self, params) -> _Plan:
+        self.plan_builds += 1
+        device = None
+        for _, conv in params:
+            for _, t in conv:
+                if t.is_cuda:
+                    device = t.device
+                    break
+            if device is not None:
+                break
+        if device is None:
+            raise RuntimeError("BucketConverter: the bucket holds no GPU tensor; there is no CPU path")
+        fp8 = self._method != "compressed-tensors"          # pass-through-only buckets use the FP8 launch's copy items
+        plan = _Plan()
+        plan.kind = "fp8" if fp8 else "int4"
+        plan.block = tuple(int(b) for b in self._block) if (self._method == "fp8" and self._block is not None) else (128, 128)
+        plan.group = int(self._group) if self._method == "compressed-tensors" else 128
+        bm, bn = plan.block
+
+        meta, off = [], 0
+        quant_rows, copy_rows, late = [], [], []       # table rows per tensor; late = results only known at run time
+        shape_rows = []
+
+        def place(name, shape, dtype):
+            nonlocal off
+            esz = torch.empty((), dtype=dtype).element_size()
+            off = -(-off // esz) * esz                  # natural alignment; real weight shapes never need padding
+            nbytes = esz
+            for d in shape:
+                nbytes *= int(d)
+            meta.append(FlattenedTensorMetadata(name, torch.Size(shape), dtype, off, off + nbytes, nbytes))
+            start = off
+            off += nbytes
+            return start, nbytes
+
+        def add_copy(name, t, pi, ci):
+            start, nbytes = place(name, t.shape, t.dtype)
+            if not nbytes:
+                return
+            if t.is_cuda and t.device == device and t.is_contiguous():
+                copy_rows.append((len(meta) - 1, t.data_ptr(), start, nbytes))
+            else:
+                late.append((len(meta) - 1, pi, ci, None))
+
+        for pi, (mn, conv) in enumerate(params):
+            for op, n, t, ci in self._route(mn, conv):
+                if op == "pass":
+                    add_copy(n, t, pi, ci)
+                elif op == "loop":
+                    # per-tensor function at run time (here only for the shapes of its outputs); copied into place afterwards
+                    outs = quantize_params(self.args, mn, [(n, t)], self.config, self.transform_ue8m0)
+                    for on, ot in outs:
+                        place(on, ot.shape, ot.dtype)
+                        late.append((len(meta) - 1, pi, ci, on))
+                elif fp8:
+                    M, N = t.shape
+                    y0, _ = place(n, (M, N), FP8_DTYPE)
+                    s0, _ = place(n.replace(".weight", ".weight_scale_inv"), (ceildiv(M, bm), ceildiv(N, bn)), torch.float32)
+                    quant_rows.append((len(meta) - 2, [t.data_ptr(), y0, s0, M, N, t.stride(0), t.stride(1), N]))
+                else:
+                    M, N = t.shape
+                    p0, _ = place(n.replace(".weight", ".weight_packed"), (M, N // 8), torch.int32)
+                    s0, _ = place(n.replace(".weight", ".weight_scale"), (M, N // plan.group), torch.bfloat16)
+                    h0, _ = place(n.replace(".weight", ".weight_shape"), (2,), torch.int32)
+                    quant_rows.append((len(meta) - 3, [t.data_ptr(), p0, s0, M * N // plan.group]))
+                    shape_rows.append((len(meta) - 1, h0, (M, N)))
+
+        plan.keepalive = []
+        if shape_rows:
+            shapes = torch.tensor([sh for _, _, sh in shape_rows], dtype=torch.int32).to(device)
+            plan.keepalive.append(shapes)
+            for k, (mi, h0, _) in enumerate(shape_rows):
+                copy_rows.append((mi, shapes.data_ptr() + 8 * k, h0, 8))
+
+        # ---- one table row per work item, in bucket order (ordered by the metadata index of the item's first output)
+        width = 8 if fp8 else 4
+        blocks, order = [], []
+        if quant_rows:
+            first = torch.tensor([mi for mi, _ in quant_rows], dtype=torch.int64)
+            rows = [r for _, r in quant_rows]
+            table, owner, local = tile_table(rows, bm, bn) if fp8 else item_table(rows, plan.group)
+            blocks.append(table)
+            order.append(first[owner] * (1 << 32) + local)
+        if copy_rows:
+            c = torch.tensor([(mi, src, dst, nb) for mi, src, dst, nb in copy_rows], dtype=torch.int64)
+            counts = (c[:, 3] + _COPY - 1) // _COPY
+            owner = torch.repeat_interleave(torch.arange(len(copy_rows)), counts)
+            start = torch.cumsum(counts, 0) - counts
+            local = torch.arange(int(counts.sum()), dtype=torch.int64) - start[owner]
+            d = c[owner]
+            nb = torch.clamp(d[:, 3] - local * _COPY, max=_COPY)
+            zero = torch.zeros_like(nb)
+            if fp8:
+                blocks.append(torch.stack([d[:, 1] + local * _COPY, d[:, 2] + local * _COPY, zero, nb, zero,
+                                           torch.full_like(nb, _lib.BUCKET_COPY_MARK), zero, zero], dim=1))
+            else:
+                blocks.append(torch.stack([d[:, 1] + local * _COPY, d[:, 2] + local * _COPY, zero, -nb], dim=1))
+            order.append(d[:, 0] * (1 << 32) + local)
+        if blocks:
+            table = torch.cat(blocks, dim=0)
+            table = table[torch.argsort(torch.cat(order), stable=True)]
+            plan.items = table.contiguous().to(device)
+            plan.n_items = table.shape[0]
+            assert table.shape[1] == width
+        else:
+            plan.items, plan.n_items = None, 0
+        plan.total_bytes = off
+        plan.metadata = meta
+        plan.late_copies = late
+        plan.device = device
+        # The table holds the addresses of the inputs, not references: a cached plan is used again only when a later
+        # bucket presents tensors with the same names, shapes, strides AND addresses, and it keeps no weight alive.
+        return plan
+
+    # ------------------------------------------------------------------ run
+
+    def convert(self, params, out: torch.Tensor | None = None, bucket_id=None) -> FlattenedBucket:
+        """``bucket_id`` (any hashable, e.g. the bucket's index in the weight-sync loop) is a promise that every call
+        with this id presents the same names, shapes, strides and dtypes; then only the addresses are compared with
+        the cached table's (0.2 us per tensor instead of 4 us for the full identity), and a bucket whose tensors
+        moved gets a new table."""
+        params = [(mn, list(conv)) for mn, conv in params]
+        if not any(conv for _, conv in params):
+            return flatten_named_tensors([])
+        if bucket_id is not None:
+            key = ("id", bucket_id, tuple([t.data_ptr() for _, conv in params for _, t in conv]))
+        else:
+            key = (self._key(params), self._config_key, self.transform_ue8m0)
+        plan = self._plans.get(key)
+        if plan is None:
+            plan = self._build(params)
+            self._plans[key] = plan
+            while len(self._plans) > self._max:
+                self._plans.popitem(last=False)
+        else:
+            self._plans.move_to_end(key)
+        device = plan.device
+        if out is None:
+            out = torch.empty(plan.total_bytes, dtype=torch.uint8, device=device)
+        elif out.dtype != torch.uint8 or out.dim() != 1 or out.numel() < plan.total_bytes or not out.is_contiguous() \
+                or out.device != device or out.data_ptr() % 16:
+            raise ValueError(f"out must be a contiguous 16-byte aligned uint8 vector of at least {plan.total_bytes} bytes on {device}")
+        launches = 0
+        if plan.n_items:
+            lib = _lib.load()
+            with torch.cuda.device(device):
+                if plan.kind == "fp8":
+                    rc = lib.wq_fp8_bucket_convert(plan.items.data_ptr(), plan.n_items, out.data_ptr(), plan.block[0],
+                                                   plan.block[1], _lib.FP8_MODE_TRITON, _lib.stream_ptr(device))
+                else:
+                    rc = lib.wq_int4_bucket_convert(plan.items.data_ptr(), plan.n_items, out.data_ptr(), plan.group,
+                                                    _lib.stream_ptr(device))
+            _lib.check(rc, "BucketConverter.convert")
+            launches = 1
+        if plan.late_copies:
+            launches += self._late(plan, params, out)
+        return FlattenedBucket(out[:plan.total_bytes], plan.metadata, launches)
+
+    def _late(self, plan, params, out) -> int:
+        """Tensors outside the one-launch kernels: per-tensor functions, then one copy each."""
+        n, cache = 0, {}
+        for mi, pi, ci, out_name in plan.late_copies:
+            m = plan.metadata[mi]
+            mn, conv = params[pi]
+            name, t = conv[ci]
+            if out_name is None:
+                src = t
+            else:
+                if (pi, ci) not in cache:
+                    cache[(pi, ci)] = dict(quantize_params(self.args, mn, [(name, t)], self.config, self.transform_ue8m0))
+                    n += 1
+                src = cache[(pi, ci)][out_name]
+            out[m.start_idx:m.end_idx].copy_(src.detach().to(out.device).contiguous().flatten().view(torch.uint8))
+            n += 1
+        return n
+
+
+def quantize_bucket(args, params, quantization_config, transform_ue8m0: bool = True,
+                    converter: BucketConverter | None = None) -> FlattenedBucket:
+    """One-call form: ``params`` = ``[(megatron_name, [(hf_name, tensor), ...]), ...]`` for a whole bucket.  Pass the
+    same ``converter`` on every sync to reuse its cached tables."""
+    conv = converter or BucketConverter(args, quantization_config, transform_ue8m0)
+    return conv.convert(params)
+
+
+def per_param_loop(args, params, quantization_config, transform_ue8m0: bool = True):
+    """The loop this module replaces, on the per-tensor functions: -> [(hf_name, tensor), ...] in bucket order."""
+    outs = []
+    for mn, conv in params:
+        outs.extend(quantize_params(args, mn, list(conv), quantization_config, transform_ue8m0))
+    return outs

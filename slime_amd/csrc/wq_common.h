@@ -129,6 +129,48 @@ __device__ __forceinline__ int find_owner(const int64_t* __restrict__ start, int
     return lo;
 }
 
+// ---- pass-through work item of a bucket launch ------------------------------------------------------
+// Copies n bytes (n <= WQ_BUCKET_COPY_BYTES) with the 256 lanes of the workgroup.  The widest access that the
+// alignment of both pointers allows is used; all loads of the 16-byte form are issued before the first store.
+constexpr int kCopyItemBytes = WQ_BUCKET_COPY_BYTES;
+template <typename V>
+__device__ __forceinline__ void copy_units(const char* src, char* dst, int n)
+{
+    const int units = n / (int)sizeof(V);
+    for (int u = threadIdx.x; u < units; u += 256) stg_nt<V>(dst + (size_t)u * sizeof(V), ldg_nt<V>(src + (size_t)u * sizeof(V)));
+    for (int b = units * (int)sizeof(V) + threadIdx.x; b < n; b += 256) stg<uint8_t>(dst + b, ldg<uint8_t>(src + b));
+}
+__device__ __forceinline__ void copy_item(const void* src_, void* dst_, int n)
+{
+    const char* src = (const char*)src_;
+    char* dst = (char*)dst_;
+    const uintptr_t a = (uintptr_t)src | (uintptr_t)dst;
+    if ((a & 15) == 0) {
+        constexpr int kSteps = kCopyItemBytes / (256 * 16);
+        const int pieces = n >> 4;
+        u32x4 v[kSteps];
+#pragma unroll
+        for (int i = 0; i < kSteps; ++i) {
+            const int p = i * 256 + threadIdx.x;
+            v[i] = ldg_nt<u32x4>(src + (size_t)(p < pieces ? p : 0) * 16);      // lanes past the end re-read piece 0
+        }
+#pragma unroll
+        for (int i = 0; i < kSteps; ++i) {
+            const int p = i * 256 + threadIdx.x;
+            if (p < pieces) stg_nt<u32x4>(dst + (size_t)p * 16, v[i]);
+        }
+        for (int b = (pieces << 4) + threadIdx.x; b < n; b += 256) stg<uint8_t>(dst + b, ldg<uint8_t>(src + b));
+    } else if ((a & 7) == 0) {
+        copy_units<u32x2>(src, dst, n);
+    } else if ((a & 3) == 0) {
+        copy_units<uint32_t>(src, dst, n);
+    } else if ((a & 1) == 0) {
+        copy_units<uint16_t>(src, dst, n);
+    } else {
+        copy_units<uint8_t>(src, dst, n);
+    }
+}
+
 // ---- 16-lane (DPP row) all-reduce max.  After it every lane of the row holds the row max.
 template <int CTRL>
 __device__ __forceinline__ uint32_t dpp_u32(uint32_t v)
@@ -201,8 +243,19 @@ __device__ __forceinline__ float fp8_scale_triton(uint32_t amax_bf16_bits)
     return a / kFp8Max;
 }
 
-// The two torch modes divide every element by the scale; the Triton mode multiplies by its reciprocal.
-constexpr bool fp8_mode_divides(int mode) { return mode != WQ_FP8_MODE_TRITON; }
+// mode UE8M0: fp32 amax floored at 1e-4f, scale = the smallest power of two >= amax / 448 (a power of two maps to
+// itself, as 2^ceil(log2(.)) does).  amax / 448 is a normal number here (>= 2.2e-7); NaN and Inf pass through.
+__device__ __forceinline__ float fp8_scale_ue8m0(uint32_t amax_bf16_bits)
+{
+    float a = u2f(amax_bf16_bits << 16);
+    a = (a != a) ? a : fmaxf(a, 1e-4f);
+    const uint32_t u = f2u(a / kFp8Max);
+    if ((u & 0x7F800000u) == 0x7F800000u || (u & 0x007FFFFFu) == 0u) return u2f(u);
+    return u2f((u & 0x7F800000u) + 0x00800000u);
+}
+
+// The two torch modes divide every element by the scale; the Triton and UE8M0 modes multiply by its reciprocal.
+constexpr bool fp8_mode_divides(int mode) { return mode != WQ_FP8_MODE_TRITON && mode != WQ_FP8_MODE_UE8M0; }
 
 // Per-block constants of the element function.
 struct Fp8BlockParams {
@@ -217,6 +270,7 @@ __device__ __forceinline__ Fp8BlockParams fp8_block_params(uint32_t amax_bf16_bi
     Fp8BlockParams p;
     p.scale = MODE == WQ_FP8_MODE_TORCH          ? fp8_scale_torch(amax_bf16_bits)
               : MODE == WQ_FP8_MODE_TORCH_DEVICE ? fp8_scale_torch_device(amax_bf16_bits)
+              : MODE == WQ_FP8_MODE_UE8M0        ? fp8_scale_ue8m0(amax_bf16_bits)
                                                  : fp8_scale_triton(amax_bf16_bits);
     p.rcp = 1.0f / p.scale;
     p.fast = amax_bf16_bits < kBf16Inf;

@@ -1,7 +1,7 @@
 // bf16 -> block-FP8 (e4m3fn) quantisation for gfx950.
 //
-// Vector kernel (128x128 blocks, unit column stride, 16-byte aligned rows): one 512-thread
-// workgroup owns one block.  Each lane issues four 16-byte loads (8 bf16 each, rows rb+32*i), so a
+// Vector kernel (128x128 blocks, unit column stride, 16-byte aligned rows): one 256-thread
+// workgroup owns one block.  Each lane issues eight 16-byte loads (8 bf16 each, rows rb+16*i), so a
 // wavefront load covers four 256-byte row segments and the whole 32 KiB block is in flight before
 // the first use.  The block lives in registers from then on: amax is an integer max over the bf16
 // magnitude bits (packed 16-bit max), reduced over 16 lanes with DPP and across the workgroup
@@ -39,13 +39,14 @@ struct Fp8QuantArgs {
     const int64_t* tile_start;
     int32_t n_desc;
     int32_t bm, bn;
+    char* out_base;       // per-tile form only: when set, y and s of every descriptor are byte offsets from here
 };
 
 __device__ __forceinline__ bool desc_vector_ok(const wq_fp8_quant_desc& d)
 {
     // 128 rows of either operand must span fewer than 2^31 bytes: lane offsets are 32-bit
     return d.sx_n == 1 && (d.sx_m & 7) == 0 && (d.N & 7) == 0 && (d.sy_m & 7) == 0 &&
-           ((uintptr_t)d.x & 15) == 0 && ((uintptr_t)d.y & 7) == 0 && d.sx_m >= 0 && d.sx_m < (1 << 22) &&
+           ((uintptr_t)d.x & 15) == 0 && ((uintptr_t)d.y & 3) == 0 && d.sx_m >= 0 && d.sx_m < (1 << 22) &&
            d.sy_m >= 0 && d.sy_m < (1 << 22);
 }
 
@@ -169,6 +170,14 @@ __global__ __launch_bounds__(kTileThreads) void fp8_block_quant_kernel(const Fp8
     } else if (GROUPED == 2) {
         d = a.descs[tile];      // M, N: what is left of the tensor from this tile's origin; s: this tile's slot
         local = 0;
+        if (a.out_base) {
+            d.y = a.out_base + (uintptr_t)d.y;
+            d.s = (float*)(a.out_base + (uintptr_t)d.s);
+        }
+        if (d.sx_m == WQ_BUCKET_COPY_MARK) {       // pass-through item: M bytes from x to y
+            copy_item(d.x, d.y, (int)d.M);
+            return;
+        }
     } else {
         d = a.d;
     }
@@ -555,7 +564,8 @@ static void launch_block_quant_any(const void* x, int64_t M, int64_t N, int64_t 
 
 static bool known_mode(int mode)
 {
-    return mode == WQ_FP8_MODE_TORCH || mode == WQ_FP8_MODE_TRITON || mode == WQ_FP8_MODE_TORCH_DEVICE;
+    return mode == WQ_FP8_MODE_TORCH || mode == WQ_FP8_MODE_TRITON || mode == WQ_FP8_MODE_TORCH_DEVICE ||
+           mode == WQ_FP8_MODE_UE8M0;
 }
 
 template <int GROUPED>
@@ -566,6 +576,8 @@ static void launch_block_quant(const Fp8QuantArgs& a, int64_t tiles, int mode, h
         fp8_block_quant_kernel<WQ_FP8_MODE_TORCH, GROUPED><<<g, kTileThreads, kOccupancyPadBytes, st>>>(a, tiles);
     else if (mode == WQ_FP8_MODE_TORCH_DEVICE)
         fp8_block_quant_kernel<WQ_FP8_MODE_TORCH_DEVICE, GROUPED><<<g, kTileThreads, kOccupancyPadBytes, st>>>(a, tiles);
+    else if (mode == WQ_FP8_MODE_UE8M0)
+        fp8_block_quant_kernel<WQ_FP8_MODE_UE8M0, GROUPED><<<g, kTileThreads, kOccupancyPadBytes, st>>>(a, tiles);
     else
         fp8_block_quant_kernel<WQ_FP8_MODE_TRITON, GROUPED><<<g, kTileThreads, kOccupancyPadBytes, st>>>(a, tiles);
 }
@@ -682,11 +694,30 @@ WQ_EXPORT int wq_fp8_block_quant_any(const void* x, int dtype, int64_t M, int64_
     if (dtype != WQ_DTYPE_BF16 && dtype != WQ_DTYPE_F32 && dtype != WQ_DTYPE_F16) return WQ_ERR_MODE;
     int rc = check_desc_host(x, M, N, y, s, bm, bn, mode);
     if (rc) return rc;
+    if (mode == WQ_FP8_MODE_UE8M0) return WQ_ERR_UNSUPPORTED;      // power-of-two scales: bf16 weights only
     if (M == 0 || N == 0) return WQ_OK;
     hipStream_t st = (hipStream_t)stream;
     if (dtype == WQ_DTYPE_F32) launch_block_quant_any<float>(x, M, N, sx_m, sx_n, (uint8_t*)y, sy_m, s, bm, bn, mode, st);
     else if (dtype == WQ_DTYPE_F16) launch_block_quant_any<_Float16>(x, M, N, sx_m, sx_n, (uint8_t*)y, sy_m, s, bm, bn, mode, st);
     else launch_block_quant_any<uint16_t>(x, M, N, sx_m, sx_n, (uint8_t*)y, sy_m, s, bm, bn, mode, st);
+    WQ_LAUNCH_CHECK();
+    return WQ_OK;
+}
+
+WQ_EXPORT int wq_fp8_bucket_convert(const wq_fp8_quant_desc* items, int64_t n_items, void* out_base, int bm, int bn,
+                                    int mode, void* stream)
+{
+    if (n_items < 0 || bm <= 0 || bn <= 0) return WQ_ERR_SHAPE;
+    if (!known_mode(mode)) return WQ_ERR_MODE;
+    if (n_items == 0) return WQ_OK;
+    if (!items || !out_base) return WQ_ERR_NULL;
+    if ((int64_t)bm * bn > (1 << 30)) return WQ_ERR_TOO_LARGE;
+    Fp8QuantArgs a{};
+    a.descs = items;
+    a.bm = bm;
+    a.bn = bn;
+    a.out_base = (char*)out_base;
+    launch_block_quant<2>(a, n_items, mode, (hipStream_t)stream);
     WQ_LAUNCH_CHECK();
     return WQ_OK;
 }

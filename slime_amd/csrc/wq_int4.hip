@@ -27,6 +27,7 @@ struct Int4PackArgs {
     const wq_int4_pack_desc* descs;
     const int64_t* work_start;
     int32_t n_desc;
+    char* out_base;       // per-item form only: when set, packed and scale of every descriptor are byte offsets from here
 };
 
 template <int L>
@@ -121,6 +122,14 @@ __global__ __launch_bounds__(256) void int4_pack_kernel(const Int4PackArgs a, co
     } else if (GROUPED == 2) {
         d = a.descs[item];
         local = 0;
+        if (a.out_base) {
+            d.packed = (int32_t*)(a.out_base + (uintptr_t)d.packed);
+            d.scale = a.out_base + (uintptr_t)d.scale;
+        }
+        if (d.n_groups < 0) {                      // pass-through item: -n_groups bytes from x to packed
+            copy_item(d.x, d.packed, (int)-d.n_groups);
+            return;
+        }
     } else {
         d = a.d;
     }
@@ -199,10 +208,12 @@ template <typename T> __device__ __forceinline__ float ld_as_f32(const T* p, int
 template <> __device__ __forceinline__ float ld_as_f32<uint16_t>(const uint16_t* p, int64_t off)
 { return u2f((uint32_t)p[off] << 16); }
 template <> __device__ __forceinline__ float ld_as_f32<float>(const float* p, int64_t off) { return p[off]; }
+template <> __device__ __forceinline__ float ld_as_f32<double>(const double* p, int64_t off) { return (float)p[off]; }
 template <typename T> __device__ __forceinline__ void st_from_f32(T* p, int64_t off, float v);
 template <> __device__ __forceinline__ void st_from_f32<uint16_t>(uint16_t* p, int64_t off, float v)
 { p[off] = (uint16_t)f32_to_bf16_bits(v); }
 template <> __device__ __forceinline__ void st_from_f32<float>(float* p, int64_t off, float v) { p[off] = v; }
+template <> __device__ __forceinline__ void st_from_f32<double>(double* p, int64_t off, float v) { p[off] = (double)v; }
 
 __device__ __forceinline__ float wave64_max_f32(float v)
 {
@@ -516,7 +527,7 @@ WQ_EXPORT int wq_int4_fake_quant(const void* x, int dtype, int64_t M, int64_t N,
                                  int bn, int sym, void* q, void* scale, void* zero, void* stream)
 {
     if (M < 0 || N < 0 || bm <= 0 || bn <= 0) return WQ_ERR_SHAPE;
-    if (dtype != WQ_DTYPE_BF16 && dtype != WQ_DTYPE_F32) return WQ_ERR_MODE;
+    if (dtype != WQ_DTYPE_BF16 && dtype != WQ_DTYPE_F32 && dtype != WQ_DTYPE_F64) return WQ_ERR_MODE;
     if (((int64_t)bm * bn) % 32 != 0) return WQ_ERR_SHAPE;
     if (!((bm == 1 && bn % 32 == 0) || (32 % bn == 0))) return WQ_ERR_UNSUPPORTED;
     if ((int64_t)bm * bn > (1 << 30)) return WQ_ERR_TOO_LARGE;
@@ -532,6 +543,9 @@ WQ_EXPORT int wq_int4_fake_quant(const void* x, int dtype, int64_t M, int64_t N,
     } else if (dtype == WQ_DTYPE_BF16)
         int4_fake_quant_kernel<uint16_t><<<grid_for_items(cdiv64(groups, 4)), 256, 0, st>>>(
             (const uint16_t*)x, M, N, sx_m, sx_n, bm, bn, sym, (uint16_t*)q, (uint16_t*)scale, (uint16_t*)zero);
+    else if (dtype == WQ_DTYPE_F64)
+        int4_fake_quant_kernel<double><<<grid_for_items(cdiv64(groups, 4)), 256, 0, st>>>(
+            (const double*)x, M, N, sx_m, sx_n, bm, bn, sym, (double*)q, (double*)scale, (double*)zero);
     else
         int4_fake_quant_kernel<float><<<grid_for_items(cdiv64(groups, 4)), 256, 0, st>>>(
             (const float*)x, M, N, sx_m, sx_n, bm, bn, sym, (float*)q, (float*)scale, (float*)zero);
@@ -561,6 +575,19 @@ WQ_EXPORT int wq_int4_group_quant_pack_asym(const void* x, int64_t M, int64_t N,
     else int4_pack_asym_kernel<16><<<g, 256, kFakeOccupancyPadBytes, st>>>(xp, sx_m, gpr, pp, (uint16_t*)scale, (uint16_t*)zero, n_groups, items);
     WQ_LAUNCH_CHECK();
     return WQ_OK;
+}
+
+WQ_EXPORT int wq_int4_bucket_convert(const wq_int4_pack_desc* items, int64_t n_items, void* out_base, int group,
+                                     void* stream)
+{
+    if (n_items < 0) return WQ_ERR_SHAPE;
+    if (group != 32 && group != 64 && group != 128) return WQ_ERR_UNSUPPORTED;
+    if (n_items == 0) return WQ_OK;
+    if (!items || !out_base) return WQ_ERR_NULL;
+    Int4PackArgs a{};
+    a.descs = items;
+    a.out_base = (char*)out_base;
+    return launch_pack<2>(a, n_items, group, (hipStream_t)stream);
 }
 
 WQ_EXPORT int wq_int4_group_quant_pack_items(const wq_int4_pack_desc* items, int64_t n_items, int group, void* stream)

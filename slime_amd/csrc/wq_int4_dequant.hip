@@ -75,6 +75,32 @@ __global__ __launch_bounds__(256) void int4_dequant_kernel(const uint32_t* __res
     }
 }
 
+// Plain form for everything the kernel above does not take: scales in fp16 or fp32 (the reference converts whatever
+// dtype it finds with .to(float32)), groups of any size >= 1 that divide the row (group 1 = one scale per element, the
+// reference's group_size <= 0 case), rows that are not a multiple of 8 long (the last word of a row is cut).  One
+// lane per packed word; with an fp32 scale the product is rounded in fp32 and again to bf16, as in the reference.
+template <typename S> __device__ __forceinline__ float scale_as_f32(const void* p, int64_t i);
+template <> __device__ __forceinline__ float scale_as_f32<uint16_t>(const void* p, int64_t i) { return u2f((uint32_t)((const uint16_t*)p)[i] << 16); }
+template <> __device__ __forceinline__ float scale_as_f32<_Float16>(const void* p, int64_t i) { return (float)((const _Float16*)p)[i]; }
+template <> __device__ __forceinline__ float scale_as_f32<float>(const void* p, int64_t i) { return ((const float*)p)[i]; }
+
+template <typename S>
+__global__ __launch_bounds__(256) void int4_dequant_any_kernel(const uint32_t* __restrict__ packed, const void* __restrict__ scale,
+                                                              uint16_t* __restrict__ y, int64_t M, int64_t N, int64_t group)
+{
+    const int64_t words_per_row = (N + 7) / 8;
+    const int64_t k = ((int64_t)blockIdx.x + (int64_t)blockIdx.y * gridDim.x) * 256 + threadIdx.x;
+    if (k >= M * words_per_row) return;
+    const int64_t row = k / words_per_row, c0 = (k - row * words_per_row) * 8;
+    const uint32_t w = packed[k];
+    const int64_t groups_per_row = N / group;
+    for (int j = 0; j < 8 && c0 + j < N; ++j) {
+        const float s = scale_as_f32<S>(scale, row * groups_per_row + (c0 + j) / group);
+        const float f = (float)((int)((w >> (4 * j)) & 0xFu) - 8) * s;
+        y[row * N + c0 + j] = (uint16_t)f32_to_bf16_bits(f);
+    }
+}
+
 // ---- QAT straight-through forward ------------------------------------------------------------------
 
 constexpr int kSteGroupsPerWg = 64;
@@ -171,6 +197,28 @@ WQ_EXPORT int wq_int4_dequant(const int32_t* packed, const void* scale, void* y,
     const int64_t items = cdiv64(n_words, kDqWordsPerWg);
     int4_dequant_kernel<false><<<grid_for_items(items), 256, kDqOccupancyPadBytes, (hipStream_t)stream>>>(
         (const uint32_t*)packed, (const uint16_t*)scale, (uint16_t*)y, n_words, group, nullptr, items);
+    WQ_LAUNCH_CHECK();
+    return WQ_OK;
+}
+
+WQ_EXPORT int wq_int4_dequant_any(const int32_t* packed, const void* scale, int scale_dtype, void* y, int64_t M, int64_t N,
+                                  int group, void* stream)
+{
+    if (M < 0 || N < 0 || group <= 0 || N % group != 0) return WQ_ERR_SHAPE;
+    if (scale_dtype != WQ_DTYPE_BF16 && scale_dtype != WQ_DTYPE_F16 && scale_dtype != WQ_DTYPE_F32) return WQ_ERR_MODE;
+    if (M == 0 || N == 0) return WQ_OK;
+    if (!packed || !scale || !y) return WQ_ERR_NULL;
+    const int salign = scale_dtype == WQ_DTYPE_F32 ? 3 : 1;
+    if (((uintptr_t)y & 1) || ((uintptr_t)packed & 3) || ((uintptr_t)scale & salign)) return WQ_ERR_ALIGN;
+    const int64_t words = M * cdiv64(N, 8);
+    const dim3 g = grid_for_items(cdiv64(words, 256));
+    hipStream_t st = (hipStream_t)stream;
+    if (scale_dtype == WQ_DTYPE_F32)
+        int4_dequant_any_kernel<float><<<g, 256, 0, st>>>((const uint32_t*)packed, scale, (uint16_t*)y, M, N, group);
+    else if (scale_dtype == WQ_DTYPE_F16)
+        int4_dequant_any_kernel<_Float16><<<g, 256, 0, st>>>((const uint32_t*)packed, scale, (uint16_t*)y, M, N, group);
+    else
+        int4_dequant_any_kernel<uint16_t><<<g, 256, 0, st>>>((const uint32_t*)packed, scale, (uint16_t*)y, M, N, group);
     WQ_LAUNCH_CHECK();
     return WQ_OK;
 }

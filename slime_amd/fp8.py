@@ -123,6 +123,34 @@ def blockwise_cast_to_fp8_triton(x: torch.Tensor, block_size=None) -> tuple[torc
     return _block_quant(x, bm, bn, _lib.FP8_MODE_TRITON, "blockwise_cast_to_fp8_triton")
 
 
+def quant_weight_ue8m0(weight_dequant: torch.Tensor, weight_block_size) -> tuple[torch.Tensor, torch.Tensor]:
+    """Block quantisation with power-of-two (UE8M0) scales: the function the reference imports from sglang and calls
+    at quantizer_fp8.py:103-106 when the rollout engine wants DeepGEMM's scale format.  -> (qweight e4m3fn [M,N],
+    scale float32 [ceil(M/128), ceil(N/128)], every entry a power of two).  The arithmetic - fp32 amax floored at
+    1e-4, ``sf = 2 ** ceil(log2(amax / 448))``, ``q = x * (1 / sf)`` - is restated from sglang / DeepGEMM, which the
+    reference does not vendor: bit parity with them is unpinned.  bf16 weights, 128x128 blocks."""
+    assert list(weight_block_size) == [128, 128]
+    if weight_dequant.dtype != torch.bfloat16:
+        raise TypeError(f"quant_weight_ue8m0: only bfloat16 weights are supported (got {weight_dequant.dtype})")
+    n, k = weight_dequant.shape[-2:]
+    q, s = _block_quant(weight_dequant.reshape(-1, k), 128, 128, _lib.FP8_MODE_UE8M0, "quant_weight_ue8m0")
+    lead = tuple(weight_dequant.shape[:-2])
+    if lead:
+        if n % 128:
+            raise ValueError("quant_weight_ue8m0: batched weights need a row count that is a multiple of 128")
+        return q.view(weight_dequant.shape), s.view(*lead, n // 128, ceildiv(k, 128))
+    return q, s
+
+
+def transform_scale_ue8m0(sf: torch.Tensor, mn: int) -> torch.Tensor:
+    """Not provided.  The reference's ``transform_scale_ue8m0`` (sglang) repacks the scales into DeepGEMM's MN-major,
+    TMA-aligned, four-exponents-per-int32 layout - a memory layout of NVIDIA's tensor memory accelerator that no kernel
+    on this hardware reads, defined by a library the reference does not vendor."""
+    raise NotImplementedError(
+        "transform_scale_ue8m0: DeepGEMM's packed TMA-aligned UE8M0 layout is NVIDIA-specific and is not produced here; "
+        "call with transform_ue8m0=False to get the power-of-two scales as float32 (the form hf_checkpoint_saver uses)")
+
+
 def _dequant(x: torch.Tensor, s: torch.Tensor, block_size: int, mode: int, out_dtype: torch.dtype, what: str):
     _lib.require_gpu(x, what)
     assert x.is_contiguous() and s.is_contiguous()
@@ -171,6 +199,23 @@ _ITEM_TABLE_MIN_TENSORS = 64     # plans with at least this many tensors pre-res
 
 def _to_device_i64(rows, device) -> torch.Tensor:
     return torch.tensor(rows, dtype=torch.int64).to(device)
+
+
+def tile_table(rows, bm: int, bn: int):
+    """One descriptor per (bm x bn) tile, moved to the tile's origin, from per-tensor rows
+    ``[x, y, s, M, N, sx_m, sx_n, sy_m]`` (addresses, or byte offsets for the bucket launches; sizes and strides in
+    elements).  -> (int64 [tiles, 8] in tensor order, row-major tiles within a tensor; owner index per tile)."""
+    desc = torch.as_tensor(rows, dtype=torch.int64).reshape(-1, 8)
+    tm, tn = (desc[:, 3] + bm - 1) // bm, (desc[:, 4] + bn - 1) // bn
+    counts = tm * tn
+    owner = torch.repeat_interleave(torch.arange(desc.shape[0]), counts)
+    local = torch.arange(int(counts.sum()), dtype=torch.int64) - (torch.cumsum(counts, 0) - counts)[owner]
+    d = desc[owner]
+    kt = tn[owner]
+    r0, c0 = (local // kt) * bm, (local % kt) * bn
+    table = torch.stack([d[:, 0] + (r0 * d[:, 5] + c0 * d[:, 6]) * 2, d[:, 1] + r0 * d[:, 7] + c0,
+                         d[:, 2] + local * 4, d[:, 3] - r0, d[:, 4] - c0, d[:, 5], d[:, 6], d[:, 7]], dim=1)
+    return table, owner, local
 
 
 class Fp8QuantPlan:
@@ -222,16 +267,7 @@ class Fp8QuantPlan:
         # there and the table would cost more host time to build than it saves.
         self._tiles = None
         if len(rows) >= _ITEM_TABLE_MIN_TENSORS:
-            desc = torch.tensor(rows, dtype=torch.int64)             # x, y, s, M, N, sx_m, sx_n, sy_m
-            start = torch.tensor(starts, dtype=torch.int64)
-            owner = torch.repeat_interleave(torch.arange(len(rows)), start[1:] - start[:-1])
-            local = torch.arange(tiles, dtype=torch.int64) - start[owner]
-            d = desc[owner]
-            kt = (d[:, 4] + self.bn - 1) // self.bn
-            tm, tn = local // kt, local % kt
-            r0, c0 = tm * self.bm, tn * self.bn
-            table = torch.stack([d[:, 0] + (r0 * d[:, 5] + c0 * d[:, 6]) * 2, d[:, 1] + r0 * d[:, 7] + c0,
-                                 d[:, 2] + local * 4, d[:, 3] - r0, d[:, 4] - c0, d[:, 5], d[:, 6], d[:, 7]], dim=1)
+            table, _, _ = tile_table(rows, self.bm, self.bn)             # rows: x, y, s, M, N, sx_m, sx_n, sy_m
             self._tiles = table.contiguous().to(self.device)
         else:
             self._descs = _to_device_i64(rows, self.device)

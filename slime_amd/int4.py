@@ -28,7 +28,12 @@ def _dtype_sel(t: torch.Tensor, what: str) -> int:
         return _lib.DTYPE_BF16
     if t.dtype == torch.float32:
         return _lib.DTYPE_F32
-    raise TypeError(f"{what}: dtype {t.dtype} is not supported (bfloat16 or float32)")
+    if t.dtype == torch.float64:
+        return _lib.DTYPE_F64
+    # the reference dispatches on float, double and bfloat16 (fake_int4_quant_cuda.cu:352-354) and raises for the rest
+    names = {torch.float16: "Half", torch.int8: "Char", torch.uint8: "Byte", torch.int16: "Short", torch.int32: "Int",
+             torch.int64: "Long", torch.bool: "Bool"}
+    raise RuntimeError(f'"{what}" not implemented for \'{names.get(t.dtype, str(t.dtype).replace("torch.", ""))}\'')
 
 
 def fake_int4_quant_cuda(x: torch.Tensor, block_size: Sequence[int], sym: bool):
@@ -165,6 +170,21 @@ def pack_layer(weight: torch.Tensor, group_size: int, sym: bool = True):
 _ITEM_TABLE_MIN_TENSORS = 64     # plans with at least this many tensors pre-resolve every work item on the host
 
 
+def item_table(rows, group: int):
+    """One descriptor per work item of WQ_INT4_GROUPS_PER_WG groups from per-tensor rows ``[x, packed, scale, n_groups]``
+    (addresses, or byte offsets for the bucket launches).  -> (int64 [items, 4] in tensor order; owner and local index
+    per item)."""
+    per = _lib.INT4_GROUPS_PER_WG
+    desc = torch.as_tensor(rows, dtype=torch.int64).reshape(-1, 4)
+    counts = (desc[:, 3] + per - 1) // per
+    owner = torch.repeat_interleave(torch.arange(desc.shape[0]), counts)
+    local = torch.arange(int(counts.sum()), dtype=torch.int64) - (torch.cumsum(counts, 0) - counts)[owner]
+    d = desc[owner]
+    table = torch.stack([d[:, 0] + local * (per * group * 2), d[:, 1] + local * (per * group // 8 * 4),
+                         d[:, 2] + local * (per * 2), torch.clamp(d[:, 3] - local * per, max=per)], dim=1)
+    return table, owner, local
+
+
 class Int4PackPlan:
     """Symmetric quantise+pack of a fixed list of contiguous bf16 weights with one launch per ``run()``.
 
@@ -209,15 +229,7 @@ class Int4PackPlan:
         # sums.  A handful of tensors keeps the search.
         self._items = None
         if len(rows) >= _ITEM_TABLE_MIN_TENSORS:
-            per = _lib.INT4_GROUPS_PER_WG
-            desc = torch.tensor(rows, dtype=torch.int64)
-            start = torch.tensor(starts, dtype=torch.int64)
-            owner = torch.repeat_interleave(torch.arange(len(rows)), start[1:] - start[:-1])
-            local = torch.arange(work, dtype=torch.int64) - start[owner]
-            items = torch.stack([desc[owner, 0] + local * (per * self.group * 2),
-                                 desc[owner, 1] + local * (per * self.group // 8 * 4),
-                                 desc[owner, 2] + local * (per * 2),
-                                 torch.clamp(desc[owner, 3] - local * per, max=per)], dim=1)
+            items, _, _ = item_table(rows, self.group)
             self._items = items.contiguous().to(self.device)
         else:
             self._descs = torch.tensor(rows, dtype=torch.int64).to(self.device)
@@ -240,11 +252,17 @@ class Int4PackPlan:
 # ------------------------------------------------------------------------------------ inverse and QAT forward
 
 
+_SCALE_DTYPES = {torch.bfloat16: _lib.DTYPE_BF16, torch.float16: _lib.DTYPE_F16, torch.float32: _lib.DTYPE_F32}
+
+
 def dequantize_int4(weight_packed: torch.Tensor, weight_scale: torch.Tensor, weight_shape, group_size: int) -> torch.Tensor:
     """pack-quantized INT4 -> bf16: ``((nibble - 8).to(f32) * scale.to(f32)).to(bf16)`` with the scale of each
     ``group_size`` columns, the arithmetic of ``_dequantize_tensor`` in
     tools/convert_k2_thinking_int4_to_bf16.py:55-84 (its unpacking step is ``compressed_tensors.unpack_from_int32``:
-    nibble j of a word at bits [4j, 4j+4), offset 8).  ``weight_shape`` is the ``.weight_shape`` tensor or a tuple."""
+    nibble j of a word at bits [4j, 4j+4), offset 8, rows cut to their length).  ``weight_shape`` is the
+    ``.weight_shape`` tensor or a tuple.  As there, the scale may have any floating dtype (bf16, fp16 and fp32 are read
+    as stored, others are converted to fp32 first) and ``group_size <= 0`` means one scale per weight element.  bf16
+    scales with groups of a multiple of 8 take the bandwidth-tuned kernel."""
     _lib.require_gpu(weight_packed, "dequantize_int4")
     shape = tuple(int(v) for v in (weight_shape.view(-1).tolist() if isinstance(weight_shape, torch.Tensor) else weight_shape))
     if len(shape) != 2:
@@ -253,18 +271,26 @@ def dequantize_int4(weight_packed: torch.Tensor, weight_scale: torch.Tensor, wei
     if weight_packed.dtype != torch.int32 or tuple(weight_packed.shape) != (M, -(-N // 8)):
         raise ValueError(f"dequantize_int4: weight_packed {tuple(weight_packed.shape)} {weight_packed.dtype} does not "
                          f"match shape {shape}")
-    if group_size <= 0 or N % group_size != 0 or group_size % 8 != 0:
-        raise ValueError(f"dequantize_int4: group_size {group_size} must be a multiple of 8 that divides N={N}")
-    scale = weight_scale.unsqueeze(1) if weight_scale.dim() == 1 else weight_scale
-    if scale.numel() != M * (N // group_size):
+    group = int(group_size) if group_size > 0 else 1
+    if N % group != 0:
         raise ValueError(f"Scale shape {tuple(weight_scale.shape)} incompatible with weight shape {shape}")
-    scale = scale.to(torch.bfloat16).contiguous()
+    scale = weight_scale.unsqueeze(1) if (weight_scale.dim() == 1 and group_size > 0) else weight_scale
+    if scale.numel() != M * (N // group):
+        raise ValueError(f"Scale shape {tuple(weight_scale.shape)} incompatible with weight shape {shape}")
+    if scale.dtype not in _SCALE_DTYPES:
+        scale = scale.to(torch.float32)
+    scale = scale.contiguous()
     packed = weight_packed.contiguous()
     y = torch.empty((M, N), dtype=torch.bfloat16, device=packed.device)
     if M and N:
+        lib = _lib.load()
         with torch.cuda.device(packed.device):
-            rc = _lib.load().wq_int4_dequant(packed.data_ptr(), scale.data_ptr(), y.data_ptr(), M, N, int(group_size),
-                                             _lib.stream_ptr(packed.device))
+            if scale.dtype == torch.bfloat16 and group % 8 == 0:
+                rc = lib.wq_int4_dequant(packed.data_ptr(), scale.data_ptr(), y.data_ptr(), M, N, group,
+                                         _lib.stream_ptr(packed.device))
+            else:
+                rc = lib.wq_int4_dequant_any(packed.data_ptr(), scale.data_ptr(), _SCALE_DTYPES[scale.dtype], y.data_ptr(),
+                                             M, N, group, _lib.stream_ptr(packed.device))
         _lib.check(rc, "dequantize_int4")
     return y
 

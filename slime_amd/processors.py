@@ -7,18 +7,24 @@ returned ``[(hf_name, tensor), ...]`` lists.
 * ``quantize_params_fp8`` / ``_quantize_param`` - processors/quantizer_fp8.py:10-118
 * ``quantize_params_compressed_tensors``   - processors/quantizer_compressed_tensors.py:268-297
 
-The UE8M0 (power-of-two scale) re-quantisation that the reference takes only when sglang's DeepGEMM
-path is active (quantizer_fp8.py:103-108) does not exist on this hardware; ``transform_ue8m0`` is
-accepted and ignored, as it is in the reference whenever that path is off.
+The UE8M0 (power-of-two scale) re-quantisation, which the reference takes only when sglang reports a DeepGEMM rollout
+engine (quantizer_fp8.py:103-108), is off unless ``set_ue8m0_requant(True)`` switches it on; then ``_quantize_param``
+returns power-of-two float32 scales, and ``transform_ue8m0=True`` - the repacking into DeepGEMM's TMA layout - raises
+``NotImplementedError`` instead of being ignored.  With the switch off ``transform_ue8m0`` has no effect, exactly as in
+the reference whenever that path is off.
 """
 
 from __future__ import annotations
 
 import re
+import threading
+from collections import OrderedDict
 
 import torch
 
-from .fp8 import FP8_DTYPE, Fp8QuantPlan, blockwise_cast_to_fp8_triton, tensor_fp8
+from . import _lib
+from .fp8 import (FP8_DTYPE, blockwise_cast_to_fp8_triton, ceildiv, quant_weight_ue8m0, tensor_fp8, tile_table,
+                  transform_scale_ue8m0)
 from .int4 import pack_layer
 
 _LAYER_RE = re.compile(r"module\.module\.decoder\.layers\.(\d+)\.(.+)")
@@ -68,12 +74,32 @@ def _fp8_route(megatron_name: str):
     return "all" if rest in _DENSE_QUANTIZED else None
 
 
+_UE8M0_REQUANT = False
+
+
+def set_ue8m0_requant(enabled: bool) -> None:
+    """Stand-in for sglang's ``should_deepgemm_weight_requant_ue8m0`` (quantizer_fp8.py:103): the reference takes the
+    power-of-two-scale branch of ``_quantize_param`` only when the rollout engine runs DeepGEMM with UE8M0 scales,
+    which no engine on this hardware does - so it is off unless a caller switches it on here."""
+    global _UE8M0_REQUANT
+    _UE8M0_REQUANT = bool(enabled)
+
+
+def ue8m0_requant_enabled() -> bool:
+    return _UE8M0_REQUANT
+
+
 def _quantize_param(name, weight, weight_block_size, transform_ue8m0=True):
     """-> [(name, qweight), (scale_name, scale)]; block scales are named ``.weight_scale_inv``, per-tensor
     scales ``.weight_scale`` (quantizer_fp8.py:98-118)."""
     assert name.endswith(".weight"), f"Expected weight parameter, got {name}"
     if weight_block_size is not None:
-        qweight, scale = blockwise_cast_to_fp8_triton(weight, weight_block_size)
+        if _UE8M0_REQUANT:
+            qweight, scale = quant_weight_ue8m0(weight, weight_block_size=weight_block_size)
+            if transform_ue8m0:
+                scale = transform_scale_ue8m0(scale, mn=qweight.shape[-2])      # raises: NVIDIA-only layout
+        else:
+            qweight, scale = blockwise_cast_to_fp8_triton(weight, weight_block_size)
         scale_name = name.replace(".weight", ".weight_scale_inv")
     else:
         qweight, scale = tensor_fp8(weight)
@@ -96,9 +122,9 @@ def quantize_params_fp8(args, megatron_name, converted_named_params, quantizatio
         assert n.endswith(".weight"), f"Expected weight parameter, got {n}"
 
     # q/k/v or gate/up of one Megatron parameter: one grouped launch instead of one launch per tensor
-    if weight_block_size is not None and len(todo) > 1 and all(
-            p.is_cuda and p.dim() == 2 and p.dtype == torch.bfloat16 for _, p in todo):
-        outs = Fp8QuantPlan([p for _, p in todo], weight_block_size, mode=1).run()
+    if weight_block_size is not None and len(todo) > 1 and not _UE8M0_REQUANT and all(
+            p.is_cuda and p.dim() == 2 and p.dtype == torch.bfloat16 and p.numel() for _, p in todo):
+        outs = _group_cast([p for _, p in todo], weight_block_size)
         result = []
         for (n, _), (q, s) in zip(todo, outs):
             result += [(n, q), (n.replace(".weight", ".weight_scale_inv"), s)]
@@ -108,6 +134,56 @@ def quantize_params_fp8(args, megatron_name, converted_named_params, quantizatio
     for n, p in todo:
         result.extend(_quantize_param(n, p, weight_block_size, transform_ue8m0))
     return result
+
+
+_GROUP_TABLES: OrderedDict = OrderedDict()
+_GROUP_LOCK = threading.Lock()
+_GROUP_STATS = {"builds": 0, "hits": 0}
+_GROUP_MAX = 4096
+
+
+def plan_cache_info() -> dict:
+    """Counters of the descriptor-table cache behind the grouped launch of ``quantize_params_fp8``."""
+    return dict(_GROUP_STATS, entries=len(_GROUP_TABLES))
+
+
+def _group_cast(weights, block_size):
+    """``blockwise_cast_to_fp8_triton`` over a few tensors with one launch -> [(qweight, scale)], fresh outputs (slices
+    of one new allocation).  The per-tile table depends only on the addresses, shapes and strides of the inputs and is
+    cached: a parameter that comes back at the same addresses on the next sync costs no host-side table work."""
+    bm, bn = int(block_size[0]), int(block_size[1])
+    device = weights[0].device
+    key = (bm, bn, device.index, tuple((w.data_ptr(), tuple(w.shape), w.stride()) for w in weights))
+    with _GROUP_LOCK:
+        entry = _GROUP_TABLES.get(key)
+        if entry is not None:
+            _GROUP_TABLES.move_to_end(key)
+            _GROUP_STATS["hits"] += 1
+    if entry is None:
+        rows, layout, off = [], [], 0
+        for w in weights:
+            M, N = w.shape
+            tm, tn = ceildiv(M, bm), ceildiv(N, bn)
+            q0 = off
+            s0 = (q0 + M * N + 15) // 16 * 16
+            off = (s0 + 4 * tm * tn + 15) // 16 * 16
+            rows.append([w.data_ptr(), q0, s0, M, N, w.stride(0), w.stride(1), N])
+            layout.append((q0, M, N, s0, tm, tn))
+        table, _, _ = tile_table(rows, bm, bn)
+        entry = (table.contiguous().to(device), table.shape[0], layout, off)
+        with _GROUP_LOCK:
+            _GROUP_TABLES[key] = entry
+            _GROUP_STATS["builds"] += 1
+            while len(_GROUP_TABLES) > _GROUP_MAX:
+                _GROUP_TABLES.popitem(last=False)
+    table, n_tiles, layout, total = entry
+    flat = torch.empty(total, dtype=torch.uint8, device=device)
+    with torch.cuda.device(device):
+        rc = _lib.load().wq_fp8_bucket_convert(table.data_ptr(), n_tiles, flat.data_ptr(), bm, bn, _lib.FP8_MODE_TRITON,
+                                               _lib.stream_ptr(device))
+    _lib.check(rc, "quantize_params_fp8")
+    return [(flat[q0:q0 + M * N].view(FP8_DTYPE).view(M, N), flat[s0:s0 + 4 * tm * tn].view(torch.float32).view(tm, tn))
+            for q0, M, N, s0, tm, tn in layout]
 
 
 def _is_ignored(name: str, ignore_rules) -> bool:
@@ -157,4 +233,4 @@ def quantize_params(args, megatron_name, converted_named_params, quantization_co
 
 
 __all__ = ["quantize_params", "quantize_params_fp8", "_quantize_param", "quantize_params_compressed_tensors",
-           "FP8_DTYPE"]
+           "set_ue8m0_requant", "ue8m0_requant_enabled", "plan_cache_info", "FP8_DTYPE"]

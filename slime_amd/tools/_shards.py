@@ -88,3 +88,22 @@ def write_config(input_path: str, output_path: str, quantization_config: dict) -
 
 def to_device(t: torch.Tensor, dev: torch.device) -> torch.Tensor:
     return t.to(dev, non_blocking=True)
+
+
+def copy_matching_files(input_path: str, output_path: str, keep, skip=()) -> None:
+    """Copies (with metadata) the plain files of a checkpoint directory for which ``keep(name)`` holds."""
+    for name in os.listdir(input_path):
+        src = os.path.join(input_path, name)
+        if name not in skip and os.path.isfile(src) and keep(name):
+            shutil.copy2(src, os.path.join(output_path, name))
+
+
+def write_index_of_directory(output_path: str) -> None:
+    """model.safetensors.index.json rebuilt from the shards that are in the directory, with empty metadata."""
+    weight_map = {}
+    for fname in list_shards(output_path):
+        with safe_open(os.path.join(output_path, fname), framework="pt") as reader:
+            for key in reader.keys():
+                weight_map[key] = fname
+    with open(os.path.join(output_path, "model.safetensors.index.json"), "w") as f:
+        json.dump({"metadata": {}, "weight_map": weight_map}, f, indent=2)

@@ -12,11 +12,13 @@ from __future__ import annotations
 import argparse
 import gc
 import os
+import sys
 from concurrent.futures import ThreadPoolExecutor
 
 import torch
 
-from ..fp8 import Fp8QuantPlan, channel_fp8, tensor_fp8
+from .. import arith
+from ..fp8 import Fp8QuantPlan, block_fp8, channel_fp8, tensor_fp8
 from . import _shards
 
 # substrings that keep a "weight" tensor in its original dtype (tools/convert_hf_to_fp8.py:134-149)
@@ -55,9 +57,16 @@ def fp8_quantization_config(strategy: str, block_size, scale_fmt, modules_to_not
             "quant_method": "compressed-tensors", "quantization_status": "compressed"}
 
 
-def process_file(input_path, output_path, filename, strategy, block_size, result_collector):
+def process_file(input_path, output_path, filename, strategy, block_size, result_collector, arithmetic=None):
+    """``arithmetic``: the torch evaluation ("device" / "cpu") the caller resolved once; worker threads do not see the
+    caller's thread-local choice, so it travels as an argument."""
     if not filename.endswith(".safetensors"):
         return
+    with arith.torch_arithmetic(arithmetic or arith.get_torch_arithmetic()):
+        _process_file(input_path, output_path, filename, strategy, block_size, result_collector)
+
+
+def _process_file(input_path, output_path, filename, strategy, block_size, result_collector):
     dev = _shards.device()
     weights = _shards.read_shard(os.path.join(input_path, filename))
     out, skipped = {}, []
@@ -69,15 +78,24 @@ def process_file(input_path, output_path, filename, strategy, block_size, result
     if todo:
         on_gpu = [_shards.to_device(weights[k], dev) for k in todo]
         if strategy not in ("tensor", "channel"):
-            plan = Fp8QuantPlan(on_gpu, block_size)
-            plan.run()
-            flat_q, flat_s = plan.flat_q.cpu(), plan.flat_s.cpu()     # two copies for the whole shard
-            qbase, sbase = plan.flat_q.data_ptr(), plan.flat_s.data_ptr()
-            for k, w, (q, s) in zip(todo, on_gpu, plan.outputs):
-                qo = q.data_ptr() - qbase
-                so = (s.data_ptr() - sbase) // 4
-                out[k] = flat_q[qo:qo + q.numel()].view(torch.float8_e4m3fn).view(q.shape)
-                out[scale_name(k, block_size)] = flat_s[so:so + s.numel()].view(s.shape)
+            # bf16 matrices (what checkpoints hold) share one launch; other float dtypes, which block_fp8 also takes,
+            # go one by one through the kernel with that dtype's arithmetic
+            planned = [i for i, w in enumerate(on_gpu) if w.dtype == torch.bfloat16 and w.dim() == 2]
+            for i, (k, w) in enumerate(zip(todo, on_gpu)):
+                if i not in planned:
+                    q, s = block_fp8(w, block_size)
+                    out[k], out[scale_name(k, block_size)] = q.cpu(), s.cpu()
+            if planned:
+                plan = Fp8QuantPlan([on_gpu[i] for i in planned], block_size)
+                plan.run()
+                flat_q, flat_s = plan.flat_q.cpu(), plan.flat_s.cpu()     # two copies for the whole shard
+                qbase, sbase = plan.flat_q.data_ptr(), plan.flat_s.data_ptr()
+                for i, (q, s) in zip(planned, plan.outputs):
+                    k = todo[i]
+                    qo = q.data_ptr() - qbase
+                    so = (s.data_ptr() - sbase) // 4
+                    out[k] = flat_q[qo:qo + q.numel()].view(torch.float8_e4m3fn).view(q.shape)
+                    out[scale_name(k, block_size)] = flat_s[so:so + s.numel()].view(s.shape)
         else:
             fn = tensor_fp8 if strategy == "tensor" else channel_fp8
             for k, w in zip(todo, on_gpu):
@@ -98,8 +116,15 @@ def convert_fp8(input_path, output_path, strategy, block_size=None, max_workers=
     os.makedirs(output_path, exist_ok=True)
     _shards.copy_side_files(input_path, output_path)
     result = _shards.ConversionResult()
+    if scale_fmt is not None:
+        # exactly what the reference tool does with the flag (tools/convert_hf_to_fp8.py:197-198): the key goes into
+        # config.json and the arithmetic stays block_fp8's - the scales written are NOT powers of two
+        print(f"convert_hf_to_fp8: --scale-fmt {scale_fmt} only records \"scale_fmt\" in config.json, as the reference "
+              "tool does; the weight_scale_inv tensors keep ordinary float32 scales (power-of-two scales: "
+              "slime_amd.quant_weight_ue8m0)", file=sys.stderr)
+    arithmetic = arith.get_torch_arithmetic()        # resolved once, on the calling thread
     with ThreadPoolExecutor(max_workers=max_workers) as pool:
-        futures = [pool.submit(process_file, input_path, output_path, f, strategy, block_size, result)
+        futures = [pool.submit(process_file, input_path, output_path, f, strategy, block_size, result, arithmetic)
                    for f in _shards.list_shards(input_path)]
         for fut in futures:
             fut.result()

@@ -15,17 +15,17 @@ from __future__ import annotations
 import argparse
 import json
 import os
-import shutil
-from collections import defaultdict
+import re
 
 import torch
-from safetensors import safe_open
 
 from ..int4 import Int4DequantPlan, dequantize_int4
 from . import _shards
 
-_PROJECTIONS = ("gate_proj", "up_proj", "down_proj")
-_SUFFIXES = ("weight_packed", "weight_scale", "weight_shape")
+# <prefix>.mlp.experts.<e>.<proj>.<part> of a routed (not shared) expert
+_EXPERT_KEY = re.compile(r"^(?P<module>.*\.mlp\.experts\.[^.]+\.(?:gate_proj|up_proj|down_proj))"
+                         r"\.(?P<part>weight_packed|weight_scale|weight_shape)$")
+_PARTS = ("weight_packed", "weight_scale", "weight_shape")
 
 
 def _load_config(model_dir: str, config_path):
@@ -37,62 +37,46 @@ def _load_config(model_dir: str, config_path):
 
 
 def _dequantize_tensor(weight_packed, weight_scale, weight_shape, group_size: int) -> torch.Tensor:
-    """Name and arguments of the reference function (:55-84); the arithmetic runs in ``wq_int4_dequant``."""
-    if group_size <= 0:
-        raise ValueError("per-channel scales (group_size <= 0) are not produced by the INT4 converters and not supported")
-    if weight_scale.dtype != torch.bfloat16:
-        raise TypeError(f"weight_scale must be bfloat16 (what pack-quantized checkpoints store), got {weight_scale.dtype}")
+    """Name and arguments of the reference function (:55-84), any scale dtype and ``group_size <= 0`` included; the
+    arithmetic runs in the HIP kernels behind ``dequantize_int4``."""
     return dequantize_int4(weight_packed.to(torch.int32), weight_scale, weight_shape, group_size)
 
 
 def _is_quantized_weight_key(key: str) -> bool:
     """Routed (not shared) expert projections only (:87-96)."""
-    if ".mlp.experts." not in key or ".shared_experts." in key:
-        return False
-    return any(key.endswith(f".{proj}.{suffix}") for proj in _PROJECTIONS for suffix in _SUFFIXES)
+    return ".shared_experts." not in key and _EXPERT_KEY.match(key) is not None
 
 
 def convert_file(input_path: str, output_path: str, group_size: int, skip_existing: bool = True):
     if skip_existing and os.path.exists(output_path):
         return
     dev = _shards.device()
-    tensors = {}
-    experts = defaultdict(lambda: defaultdict(dict))
-    for key, tensor in _shards.read_shard(input_path).items():
-        parts = key.split(".")
-        if not _is_quantized_weight_key(key) or "experts" not in parts:
-            tensors[key] = tensor
-            continue
-        at = parts.index("experts")
-        experts[".".join(parts[:at + 2])][parts[-2]][parts[-1]] = tensor
-    names, packeds, scales, shapes = [], [], [], []
-    for prefix, components in experts.items():
-        for proj in _PROJECTIONS:
-            data = components.get(proj, {})
-            if not set(_SUFFIXES).issubset(data):
-                for suffix, value in data.items():          # incomplete: stays quantized
-                    tensors[f"{prefix}.{proj}.{suffix}"] = value
-                continue
-            if data["weight_scale"].dtype != torch.bfloat16:
-                raise TypeError(f"{prefix}.{proj}.weight_scale must be bfloat16 (what pack-quantized checkpoints store), "
-                                f"got {data['weight_scale'].dtype}")
-            names.append(f"{prefix}.{proj}.weight")
-            packeds.append(_shards.to_device(data["weight_packed"].to(torch.int32), dev))
-            scales.append(_shards.to_device(data["weight_scale"], dev))
-            shapes.append(data["weight_shape"])
-    if names:
-        if group_size <= 0 or group_size & (group_size - 1):
-            # not a power of two: one kernel launch per tensor
-            for name, p, sc, sh in zip(names, packeds, scales, shapes):
-                tensors[name] = _dequantize_tensor(p, sc, sh, group_size).cpu()
-        else:
-            plan = Int4DequantPlan(packeds, scales, shapes, group_size)     # one launch and one copy for the shard
-            plan.run()
-            flat = plan.flat_y.cpu()
-            base = plan.flat_y.data_ptr()
-            for name, y in zip(names, plan.outputs):
-                off = (y.data_ptr() - base) // 2
-                tensors[name] = flat[off:off + y.numel()].view(y.shape)
+    shard = _shards.read_shard(input_path)
+    modules = {}                                  # module name -> {part: tensor}, in shard order
+    for key, tensor in shard.items():
+        m = _EXPERT_KEY.match(key) if _is_quantized_weight_key(key) else None
+        if m:
+            modules.setdefault(m["module"], {})[m["part"]] = tensor
+    complete = {name: parts for name, parts in modules.items() if all(p in parts for p in _PARTS)}
+    # everything that is not part of a complete triple is kept as it is (an incomplete triple stays quantized)
+    tensors = {key: t for key, t in shard.items()
+               if not (_is_quantized_weight_key(key) and _EXPERT_KEY.match(key)["module"] in complete)}
+    one_launch = group_size > 0 and group_size & (group_size - 1) == 0 and group_size >= 8
+    bucket = []
+    for name, parts in complete.items():
+        packed = _shards.to_device(parts["weight_packed"].to(torch.int32), dev)
+        scale = _shards.to_device(parts["weight_scale"], dev)
+        if one_launch and scale.dtype == torch.bfloat16:
+            bucket.append((f"{name}.weight", packed, scale, parts["weight_shape"]))
+        else:       # fp16 / fp32 scales, per-element scales, odd group sizes: one launch per tensor
+            tensors[f"{name}.weight"] = _dequantize_tensor(packed, scale, parts["weight_shape"], group_size).cpu()
+    if bucket:
+        plan = Int4DequantPlan([b[1] for b in bucket], [b[2] for b in bucket], [b[3] for b in bucket], group_size)
+        plan.run()                                # one launch and one copy for the shard
+        flat, base = plan.flat_y.cpu(), plan.flat_y.data_ptr()
+        for (name, *_), y in zip(bucket, plan.outputs):
+            off = (y.data_ptr() - base) // 2
+            tensors[name] = flat[off:off + y.numel()].view(y.shape)
     os.makedirs(os.path.dirname(output_path), exist_ok=True)
     _shards.write_shard(tensors, output_path, with_format_tag=False)
 
@@ -114,27 +98,18 @@ def main(argv=None):
     if not os.path.isdir(model_dir):
         raise FileNotFoundError(f"Model directory not found: {model_dir}")
     _, _, group_size = _load_config(model_dir, args.config_path)
-    names = args.files if args.files else _shards.list_shards(model_dir)
-    if not names:
+    shards = [n for n in (args.files or _shards.list_shards(model_dir)) if os.path.isfile(os.path.join(model_dir, n))]
+    if not (args.files or shards):
         print("No safetensors checkpoints found.")
         return
-    for name in names:
-        path = os.path.join(model_dir, name)
-        if os.path.isfile(path):
-            print(f"Converting {name}")
-            convert_file(path, os.path.join(output_dir, name), group_size, skip_existing=not args.overwrite)
-    for fname in os.listdir(model_dir):
-        if fname == "model.safetensors.index.json":
-            continue
-        if fname.endswith(".json") or fname.endswith(".py") or fname.startswith("tokenizer"):
-            shutil.copy2(os.path.join(model_dir, fname), os.path.join(output_dir, fname))
-    weight_map = {}
-    for fname in _shards.list_shards(output_dir):
-        with safe_open(os.path.join(output_dir, fname), framework="pt") as reader:
-            for key in reader.keys():
-                weight_map[key] = fname
-    with open(os.path.join(output_dir, "model.safetensors.index.json"), "w") as f:
-        json.dump({"metadata": {}, "weight_map": weight_map}, f, indent=2)
+    for name in shards:
+        print(f"Converting {name}")
+        convert_file(os.path.join(model_dir, name), os.path.join(output_dir, name), group_size,
+                     skip_existing=not args.overwrite)
+    os.makedirs(output_dir, exist_ok=True)
+    _shards.copy_matching_files(model_dir, output_dir, skip=("model.safetensors.index.json",),
+                                keep=lambda n: n.endswith((".json", ".py")) or n.startswith("tokenizer"))
+    _shards.write_index_of_directory(output_dir)
     print(f"\nSuccessful! Output saved to: {output_dir}")
 
 

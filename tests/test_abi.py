@@ -119,3 +119,82 @@ def test_shim_module_does_not_shadow_the_function():
 
     with pytest.raises(RuntimeError):
         slime_amd.fake_int4_quant_cuda(torch.zeros(4, 32), (1, 32), True)      # reaches the function: CPU input refused
+
+
+def test_top_level_extension_name_resolves_unchanged():
+    # the reference's call sites do exactly this (tools/convert_hf_to_int4_direct.py:26, quantizer_compressed_tensors.py:236)
+    import importlib
+    import sys
+
+    sys.modules.pop("fake_int4_quant_cuda", None)
+    mod = importlib.import_module("fake_int4_quant_cuda")
+    import slime_amd.int4
+
+    assert mod.fake_int4_quant_cuda is slime_amd.int4.fake_int4_quant_cuda
+    assert os.path.dirname(os.path.abspath(mod.__file__)) == ROOT
+
+
+def test_torch_arithmetic_is_per_thread():
+    import threading
+
+    import slime_amd
+    from slime_amd import arith
+
+    assert slime_amd.get_torch_arithmetic() == "device"
+    seen, go, done = {}, threading.Event(), threading.Event()
+
+    def other():
+        seen["before"] = slime_amd.get_torch_arithmetic(), arith.fp8_torch_mode()
+        go.wait(5)
+        seen["during"] = slime_amd.get_torch_arithmetic(), arith.fp8_torch_mode(), arith.div7_rule()
+        with slime_amd.torch_arithmetic("cpu"):
+            seen["own"] = slime_amd.get_torch_arithmetic()
+        done.set()
+
+    t = threading.Thread(target=other)
+    t.start()
+    with slime_amd.torch_arithmetic("cpu"):
+        assert (slime_amd.get_torch_arithmetic(), arith.fp8_torch_mode(), arith.div7_rule()) == ("cpu", 0, 0)
+        with slime_amd.torch_arithmetic("device"):                 # re-entrant
+            assert arith.fp8_torch_mode() == 2
+        assert arith.fp8_torch_mode() == 0
+        go.set()
+        assert done.wait(5)
+    t.join()
+    assert seen == {"before": ("device", 2), "during": ("device", 2, 1), "own": "cpu"}
+    assert slime_amd.get_torch_arithmetic() == "device"
+    try:                                                            # the process default is what other threads inherit
+        slime_amd.set_torch_arithmetic("cpu")
+        got = []
+        t = threading.Thread(target=lambda: got.append(slime_amd.get_torch_arithmetic()))
+        t.start()
+        t.join()
+        assert got == ["cpu"]
+    finally:
+        slime_amd.set_torch_arithmetic("device")
+    with pytest.raises(ValueError):
+        slime_amd.set_torch_arithmetic("gpu")
+
+
+def test_ue8m0_requests_are_not_ignored():
+    import torch
+
+    import slime_amd
+    from slime_amd import processors
+
+    assert not processors.ue8m0_requant_enabled()
+    with pytest.raises(NotImplementedError, match="TMA"):
+        slime_amd.transform_scale_ue8m0(torch.ones(2, 2), mn=256)
+    with pytest.raises(AssertionError):
+        slime_amd.quant_weight_ue8m0(torch.zeros(128, 128, dtype=torch.bfloat16), [64, 64])
+    assert lib_rc("wq_fp8_block_quant", None, 4, 4, 4, 1, None, 4, None, 128, 128, 3, None) == -1      # mode 3 is known
+    assert lib_rc("wq_fp8_block_quant_any", None, 1, 4, 4, 4, 1, None, 4, None, 128, 128, 3, None) in (-1, -4)
+    assert lib_rc("wq_int4_dequant_any", None, None, 7, None, 4, 8, 8, None) == -3
+    assert lib_rc("wq_int4_dequant_any", None, None, 0, None, 4, 8, 3, None) == -2
+    assert lib_rc("wq_fp8_bucket_convert", None, 3, None, 128, 128, 1, None) == -1
+    assert lib_rc("wq_int4_bucket_convert", None, 3, None, 48, None) == -4
+    assert lib_rc("wq_delta_xor_noalloc", None, None, None, (4 << 30) + 1, 0, None, None) == -6
+
+
+def lib_rc(name, *args):
+    return getattr(_lib.load(), name)(*args)

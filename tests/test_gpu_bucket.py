@@ -1,0 +1,183 @@
+"""One-launch bucket conversion against the per-parameter loop it replaces: same names in the same order, same
+shapes and dtypes, same bytes - and against the CPU oracle for the quantised members."""
+
+import pytest
+import torch
+
+import slime_amd
+from oracle import c_oracle as C
+from slime_amd import bucket as B
+from tests import wq_inputs as I
+
+pytestmark = pytest.mark.gpu
+
+FP8_CFG = {"quant_method": "fp8", "fmt": "e4m3", "activation_scheme": "dynamic", "weight_block_size": [128, 128]}
+INT4_CFG = {"quant_method": "compressed-tensors",
+            "config_groups": {"group_0": {"weights": {"group_size": 128, "symmetric": True, "num_bits": 4}}},
+            "ignore": ["re:.*lm_head.*", "re:.*norm.*", "re:.*embed.*", "re:.*self_attn.*", "re:.*shared_experts.*",
+                       "re:.*mlp\\.(gate|up|gate_up|down)_proj.*", "re:.*mlp\\.gate\\.*"]}      # the converter's default rules
+L = "module.module.decoder.layers.{}."
+
+
+def _moe_layer(layer, cuda, seed, experts=3, hidden=256, ffn=384):
+    """A small MoE layer after name conversion: q/k/v from one fused parameter, gate/up as chunk views of one fc1
+    weight per expert, norms (1-D), a router (fp32) - the shapes of what _convert_to_hf_core yields."""
+    hf = f"model.layers.{layer}."
+    g = lambda *sh, s=0: I.weights(*sh, seed=seed + s).to(cuda)
+    params = [
+        (L.format(layer) + "self_attention.linear_qkv.layer_norm_weight", [(hf + "input_layernorm.weight", g(1, hidden, s=1)[0])]),
+        (L.format(layer) + "self_attention.linear_qkv.weight",
+         [(hf + "self_attn.q_proj.weight", g(512, hidden, s=2)), (hf + "self_attn.k_proj.weight", g(128, hidden, s=3)),
+          (hf + "self_attn.v_proj.weight", g(128, hidden, s=4))]),
+        (L.format(layer) + "self_attention.linear_proj.weight", [(hf + "self_attn.o_proj.weight", g(hidden, 512, s=5))]),
+        (L.format(layer) + "mlp.router.weight", [(hf + "mlp.gate.weight", g(experts, hidden, s=6).float())]),
+    ]
+    for e in range(experts):
+        fc1 = g(2 * ffn, hidden, s=10 + 2 * e)
+        gate, up = fc1.chunk(2, dim=0)
+        params.append((L.format(layer) + f"mlp.experts.linear_fc1.weight{e}",
+                       [(hf + f"mlp.experts.{e}.gate_proj.weight", gate), (hf + f"mlp.experts.{e}.up_proj.weight", up)]))
+        params.append((L.format(layer) + f"mlp.experts.linear_fc2.weight{e}",
+                       [(hf + f"mlp.experts.{e}.down_proj.weight", g(hidden, ffn, s=11 + 2 * e))]))
+    return params
+
+
+def _same_as_loop(bucket, want):
+    got = bucket.reconstruct_tensors()
+    assert [n for n, _ in got] == [n for n, _ in want]
+    for (n, a), (_, b), m in zip(got, want, bucket.metadata):
+        assert a.shape == b.shape and a.dtype == b.dtype and m.numel == b.numel() * b.element_size(), n
+        assert I.same_bits(a.cpu(), b.cpu()), n
+    ends = [m.end_idx for m in bucket.metadata]
+    assert all(m.start_idx >= e for m, e in zip(bucket.metadata[1:], ends))         # in order, no overlap
+    assert bucket.get_flattened_tensor().dtype == torch.uint8 and bucket.get_flattened_tensor().numel() == ends[-1]
+
+
+def test_fp8_bucket_equals_per_param_loop_and_oracle(cuda):
+    params = _moe_layer(0, cuda, 100) + _moe_layer(1, cuda, 200) + [
+        ("module.module.embedding.word_embeddings.weight", [("model.embed_tokens.weight", I.weights(1000, 256, seed=7).to(cuda))]),
+        ("module.module.decoder.final_layernorm.weight", [("model.norm.weight", I.weights(1, 256, seed=8)[0].to(cuda))])]
+    conv = B.BucketConverter(None, FP8_CFG)
+    out = conv.convert(params)
+    want = B.per_param_loop(None, params, FP8_CFG)
+    _same_as_loop(out, want)
+    assert out.launches == 1 and conv.plan_builds == 1
+    # every size here is a multiple of its successor's element size: the buffer is the plain concatenation
+    assert torch.equal(out.get_flattened_tensor(), B.flatten_named_tensors(want).get_flattened_tensor())
+    # quantised members against the CPU oracle (weight-sync arithmetic = mode 1)
+    named = dict(out.reconstruct_tensors())
+    for mn, cv in params:
+        for n, t in cv:
+            if n.endswith("proj.weight"):
+                qo, so = C.fp8_block_quant(t.cpu().contiguous(), (128, 128), 1)
+                assert torch.equal(named[n].cpu().view(torch.uint8), qo), n
+                assert torch.equal(named[n.replace(".weight", ".weight_scale_inv")].cpu().view(torch.int32), so.view(torch.int32)), n
+    # same tensors again: cached table, fresh buffer; inputs changed in place: outputs follow
+    params[1][1][0][1].mul_(3)
+    out2 = conv.convert(params)
+    assert conv.plan_builds == 1 and out2.get_flattened_tensor().data_ptr() != out.get_flattened_tensor().data_ptr()
+    _same_as_loop(out2, B.per_param_loop(None, params, FP8_CFG))
+    # same shapes at other addresses: a new table
+    moved = [(mn, [(n, t.clone()) for n, t in cv]) for mn, cv in params]
+    _same_as_loop(conv.convert(moved), B.per_param_loop(None, moved, FP8_CFG))
+    assert conv.plan_builds == 2
+    # into a caller-owned buffer
+    buf = torch.empty(out.get_flattened_tensor().numel() + 64, dtype=torch.uint8, device=cuda)
+    out3 = conv.convert(moved, out=buf)
+    assert out3.get_flattened_tensor().data_ptr() == buf.data_ptr()
+    _same_as_loop(out3, B.per_param_loop(None, moved, FP8_CFG))
+
+
+def test_fp8_bucket_odd_members(cuda):
+    # ragged shapes, a strided quantised member (generic tiles), a non-contiguous pass-through, members whose byte
+    # sizes put the next one at odd offsets (4-byte and 2-byte aligned destinations), an empty tensor, an fp32 weight
+    # and a *_scale entry that the expert rule drops
+    w = I.weights(300, 200, seed=1).to(cuda)
+    wide = I.weights(264, 520, seed=2).to(cuda)
+    params = [
+        ("module.module.decoder.layers.0.mlp.router.expert_bias", [("model.layers.0.mlp.gate.e_score_correction_bias", torch.arange(3, device=cuda, dtype=torch.float32))]),
+        (L.format(0) + "self_attention.linear_proj.weight", [("model.layers.0.self_attn.o_proj.weight", w)]),
+        ("module.module.x.odd", [("odd.bf16", I.weights(1, 3, seed=3)[0].to(cuda))]),
+        (L.format(0) + "mlp.linear_fc2.weight", [("model.layers.0.mlp.down_proj.weight", wide[:, 8:][:, ::2])]),
+        ("module.module.x.strided", [("strided.pass", wide.t())]),
+        ("module.module.x.empty", [("empty", torch.empty(0, 4, device=cuda, dtype=torch.bfloat16))]),
+        (L.format(0) + "mlp.linear_fc1.weight", [("model.layers.0.mlp.gate_proj.weight", I.weights(7, 7168, seed=4).to(cuda)),
+                                                 ("model.layers.0.mlp.up_proj.weight", I.weights(129, 127, seed=5).to(cuda).float())]),
+        (L.format(0) + "mlp.experts.linear_fc1.weight0", [("model.layers.0.mlp.experts.0.gate_proj.weight", I.weights(128, 128, seed=6).to(cuda)),
+                                                         ("model.layers.0.mlp.experts.0.gate_proj.weight_scale", torch.ones(1, device=cuda))]),
+    ]
+    conv = B.BucketConverter(None, FP8_CFG)
+    want = B.per_param_loop(None, params, FP8_CFG)
+    assert "model.layers.0.mlp.experts.0.gate_proj.weight_scale" not in [n for n, _ in want]
+    for _ in range(2):
+        _same_as_loop(conv.convert(params), want)
+    assert conv.plan_builds == 1
+    o, so = C.fp8_block_quant(wide[:, 8:][:, ::2].cpu(), (128, 128), 1)
+    named = dict(conv.convert(params).reconstruct_tensors())
+    assert torch.equal(named["model.layers.0.mlp.down_proj.weight"].cpu().view(torch.uint8), o)
+
+
+def test_bucket_other_configurations(cuda):
+    params = _moe_layer(0, cuda, 300, experts=2)
+    for cfg in (None, {"quant_method": "awq"}, {**FP8_CFG, "weight_block_size": None}, {**FP8_CFG, "weight_block_size": [64, 32]}):
+        conv = B.BucketConverter(None, cfg)
+        _same_as_loop(conv.convert(params), B.per_param_loop(None, params, cfg))
+    assert B.BucketConverter(None, FP8_CFG).convert([]).get_flattened_tensor().numel() == 0
+    assert B.quantize_bucket(None, [("m", [])], FP8_CFG).get_metadata() == []
+    with pytest.raises(ValueError):
+        B.BucketConverter(None, FP8_CFG).convert(params, out=torch.empty(16, dtype=torch.uint8, device=cuda))
+
+
+def test_int4_bucket_equals_per_param_loop_and_oracle(cuda):
+    params = _moe_layer(0, cuda, 400) + _moe_layer(3, cuda, 500) + [
+        ("module.module.output_layer.weight", [("lm_head.weight", I.weights(640, 256, seed=9).to(cuda))])]
+    conv = B.BucketConverter(None, INT4_CFG)
+    out = conv.convert(params)
+    want = B.per_param_loop(None, params, INT4_CFG)
+    _same_as_loop(out, want)
+    assert out.launches == 1
+    assert torch.equal(out.get_flattened_tensor(), B.flatten_named_tensors(want).get_flattened_tensor())
+    named = dict(out.reconstruct_tensors())
+    n_q = 0
+    for mn, cv in params:
+        for n, t in cv:
+            if ".experts." in n:
+                po, so, _ = C.int4_pack_layer(t.cpu().contiguous(), 128, True)
+                assert torch.equal(named[n.replace(".weight", ".weight_packed")].cpu(), po), n
+                assert I.same_bits(named[n.replace(".weight", ".weight_scale")].cpu(), so), n
+                assert named[n.replace(".weight", ".weight_shape")].tolist() == list(t.shape)
+                n_q += 1
+            elif "self_attn" in n or n == "lm_head.weight":
+                assert I.same_bits(named[n].cpu(), t.cpu())              # ignored by the rules: passes through
+    assert n_q == 18
+    _same_as_loop(conv.convert(params), want)
+    assert conv.plan_builds == 1
+
+
+def test_int4_bucket_asymmetric_and_other_groups(cuda):
+    params = _moe_layer(0, cuda, 600, experts=2)
+    asym = {**INT4_CFG, "config_groups": {"group_0": {"weights": {"group_size": 128, "symmetric": False}}}}
+    g32 = {**INT4_CFG, "config_groups": {"group_0": {"weights": {"group_size": 32, "symmetric": True}}}}
+    g256 = {**INT4_CFG, "config_groups": {"group_0": {"weights": {"group_size": 256, "symmetric": True}}}, "ignore": []}
+    everything = {**INT4_CFG, "ignore": []}       # nothing ignored: the fp32 router goes through the per-tensor path
+    for cfg in (asym, g32, everything):
+        _same_as_loop(B.BucketConverter(None, cfg).convert(params), B.per_param_loop(None, params, cfg))
+    one = [(L.format(0) + "mlp.experts.linear_fc2.weight0", [("model.layers.0.mlp.experts.0.down_proj.weight", I.weights(64, 512, seed=3).to(cuda))])]
+    _same_as_loop(B.BucketConverter(None, g256).convert(one), B.per_param_loop(None, one, g256))
+
+
+def test_quantize_params_fp8_caches_its_table(cuda):
+    # the per-parameter entry point groups q/k/v (or gate/up) of one parameter into one launch; the same tensors
+    # presented again reuse the cached descriptor table
+    from slime_amd import processors
+
+    params = _moe_layer(0, cuda, 700, experts=1)
+    mn, cv = params[1]
+    first = processors.quantize_params_fp8(None, mn, cv, FP8_CFG)
+    builds = processors.plan_cache_info()["builds"]
+    again = processors.quantize_params_fp8(None, mn, cv, FP8_CFG)
+    assert processors.plan_cache_info()["builds"] == builds
+    for (n0, a), (n1, b), (_, t) in zip(first[::2], again[::2], cv):
+        qo, _ = C.fp8_block_quant(t.cpu(), (128, 128), 1)
+        assert n0 == n1 and torch.equal(a.cpu().view(torch.uint8), qo) and torch.equal(b.cpu().view(torch.uint8), qo)
+        assert a.data_ptr() != b.data_ptr()          # fresh outputs on every call, like the reference

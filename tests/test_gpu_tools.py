@@ -188,3 +188,29 @@ def test_convert_int4_experts_to_bf16(tmp_path, cuda):
     before = os.path.getmtime(out / "model-00001-of-00001.safetensors")
     K2.main(["--model-dir", str(src), "--output-dir", str(out)])
     assert os.path.getmtime(out / "model-00001-of-00001.safetensors") == before
+
+
+def test_convert_int4_experts_with_other_scale_dtypes(tmp_path, cuda):
+    # the reference converts whatever scale dtype the shard holds with .to(float32) (:150): fp16 and fp32 scales go
+    # through, each against the oracle with that dtype's arithmetic; bf16 members of the same shard share one launch
+    src = tmp_path / "int4"
+    src.mkdir()
+    shard, want = {}, {}
+    for e, dt in enumerate((torch.bfloat16, torch.float16, torch.float32)):
+        w = I.weights(48, 256, seed=20 + e)
+        p, sc, _ = C.int4_pack_layer(w, 32, True)
+        sc = (sc.float() * (1 + 2.0 ** -12)).to(dt) if dt != torch.bfloat16 else sc     # not bf16-representable
+        name = f"model.layers.1.mlp.experts.{e}.down_proj"
+        shard[f"{name}.weight_packed"], shard[f"{name}.weight_scale"] = p, sc
+        shard[f"{name}.weight_shape"] = torch.tensor([48, 256], dtype=torch.int32)
+        want[f"{name}.weight"] = C.int4_dequant_any(p, sc, (48, 256), 32)
+    save_file(shard, str(src / "model.safetensors"))
+    json.dump({"hidden_size": 256, "moe_intermediate_size": 48,
+               "quantization_config": {"config_groups": {"group_0": {"weights": {"group_size": 32}}}}},
+              open(src / "config.json", "w"))
+    out = tmp_path / "bf16"
+    K2.main(["--model-dir", str(src), "--output-dir", str(out)])
+    got = load_file(str(out / "model.safetensors"))
+    assert set(got) == set(want)
+    for name, t in want.items():
+        assert got[name].dtype == torch.bfloat16 and I.same_bits(got[name], t), name

@@ -371,3 +371,49 @@ def test_fp32_floor_is_fp32_1e_12():
     assert Fraction(s0.item()) == rn_f32(rn_f32(Fraction(1, 10 ** 12)) / 448)
     _, s2 = C.fp8_block_quant(w, (4, 4), 2)
     assert Fraction(s2.item()) == rn_f32(rn_f32(Fraction(1, 10 ** 12)) * rn_f32(Fraction(1, 448)))
+
+
+# ------------------------------------------------------------------ power-of-two (UE8M0) scales: PARITY UNPINNED
+# The arithmetic lives in sglang / DeepGEMM, which the reference does not vendor.  These tests pin what the
+# mathematics fixes, and that the two restatements (literal log2 / ceil / pow chain, exponent arithmetic) agree.
+
+def test_ue8m0_scale_is_the_smallest_power_of_two_not_below_amax_over_448_for_every_bf16_amax():
+    bits = torch.arange(0, 0x7F80, dtype=torch.int32)
+    n = bits.numel()
+    w = torch.zeros(128, 128 * n, dtype=torch.bfloat16)
+    w[0, ::128] = bits.to(torch.int16).view(torch.bfloat16)
+    q, s = T.quant_weight_ue8m0_ref(w)
+    qo, so = C.fp8_block_quant(w, (128, 128), 3)
+    assert torch.equal(s.view(torch.int32), so.view(torch.int32)) and torch.equal(q.view(torch.uint8), qo)
+    s64 = so.double().view(-1)
+    amax = w[0, ::128].double().clamp(min=float(torch.tensor(1e-4, dtype=torch.float32)))
+    mant, _ = torch.frexp(s64)
+    assert (mant == 0.5).all()                                         # a power of two
+    assert (s64 * 448 >= amax).all() and (s64 * 448 < 2 * amax).all()  # the smallest one that keeps |q| <= 448
+    exact = amax == 448 * s64                                          # amax = 1.75 * 2^k: amax / 448 is itself a power of two
+    assert int(exact.sum()) > 100
+
+
+def test_ue8m0_codes_are_one_rounding_of_an_exact_scaling():
+    w = I.zero_blocks(I.weights(300, 520, seed=3), 0.2, seed=1)
+    w[200:, 300:] = I.subnormal_block(100, 220, seed=2)
+    qo, so = C.fp8_block_quant(w, (128, 128), 3)
+    q, s = T.quant_weight_ue8m0_ref(w)
+    assert torch.equal(q.view(torch.uint8), qo) and torch.equal(s.view(torch.int32), so.view(torch.int32))
+    full = T._expand_scale(so, 300, 520, 128).double()
+    exact = w.double() / full                                           # a power-of-two divisor: exact in fp64 and fp32
+    assert (exact.abs() <= 448).all()
+    assert torch.equal(qo, C.f32_to_e4m3fn(exact.float()))              # codes = RNE of the exactly scaled value
+    assert ((qo & 0x7F) <= 0x7E).all()
+    deq = C.e4m3fn_to_f32(qo).double() * full
+    step = full * torch.clamp(2.0 ** (torch.floor(torch.log2(exact.abs().clamp(min=2.0 ** -6))) - 3), min=2.0 ** -9)
+    assert ((deq - w.double()).abs() <= step / 2).all()                 # within half an e4m3 step of the block
+    zero = so[0, 4] if float(w[:128, 512:].abs().max()) == 0 else None
+    assert so.min() >= 2.0 ** -22                                       # the 1e-4 floor: 1e-4 / 448 rounds up to 2^-22
+
+
+def test_ue8m0_differs_from_the_plain_block_scale():
+    w = I.weights(256, 256, seed=5)
+    _, s0 = C.fp8_block_quant(w, (128, 128), 1)
+    _, s3 = C.fp8_block_quant(w, (128, 128), 3)
+    assert (s3 >= s0).all() and not torch.equal(s0, s3)

@@ -298,3 +298,61 @@ def test_fake_ste_is_idempotent_up_to_scale_rounding_and_bounded():
     assert ((y.float().view(64, 8, 128) - w.float().view(64, 8, 128)).abs() <= step * 0.5 * 1.02 + amax * 2.0 ** -8).all()
     # at most 15 distinct values per group
     assert max(len(set(r)) for r in y.float().view(-1, 128).tolist()) <= 15
+
+
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("gs", [128, 32, 24, 1, -1])
+def test_int4_dequant_any_c_equals_torch(dt, gs):
+    # the inputs the reference's _dequantize_tensor accepts beyond bf16 scales and whole groups of 8: other scale
+    # dtypes (converted with .to(float32)), one scale per element (group_size <= 0), rows not a multiple of 8 long
+    g = I.gen(gs + 200)
+    M, N = 9, 96 if gs in (24, 32) else 128
+    if gs in (1, -1):
+        N = 52                                                      # ragged: 7 words per row, the last one cut
+    packed = torch.randint(-2 ** 31, 2 ** 31 - 1, (M, -(-N // 8)), generator=g, dtype=torch.int64).to(torch.int32)
+    group = gs if gs > 0 else 1
+    scale = (torch.rand(M, N // group, generator=g) * 0.02 + 1e-4).to(dt)
+    want = T.int4_dequant_ref(packed, scale, (M, N), gs)
+    got = C.int4_dequant_any(packed, scale, (M, N), gs)
+    assert I.same_bits(got, want)
+    if dt == torch.bfloat16 and gs in (128, 32):
+        assert I.same_bits(got, C.int4_dequant(packed, scale, (M, N), gs))
+
+
+def test_int4_dequant_fp32_scale_rounds_twice():
+    # fp32 scale: (int8 * scale) is rounded to fp32 and then to bf16.  With scale = RN(m / 3) for a bf16 midpoint m the
+    # exact product 3 * scale lies a hair off m, the fp32 rounding lands ON m and the tie then goes to even - a single
+    # rounding of the exact product would go to the nearer neighbour instead.
+    from fractions import Fraction
+
+    from tests import exact_arith as X
+
+    word = 0xBBBBBBBB - (1 << 32)                                  # eight nibbles 0xB: q = 3
+    packed = torch.tensor([[word]], dtype=torch.int32)
+    hits = 0
+    for k in range(64):
+        mid = (1 + (2 * k + 1) * 2.0 ** -8) * 2.0 ** (k % 5 - 2)
+        s = torch.tensor([[mid / 3]], dtype=torch.float32)
+        got = C.int4_dequant_any(packed, s, (1, 8), 8)
+        exact = 3 * Fraction(float(s))
+        twice = X.rn_bf16(X.rn_f32(exact))
+        if exact == Fraction(mid):                                  # m divisible by 3: nothing to round
+            continue
+        assert X.rn_f32(exact) == Fraction(mid)
+        assert all(Fraction(float(v)) == twice for v in got[0])
+        assert I.same_bits(got, T.int4_dequant_ref(packed, s, (1, 8), 8))
+        hits += twice != X.rn_bf16(exact)
+    assert hits >= 16
+
+
+@pytest.mark.parametrize("sym", [True, False])
+def test_fake_quant_fp64_converts_to_fp32_on_load(sym):
+    # the reference dispatches float, double and bfloat16 (fake_int4_quant_cuda.cu:352) and casts each element to
+    # float first (:70): an fp64 input gives the fp32 input's codes, stored as doubles
+    g = I.gen(5)
+    x64 = torch.randn(8, 256, generator=g, dtype=torch.float64) * 0.02
+    q, s, z = C.int4_fake_quant(x64, (1, 128), sym)
+    q32, s32, z32 = C.int4_fake_quant(x64.float(), (1, 128), sym)
+    assert q.dtype == torch.float64 and torch.equal(q, q32.double()) and torch.equal(s, s32.double())
+    if not sym:
+        assert torch.equal(z, z32.double())
