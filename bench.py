@@ -336,7 +336,12 @@ def bench_bucket(dev, steps, warmup, layers):
     one_bucket()
     torch.cuda.synchronize()
     first_ms = (time.perf_counter() - t0) * 1e3
-    wall1, ev1, _ = _time_launches(one_bucket, steps, warmup)
+    wall1, _, _ = _time_launches(one_bucket, steps, warmup)
+    conv.time_kernels = True
+    for _ in range(steps):
+        one_bucket()
+    torch.cuda.synchronize()
+    ev1 = conv.kernel_ms() / steps
     launches1 = state["out"].launches
     named = dict(state["out"].reconstruct_tensors())
     for n, t in (quantised[0], quantised[5], quantised[-1]):
@@ -345,16 +350,22 @@ def bench_bucket(dev, steps, warmup, layers):
         assert torch.equal(named[n.replace(".weight", ".weight_scale_inv")].cpu().view(torch.int32), so.view(torch.int32))
     assert torch.equal(named["model.layers.0.mlp.gate.weight"], whole[4][1][0][1])
     del named
-    wallL, evL, _ = _time_launches(per_layer_buckets, steps, warmup)
+    conv.time_kernels = False
+    wallL, _, _ = _time_launches(per_layer_buckets, steps, warmup)
+    conv.time_kernels = True
+    for _ in range(steps):
+        per_layer_buckets()
+    torch.cuda.synchronize()
+    evL = conv.kernel_ms() / steps
     launchesL = sum(b.launches for b in state["out"])
     out = {"workload": f"Qwen3-30B-A3B-shaped state dict after name conversion, {layers} layers, {n_tensors} tensors "
                        f"({len(quantised)} quantised to block-FP8 with the weight-sync arithmetic, the rest copied), written "
                        "into the one uint8 buffer + metadata a FlattenedTensorBucket consumer reads; fresh output buffer per sync",
            "tensors": n_tensors, "bf16_GB": 2 * elements / 1e9,
-           "one_bucket": {"launches_per_sync": launches1, "ms_per_sync_gpu": ev1, "ms_per_sync_wall": wall1,
+           "one_bucket": {"launches_per_sync": launches1, "ms_per_sync_kernels": ev1, "ms_per_sync_wall": wall1,
                           "first_call_ms_table_build": first_ms, "hbm_frac": algo_bytes / ev1 / 1e6 / HBM_PEAK_GBS,
                           "bf16_GBps": 2 * elements / ev1 / 1e6},
-           "bucket_per_layer": {"launches_per_sync": launchesL, "ms_per_sync_gpu": evL, "ms_per_sync_wall": wallL,
+           "bucket_per_layer": {"launches_per_sync": launchesL, "ms_per_sync_kernels": evL, "ms_per_sync_wall": wallL,
                                 "hbm_frac": algo_bytes / evL / 1e6 / HBM_PEAK_GBS, "bf16_GBps": 2 * elements / evL / 1e6},
            "table_builds": conv.plan_builds, "parity_tensors_checked": 3}
     del state, conv, whole, per_layer, quantised
@@ -389,8 +400,7 @@ def bench_int4_pack(dev, steps, warmup, layers):
 
 def bench_int4_inverse(dev, steps, warmup, layers, which):
     """INT4 -> bf16 (`which == "int4deq"`) or the QAT quantise-dequantise forward (`"ste"`) over the expert weights
-    of `layers` Qwen3-30B-A3B layers; the 128 experts of a projection are one [128*rows, cols] tensor, one launch
-    each (no grouped form exists for these two)."""
+    of `layers` Qwen3-30B-A3B layers, every expert its own tensor, one launch per step."""
     import torch
 
     import slime_amd
@@ -419,10 +429,15 @@ def bench_int4_inverse(dev, steps, warmup, layers, which):
         def run():
             plan.run()
     else:
+        # every expert its own weight (views of the layer's tensors), all of them through one launch
+        per_expert = []
+        for t in tensors:
+            r = t.shape[0] // 128
+            per_expert += [t[e * r:(e + 1) * r] for e in range(128)]
+        ste_plan = slime_amd.Int4StePlan(per_expert, 128)
+
         def run():
-            for i, t in enumerate(tensors):
-                outs[i] = None          # free the previous output first: the allocator reuses the block
-                outs[i] = slime_amd.fake_int4_quantization_ste(t, 128)
+            outs[0] = ste_plan.run()
 
     wall_ms, ev_ms, ev_min = _time_launches(run, steps, warmup)
     elements = sum((t[2][0] * t[2][1]) if which == "int4deq" else t.numel() for t in tensors)
@@ -435,13 +450,14 @@ def bench_int4_inverse(dev, steps, warmup, layers, which):
             got = torch.cat([plan.outputs[idx * 128 + e] for e in range(-(-1024 // r))])[:1024]
         else:
             want = c_oracle.int4_fake_ste(tensors[idx][:1024].cpu(), 128, 1)
-            got = outs[idx][:1024]
+            r = tensors[idx].shape[0] // 128
+            got = torch.cat([outs[0][idx * 128 + e] for e in range(-(-1024 // r))])[:1024]
         assert torch.equal(got.cpu().view(torch.int16), want.view(torch.int16))
-    launches = 1 if which == "int4deq" else len(tensors)
+    launches = 1
     out = {"workload": f"Qwen3-30B-A3B experts, {layers} layers x (gate, up [128x768,2048], down [128x2048,768]), "
                        + ("INT4 group 128 -> bf16" if which == "int4deq" else "INT4 QAT quantise-dequantise forward")
-                       + (f", {len(tensors) * 128} expert tensors in one launch" if which == "int4deq"
-                          else f", {len(tensors)} launches per step"),
+                       + f", {len(tensors) * 128} expert tensors in one launch"
+,
            "launches": launches, "bf16_GB": 2 * elements / 1e9, "kernel_ms": ev_ms, "wall_ms": wall_ms,
            "bf16_GBps": 2 * elements / ev_ms / 1e6, "algo_GBps": algo_bytes / ev_ms / 1e6,
            "hbm_frac": algo_bytes / ev_ms / 1e6 / HBM_PEAK_GBS, "parity_tensors_checked": 2}
@@ -474,17 +490,26 @@ def bench_delta(dev, steps, warmup):
     assert results[3].tolist() == [changed, int(delta_ref.adler32_ref(check_new), 16)]
     del diffs
 
+    plan = delta.XorDiffPlan(news, olds)             # per-chunk descriptors built once; two launches per run
+
     def run():
-        delta.xor_diff_many(news, olds, update_snapshot=True)
+        plan.run(update_snapshot=True)
 
     wall_ms, ev_ms, ev_min = _time_launches(run, steps, warmup)
+    news[5][:4096] ^= 3                                # the timed form, checked too: a fresh difference in one tensor
+    check_new, check_old = news[5].cpu().numpy(), olds[5].cpu().numpy().copy()
+    diffs, results = plan.run(update_snapshot=True)
+    torch.cuda.synchronize()
+    want, changed = delta_ref.xor_delta_ref(check_new, check_old)
+    assert np.array_equal(diffs[5].cpu().numpy(), want) and np.array_equal(olds[5].cpu().numpy(), check_new)
+    assert results[5].tolist() == [changed, int(delta_ref.adler32_ref(check_new), 16)] and changed == 4096
     nbytes = sum(nw.numel() for nw in news)
     out = {"workload": "Qwen3-4B-shaped state dict (252 bf16 tensors, 7.27 GB) against its snapshot in HBM: xor diff, "
                        "changed-byte count, adler32, snapshot update; two launches for the whole bucket",
            "tensors": len(news), "weight_GB": nbytes / 1e9, "kernel_ms": ev_ms, "wall_ms": wall_ms,
            "weight_GBps": nbytes / ev_ms / 1e6, "algo_GBps": 4 * nbytes / ev_ms / 1e6,
-           "hbm_frac": 4 * nbytes / ev_ms / 1e6 / HBM_PEAK_GBS, "parity_tensors_checked": 1}
-    del news, olds
+           "hbm_frac": 4 * nbytes / ev_ms / 1e6 / HBM_PEAK_GBS, "parity_tensors_checked": 2}
+    del news, olds, plan
     torch.cuda.empty_cache()
     return out
 

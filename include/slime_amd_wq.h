@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define WQ_ABI_VERSION 11
+#define WQ_ABI_VERSION 12
 
 enum {
     WQ_OK = 0,
@@ -162,6 +162,19 @@ typedef struct wq_fp8_dequant_desc {
 int wq_fp8_block_dequant_grouped(const wq_fp8_dequant_desc *descs, const int64_t *work_start, int n_desc,
                                  int64_t total_work, int out_dtype, int block, int mode, void *stream);
 
+/* The grouped form with the owner of every work item resolved beforehand: one descriptor per work item - the tensor
+ * (x, s, y, M, N as in wq_fp8_dequant_desc) and the index of the item inside it.  48 bytes of table per 24 KiB of
+ * traffic; saves the per-workgroup search. */
+typedef struct wq_fp8_dequant_item {
+    const void *x;
+    const float *s;
+    void *y;
+    int64_t M, N;
+    int64_t item;
+} wq_fp8_dequant_item;
+int wq_fp8_block_dequant_items(const wq_fp8_dequant_item *items, int64_t n_items, int out_dtype, int block, int mode,
+                               void *stream);
+
 /* ---------------------------------------------------------------------------------------------
  * "Fake" INT4 quantisation: per (bm x bn) group, q = rintf(x/scale) [+ zero] stored in the input
  * dtype, plus scale and zero point [ceil(M/bm), ceil(N/bn)] in the input dtype.
@@ -218,6 +231,35 @@ int wq_int4_bucket_convert(const wq_int4_pack_desc *items, int64_t n_items, void
 int wq_int4_group_quant_pack_asym(const void *x, int64_t M, int64_t N, int64_t sx_m, int group,
                                   int32_t *packed, void *scale, void *zero, void *stream);
 
+/* wq_int4_group_quant_pack_asym over many contiguous tensors in one launch (the experts of a layer under an asymmetric
+ * compressed-tensors configuration): one descriptor per work item of WQ_INT4_GROUPS_PER_WG groups, pointing at the
+ * item's first group in x (16-byte aligned), packed, scale and zero; n_groups = the groups of the item.  With a
+ * non-NULL out_base (zero_base) the packed and scale (zero) fields are byte offsets from it, and an item with
+ * n_groups < 0 copies -n_groups bytes (at most WQ_BUCKET_COPY_BYTES) from x to out_base + packed: the asymmetric
+ * counterpart of wq_int4_bucket_convert. */
+typedef struct wq_int4_pack_asym_item {
+    const void *x;
+    int32_t *packed;
+    void *scale;     /* bf16 */
+    void *zero;      /* bf16 */
+    int64_t n_groups;
+} wq_int4_pack_asym_item;
+int wq_int4_group_quant_pack_asym_items(const wq_int4_pack_asym_item *items, int64_t n_items, void *out_base,
+                                        void *zero_base, int group, void *stream);
+
+/* The zero points of many tensors packed into the AWQ layout of pack_layer (tools/convert_hf_to_int4_direct.py:134-141)
+ * in one launch: per tensor `zero` bf16 [M, G] as wq_int4_group_quant_pack_asym writes it -> `out` int32 [G, M/8],
+ * word (g, r) = sum over k < 8 of zero[8r + k, g] << 4 * (0,4,1,5,2,6,3,7)[k].  M must be a multiple of 8 (the
+ * reference's reshape fails otherwise).  `descs` DEVICE array, `word_start` DEVICE int64[n_desc + 1] exclusive prefix
+ * sum of G * M / 8.  `zero` / `out` are addresses, or byte offsets from zero_base / out_base when those are non-NULL. */
+typedef struct wq_int4_zp_desc {
+    const void *zero;
+    int32_t *out;
+    int64_t M, G;
+} wq_int4_zp_desc;
+int wq_int4_zero_point_pack_grouped(const wq_int4_zp_desc *descs, const int64_t *word_start, int n_desc,
+                                    int64_t total_words, const void *zero_base, void *out_base, void *stream);
+
 /* INT4 pack-quantized -> bf16: y[i,j] = bf16((nibble(i,j) - 8) * f32(scale[i, j/group])), nibble j of word c at
  * bits [4j,4j+4).  packed int32 [M,N/8], scale bf16 [M,N/group], y bf16 [M,N], all contiguous; N % group == 0,
  * group % 8 == 0.  Replaces _dequantize_tensor, tools/convert_k2_thinking_int4_to_bf16.py:55-84 (whose unpacking
@@ -254,6 +296,18 @@ int wq_int4_dequant_items(const wq_int4_dequant_item *items, int64_t n_items, in
  * (amax * RN(1/7), which is also what fake_int4_quant_cuda.cu:59 computes); x / s is an IEEE division in both. */
 enum { WQ_DIV7_IEEE = 0, WQ_DIV7_DEVICE = 1 };
 int wq_int4_fake_quant_ste(const void *x, void *y, int64_t M, int64_t N, int group, int div7, void *stream);
+
+/* The same forward over many contiguous tensors in one launch (the expert weights of a grouped linear layer, which
+ * the patched forward quantises one by one, docker/patch/latest/megatron.patch:256-279): one descriptor per work item
+ * of WQ_INT4_GROUPS_PER_WG groups, pointing at the item's first group in x and y (16-byte aligned).  With a non-NULL
+ * y_base the y fields are byte offsets from it, so that a table built once serves a fresh output buffer every step. */
+typedef struct wq_int4_ste_item {
+    const void *x;
+    void *y;
+    int64_t n_groups;
+} wq_int4_ste_item;
+int wq_int4_fake_quant_ste_items(const wq_int4_ste_item *items, int64_t n_items, void *y_base, int group, int div7,
+                                 void *stream);
 
 /* ---------------------------------------------------------------------------------------------
  * Byte-level delta of a tensor against its snapshot (delta weight sync).
@@ -309,6 +363,20 @@ typedef struct wq_delta_desc {
 } wq_delta_desc;
 int wq_delta_xor_grouped(const wq_delta_desc *descs, const int64_t *chunk_start, int n_desc,
                          int64_t total_chunks, int write_diff, int update_old, void *stream);
+
+/* wq_delta_xor_grouped with the owner of every chunk resolved beforehand: `items` holds one descriptor per
+ * WQ_DELTA_CHUNK of every tensor (the tensor's buffers and the chunk's index inside it); `descs` is still needed,
+ * per tensor, by the pass that folds the per-chunk sums into `result`. */
+typedef struct wq_delta_chunk_item {
+    const void *new_bytes;
+    void *old_bytes;
+    void *diff;
+    int64_t n;
+    void *workspace;
+    int64_t chunk;
+} wq_delta_chunk_item;
+int wq_delta_xor_items(const wq_delta_chunk_item *items, int64_t n_items, const wq_delta_desc *descs, int n_desc,
+                       int write_diff, int update_old, void *stream);
 
 /* ---------------------------------------------------------------------------------------------
  * Self-checks and calibration helpers (used by the test-suite and the benchmark, not by callers).

@@ -26,9 +26,11 @@ from .fp8 import (
 from .int4 import (
     Int4DequantPlan,
     Int4PackPlan,
+    Int4StePlan,
     dequantize_int4,
     fake_int4_quant_cuda,
     fake_int4_quantization_ste,
+    fake_int4_quantization_ste_many,
     pack_layer,
     pack_to_int32,
     quantize,
@@ -46,7 +48,7 @@ from .processors import (
 quantize_weight = blockwise_cast_to_fp8_triton
 
 __all__ = [
-    "BucketConverter", "FlattenedBucket", "FlattenedTensorMetadata", "quantize_bucket", "quant_weight_ue8m0",
+    "Int4StePlan", "fake_int4_quantization_ste_many", "BucketConverter", "FlattenedBucket", "FlattenedTensorMetadata", "quantize_bucket", "quant_weight_ue8m0",
     "set_ue8m0_requant", "transform_scale_ue8m0",
     "Fp8DequantPlan", "Fp8QuantPlan", "Int4DequantPlan", "Int4PackPlan", "block_fp8", "block_fp8_many",
     "blockwise_cast_to_fp8_triton", "channel_fp8", "dequantize_int4", "fake_int4_quant_cuda",

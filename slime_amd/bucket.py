@@ -28,8 +28,8 @@ import torch
 
 from . import _lib
 from .fp8 import FP8_DTYPE, ceildiv, tile_table
-from .int4 import item_table
-from .processors import _fp8_route, _is_ignored, quantize_params
+from .int4 import item_table, zero_point_rows
+from .processors import _fp8_route, _is_ignored, quantize_params, ue8m0_requant_enabled
 
 _COPY = _lib.BUCKET_COPY_BYTES
 
@@ -54,7 +54,7 @@ class FlattenedBucket:
 
     def __init__(self, flattened_tensor: torch.Tensor, metadata: Sequence[FlattenedTensorMetadata], launches: int = 0):
         self.flattened_tensor = flattened_tensor
-        self.metadata = list(metadata)
+        self.metadata = metadata if isinstance(metadata, list) else list(metadata)     # shared with the cached plan: read-only
         self.launches = launches            # kernel launches this bucket cost (diagnostic)
 
     def get_flattened_tensor(self) -> torch.Tensor:
@@ -84,16 +84,17 @@ def flatten_named_tensors(named_tensors) -> FlattenedBucket:
 
 
 class _Plan:
-    __slots__ = ("kind", "items", "n_items", "total_bytes", "metadata", "keepalive", "late_copies", "group", "block", "device")
+    __slots__ = ("kind", "items", "n_items", "total_bytes", "metadata", "keepalive", "late_copies", "group", "block", "device",
+                 "zero_bytes", "zp_rows", "zp_start", "zp_words", "n_zp")
 
 
 class BucketConverter:
     """Converts buckets of one model under one ``quantization_config``; see the module docstring.
 
-    ``convert(params)`` -> ``FlattenedBucket``.  ``params`` is ``[(megatron_name, [(hf_name, tensor), ...]), ...]`` -
+    ``convert(params)`` -> ``FlattenedBucket``.  ``params`` is a list ``[(megatron_name, [(hf_name, tensor), ...]), ...]`` -
     what ``_convert_to_hf_core`` yields per Megatron parameter.  Tensors the one-launch kernels do not take
-    (FP8: not 2-D bf16 on the GPU; INT4: not contiguous 16-byte aligned bf16 with 32 / 64 / 128 groups, or asymmetric;
-    per-tensor FP8 configurations) go through the per-tensor functions first and are copied in by the same launch, so
+    (FP8: not 2-D bf16 on the GPU; INT4: not contiguous 16-byte aligned bf16 with 32 / 64 / 128 groups; per-tensor FP8
+    configurations) go through the per-tensor functions first and are copied in by the same launch, so
     the result is always what the per-parameter loop gives.
     """
 
@@ -105,6 +106,8 @@ class BucketConverter:
         self._plans: OrderedDict = OrderedDict()
         self._max = int(max_cached_plans)
         self.plan_builds = 0
+        self.time_kernels = False       # when set, convert() brackets its launch with events (kernel_ms())
+        self.kernel_events = []
         method = None if quantization_config is None else quantization_config["quant_method"]
         self._method = method if method in ("fp8", "compressed-tensors") else None
         if self._method == "fp8":
@@ -121,8 +124,6 @@ class BucketConverter:
     def _route(self, megatron_name, converted):
         """-> list of ("quant" | "pass" | "loop", hf_name, tensor, index in `converted`).  "loop": quantised, but by the
         per-tensor function."""
-        from . import processors
-
         if self._method == "fp8":
             route = _fp8_route(megatron_name)
             if route is None:
@@ -132,7 +133,7 @@ class BucketConverter:
                 if route == "skip_scales" and n.endswith("_scale"):
                     continue
                 assert n.endswith(".weight"), f"Expected weight parameter, got {n}"
-                one_launch = (self._block is not None and not processors.ue8m0_requant_enabled() and t.is_cuda
+                one_launch = (self._block is not None and not ue8m0_requant_enabled() and t.is_cuda
                               and t.dim() == 2 and t.dtype == torch.bfloat16 and t.numel() > 0)
                 ops.append(("quant" if one_launch else "loop", n, t, ci))
             return ops
@@ -142,9 +143,9 @@ class BucketConverter:
                 if _is_ignored(n, self._ignore) or not n.endswith(".weight") or t.dim() < 2:
                     ops.append(("pass", n, t, ci))
                     continue
-                one_launch = (self._sym and t.is_cuda and t.dim() == 2 and t.dtype == torch.bfloat16 and t.is_contiguous()
+                one_launch = (t.is_cuda and t.dim() == 2 and t.dtype == torch.bfloat16 and t.is_contiguous()
                               and t.data_ptr() % 16 == 0 and self._group in (32, 64, 128) and t.numel() > 0
-                              and t.shape[1] % self._group == 0)
+                              and t.shape[1] % self._group == 0 and (self._sym or t.shape[0] % 8 == 0))
                 ops.append(("quant" if one_launch else "loop", n, t, ci))
             return ops
         return [("pass", n, t, ci) for ci, (n, t) in enumerate(converted)]
@@ -169,14 +170,15 @@ class BucketConverter:
             raise RuntimeError("BucketConverter: the bucket holds no GPU tensor; there is no CPU path")
         fp8 = self._method != "compressed-tensors"          # pass-through-only buckets use the FP8 launch's copy items
         plan = _Plan()
-        plan.kind = "fp8" if fp8 else "int4"
+        asym = not fp8 and not self._sym
+        plan.kind = "fp8" if fp8 else ("int4_asym" if asym else "int4")
         plan.block = tuple(int(b) for b in self._block) if (self._method == "fp8" and self._block is not None) else (128, 128)
         plan.group = int(self._group) if self._method == "compressed-tensors" else 128
         bm, bn = plan.block
 
         meta, off = [], 0
         quant_rows, copy_rows, late = [], [], []       # table rows per tensor; late = results only known at run time
-        shape_rows = []
+        shape_rows, zp_entries, zero_off = [], [], 0
 
         def place(name, shape, dtype):
             nonlocal off
@@ -216,10 +218,18 @@ class BucketConverter:
                     quant_rows.append((len(meta) - 2, [t.data_ptr(), y0, s0, M, N, t.stride(0), t.stride(1), N]))
                 else:
                     M, N = t.shape
+                    if asym:        # zero points first, as the per-parameter loop emits them
+                        G = N // plan.group
+                        z0, _ = place(n.replace(".weight", ".weight_zero_point"), (G, M // 8), torch.int32)
+                        zp_entries.append((zero_off, z0, M, G))
                     p0, _ = place(n.replace(".weight", ".weight_packed"), (M, N // 8), torch.int32)
                     s0, _ = place(n.replace(".weight", ".weight_scale"), (M, N // plan.group), torch.bfloat16)
                     h0, _ = place(n.replace(".weight", ".weight_shape"), (2,), torch.int32)
-                    quant_rows.append((len(meta) - 3, [t.data_ptr(), p0, s0, M * N // plan.group]))
+                    if asym:
+                        quant_rows.append((len(meta) - 4, [t.data_ptr(), p0, s0, zero_off, M * N // plan.group]))
+                        zero_off += (2 * M * G + 15) // 16 * 16
+                    else:
+                        quant_rows.append((len(meta) - 3, [t.data_ptr(), p0, s0, M * N // plan.group]))
                     shape_rows.append((len(meta) - 1, h0, (M, N)))
 
         plan.keepalive = []
@@ -230,12 +240,19 @@ class BucketConverter:
                 copy_rows.append((mi, shapes.data_ptr() + 8 * k, h0, 8))
 
         # ---- one table row per work item, in bucket order (ordered by the metadata index of the item's first output)
-        width = 8 if fp8 else 4
+        width = 8 if fp8 else (5 if asym else 4)
         blocks, order = [], []
         if quant_rows:
             first = torch.tensor([mi for mi, _ in quant_rows], dtype=torch.int64)
             rows = [r for _, r in quant_rows]
-            table, owner, local = tile_table(rows, bm, bn) if fp8 else item_table(rows, plan.group)
+            if asym:
+                # x, packed, scale and the zero scratch advance with the item; n_groups is what is left of the tensor
+                full = torch.tensor(rows, dtype=torch.int64)
+                table4, owner, local = item_table(full[:, [0, 1, 2, 4]], plan.group)
+                zcol = full[owner, 3] + local * (_lib.INT4_GROUPS_PER_WG * 2)
+                table = torch.cat([table4[:, :3], zcol.unsqueeze(1), table4[:, 3:]], dim=1)
+            else:
+                table, owner, local = tile_table(rows, bm, bn) if fp8 else item_table(rows, plan.group)
             blocks.append(table)
             order.append(first[owner] * (1 << 32) + local)
         if copy_rows:
@@ -250,6 +267,8 @@ class BucketConverter:
             if fp8:
                 blocks.append(torch.stack([d[:, 1] + local * _COPY, d[:, 2] + local * _COPY, zero, nb, zero,
                                            torch.full_like(nb, _lib.BUCKET_COPY_MARK), zero, zero], dim=1))
+            elif asym:
+                blocks.append(torch.stack([d[:, 1] + local * _COPY, d[:, 2] + local * _COPY, zero, zero, -nb], dim=1))
             else:
                 blocks.append(torch.stack([d[:, 1] + local * _COPY, d[:, 2] + local * _COPY, zero, -nb], dim=1))
             order.append(d[:, 0] * (1 << 32) + local)
@@ -261,6 +280,10 @@ class BucketConverter:
             assert table.shape[1] == width
         else:
             plan.items, plan.n_items = None, 0
+        plan.zero_bytes, plan.n_zp = zero_off, len(zp_entries)
+        if zp_entries:
+            zrows, zstart, plan.zp_words = zero_point_rows(zp_entries)
+            plan.zp_rows, plan.zp_start = zrows.to(device), zstart.to(device)
         plan.total_bytes = off
         plan.metadata = meta
         plan.late_copies = late
@@ -276,15 +299,18 @@ class BucketConverter:
         with this id presents the same names, shapes, strides and dtypes; then only the addresses are compared with
         the cached table's (0.2 us per tensor instead of 4 us for the full identity), and a bucket whose tensors
         moved gets a new table."""
-        params = [(mn, list(conv)) for mn, conv in params]
-        if not any(conv for _, conv in params):
-            return flatten_named_tensors([])
         if bucket_id is not None:
-            key = ("id", bucket_id, tuple([t.data_ptr() for _, conv in params for _, t in conv]))
+            key = ("id", bucket_id, tuple([t.data_ptr() for _, conv in params for _, t in conv]), ue8m0_requant_enabled())
+            if not key[2]:
+                return flatten_named_tensors([])
         else:
-            key = (self._key(params), self._config_key, self.transform_ue8m0)
+            params = [(mn, list(conv)) for mn, conv in params]
+            if not any(conv for _, conv in params):
+                return flatten_named_tensors([])
+            key = (self._key(params), self._config_key, self.transform_ue8m0, ue8m0_requant_enabled())
         plan = self._plans.get(key)
         if plan is None:
+            params = [(mn, list(conv)) for mn, conv in params]
             plan = self._build(params)
             self._plans[key] = plan
             while len(self._plans) > self._max:
@@ -300,18 +326,41 @@ class BucketConverter:
         launches = 0
         if plan.n_items:
             lib = _lib.load()
+            if self.time_kernels:
+                ev = (torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+                ev[0].record(torch.cuda.current_stream(device))
             with torch.cuda.device(device):
                 if plan.kind == "fp8":
                     rc = lib.wq_fp8_bucket_convert(plan.items.data_ptr(), plan.n_items, out.data_ptr(), plan.block[0],
                                                    plan.block[1], _lib.FP8_MODE_TRITON, _lib.stream_ptr(device))
+                elif plan.kind == "int4_asym":
+                    # the pack kernel leaves every group's zero point in a scratch buffer; a second launch packs them
+                    # eight rows to a word into their place in the bucket
+                    zero = torch.empty(max(plan.zero_bytes, 16), dtype=torch.uint8, device=device)
+                    rc = lib.wq_int4_group_quant_pack_asym_items(plan.items.data_ptr(), plan.n_items, out.data_ptr(),
+                                                                 zero.data_ptr(), plan.group, _lib.stream_ptr(device))
+                    if rc == 0 and plan.n_zp:
+                        rc = lib.wq_int4_zero_point_pack_grouped(plan.zp_rows.data_ptr(), plan.zp_start.data_ptr(), plan.n_zp,
+                                                                 plan.zp_words, zero.data_ptr(), out.data_ptr(),
+                                                                 _lib.stream_ptr(device))
+                        launches += 1
                 else:
                     rc = lib.wq_int4_bucket_convert(plan.items.data_ptr(), plan.n_items, out.data_ptr(), plan.group,
                                                     _lib.stream_ptr(device))
             _lib.check(rc, "BucketConverter.convert")
-            launches = 1
+            launches += 1
+            if self.time_kernels:
+                ev[1].record(torch.cuda.current_stream(device))
+                self.kernel_events.append(ev)
         if plan.late_copies:
             launches += self._late(plan, params, out)
         return FlattenedBucket(out[:plan.total_bytes], plan.metadata, launches)
+
+    def kernel_ms(self) -> float:
+        """Sum of the launch times recorded while ``time_kernels`` was set (call after a synchronize); clears the list."""
+        total = sum(a.elapsed_time(b) for a, b in self.kernel_events)
+        self.kernel_events = []
+        return total
 
     def _late(self, plan, params, out) -> int:
         """Tensors outside the one-launch kernels: per-tensor functions, then one copy each."""
@@ -319,7 +368,7 @@ class BucketConverter:
         for mi, pi, ci, out_name in plan.late_copies:
             m = plan.metadata[mi]
             mn, conv = params[pi]
-            name, t = conv[ci]
+            name, t = (conv if isinstance(conv, (list, tuple)) else list(conv))[ci]
             if out_name is None:
                 src = t
             else:

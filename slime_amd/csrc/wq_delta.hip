@@ -148,9 +148,12 @@ struct DeltaArgs {
     const wq_delta_desc* descs;      // grouped launch: device arrays
     const int64_t* chunk_start;
     int n_desc;
+    const wq_delta_chunk_item* items;   // per-chunk form
 };
 
-template <bool DIFF, bool UPDATE, bool GROUPED>
+// GROUPED: 0 = one tensor in the kernel arguments, 1 = descriptor array + prefix sums (the owner of a chunk is
+// searched), 2 = one pre-resolved descriptor per chunk
+template <bool DIFF, bool UPDATE, int GROUPED>
 __global__ __launch_bounds__(256) void delta_xor_kernel(const DeltaArgs a, int64_t items)
 {
     __shared__ uint32_t red[16][4];      // per 16-lane row: changed, S, P, Q
@@ -158,10 +161,14 @@ __global__ __launch_bounds__(256) void delta_xor_kernel(const DeltaArgs a, int64
     if (slot >= items) return;
     int64_t item = xcd_chunked_item(slot, items, kDeltaItemsPerXcdRun);
     wq_delta_desc d;
-    if (GROUPED) {
+    if (GROUPED == 1) {
         const int di = find_owner(a.chunk_start, a.n_desc, item, items);
         d = a.descs[di];
         item -= a.chunk_start[di];
+    } else if (GROUPED == 2) {
+        const wq_delta_chunk_item it = a.items[item];
+        d = wq_delta_desc{it.new_bytes, it.old_bytes, it.diff, it.n, it.workspace, nullptr};
+        item = it.chunk;
     } else {
         d = a.d;
     }
@@ -352,7 +359,7 @@ WQ_EXPORT int64_t wq_delta_workspace_bytes(int64_t n)
     return cdiv64(n > 0 ? n : 1, kDeltaChunk) * 32;      // 24 bytes of partials + a 4-byte scan slot, rounded up
 }
 
-template <bool GROUPED>
+template <int GROUPED>
 static void launch_delta_xor(const DeltaArgs& a, int64_t items, bool diff, bool update, hipStream_t st)
 {
     const dim3 g = grid_for_items(items);
@@ -376,7 +383,7 @@ WQ_EXPORT int wq_delta_xor(const void* new_bytes, void* old_bytes, void* diff, i
     DeltaArgs a{};
     a.d = wq_delta_desc{new_bytes, old_bytes, diff, n, workspace, result};
     if (items > 0) {
-        launch_delta_xor<false>(a, items, diff != nullptr, update_old != 0, st);
+        launch_delta_xor<0>(a, items, diff != nullptr, update_old != 0, st);
         WQ_LAUNCH_CHECK();
     }
     delta_fold_kernel<false><<<1, kFoldThreads, 0, st>>>(a);
@@ -439,7 +446,27 @@ WQ_EXPORT int wq_delta_xor_grouped(const wq_delta_desc* descs, const int64_t* ch
     a.chunk_start = chunk_start;
     a.n_desc = n_desc;
     if (total_chunks > 0) {
-        launch_delta_xor<true>(a, total_chunks, write_diff != 0, update_old != 0, st);
+        launch_delta_xor<1>(a, total_chunks, write_diff != 0, update_old != 0, st);
+        WQ_LAUNCH_CHECK();
+    }
+    delta_fold_kernel<true><<<n_desc, kFoldThreads, 0, st>>>(a);
+    WQ_LAUNCH_CHECK();
+    return WQ_OK;
+}
+
+WQ_EXPORT int wq_delta_xor_items(const wq_delta_chunk_item* items, int64_t n_items, const wq_delta_desc* descs, int n_desc,
+                                 int write_diff, int update_old, void* stream)
+{
+    if (n_desc < 0 || n_items < 0) return WQ_ERR_SHAPE;
+    if (n_desc == 0) return WQ_OK;
+    if (!descs || (n_items > 0 && !items)) return WQ_ERR_NULL;
+    hipStream_t st = (hipStream_t)stream;
+    DeltaArgs a{};
+    a.descs = descs;
+    a.n_desc = n_desc;
+    a.items = items;
+    if (n_items > 0) {
+        launch_delta_xor<2>(a, n_items, write_diff != 0, update_old != 0, st);
         WQ_LAUNCH_CHECK();
     }
     delta_fold_kernel<true><<<n_desc, kFoldThreads, 0, st>>>(a);

@@ -33,6 +33,7 @@ struct DeqArgs {
     const int64_t* work_start;
     int32_t n_desc;
     int32_t block;
+    const wq_fp8_dequant_item* items;     // per-item form
 };
 
 // RNE fp32 -> bf16 for two values packed in a dword (v_cvt_pk_bf16_f32).
@@ -69,7 +70,9 @@ __device__ __forceinline__ f32x4 dequant4_f32(uint32_t codes, float sc)
 }
 
 // OUT: WQ_DTYPE_BF16 (the reference tool's default dtype) or WQ_DTYPE_F32 (the un-rounded product).
-template <int MODE, bool GROUPED, int OUT>
+// GROUPED: 0 = one tensor in the kernel arguments, 1 = descriptor array + prefix sums (the owner of a work item is
+// searched), 2 = one pre-resolved descriptor per work item (a single scalar load, no search)
+template <int MODE, int GROUPED, int OUT>
 __global__ __launch_bounds__(256) void fp8_block_dequant_kernel(const DeqArgs a, const int64_t total_work)
 {
     const int64_t slot = (int64_t)blockIdx.x + (int64_t)blockIdx.y * gridDim.x;
@@ -77,10 +80,14 @@ __global__ __launch_bounds__(256) void fp8_block_dequant_kernel(const DeqArgs a,
     const int64_t item = xcd_chunked_item(slot, total_work, kDeqItemsPerXcdRun);
     wq_fp8_dequant_desc d;
     int64_t local = item;
-    if (GROUPED) {
+    if (GROUPED == 1) {
         const int di = find_owner(a.work_start, a.n_desc, item, total_work);
         d = a.descs[di];
         local = item - a.work_start[di];
+    } else if (GROUPED == 2) {
+        const wq_fp8_dequant_item it = a.items[item];
+        d = wq_fp8_dequant_desc{it.x, it.s, it.y, it.M, it.N};
+        local = it.item;
     } else {
         d = a.d;
     }
@@ -165,7 +172,7 @@ static inline int64_t deq_work_items(int64_t M, int64_t N)
 
 using namespace wq;
 
-template <bool GROUPED>
+template <int GROUPED>
 static int launch_deq(const DeqArgs& a, int64_t work, int mode, int out_dtype, hipStream_t st)
 {
     const dim3 g = grid_for_items(work);
@@ -201,7 +208,7 @@ WQ_EXPORT int wq_fp8_block_dequant(const void* x, const float* s, void* y, int o
     DeqArgs a{};
     a.d = wq_fp8_dequant_desc{x, s, y, M, N};
     a.block = block;
-    return launch_deq<false>(a, deq_work_items(M, N), mode, out_dtype, (hipStream_t)stream);
+    return launch_deq<0>(a, deq_work_items(M, N), mode, out_dtype, (hipStream_t)stream);
 }
 
 WQ_EXPORT int wq_fp8_block_dequant_grouped(const wq_fp8_dequant_desc* descs, const int64_t* work_start, int n_desc,
@@ -217,5 +224,19 @@ WQ_EXPORT int wq_fp8_block_dequant_grouped(const wq_fp8_dequant_desc* descs, con
     a.work_start = work_start;
     a.n_desc = n_desc;
     a.block = block;
-    return launch_deq<true>(a, total_work, mode, out_dtype, (hipStream_t)stream);
+    return launch_deq<1>(a, total_work, mode, out_dtype, (hipStream_t)stream);
+}
+
+WQ_EXPORT int wq_fp8_block_dequant_items(const wq_fp8_dequant_item* items, int64_t n_items, int out_dtype, int block,
+                                         int mode, void* stream)
+{
+    if (n_items < 0) return WQ_ERR_SHAPE;
+    int rc = check_deq(block, mode, out_dtype);
+    if (rc) return rc;
+    if (n_items == 0) return WQ_OK;
+    if (!items) return WQ_ERR_NULL;
+    DeqArgs a{};
+    a.items = items;
+    a.block = block;
+    return launch_deq<2>(a, n_items, mode, out_dtype, (hipStream_t)stream);
 }

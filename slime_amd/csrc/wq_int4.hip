@@ -392,12 +392,16 @@ __device__ __forceinline__ uint32_t code_literal_asym(float q, float z, float sb
     return (uint32_t)(int)__builtin_rintf(r);
 }
 
-template <int L>
+// ITEMS: one pre-resolved descriptor per work item (many contiguous tensors in one launch), pointing at the item's
+// first group; rows are then contiguous and groups are addressed flat.
+template <int L, bool ITEMS>
 __global__ __launch_bounds__(256) void int4_pack_asym_kernel(const uint16_t* __restrict__ x, int64_t sx_m,
                                                             int groups_per_row, uint32_t* __restrict__ packed,
                                                             uint16_t* __restrict__ scale_out,
                                                             uint16_t* __restrict__ zero_out, int64_t n_groups,
-                                                            int64_t total_items)
+                                                            int64_t total_items,
+                                                            const wq_int4_pack_asym_item* __restrict__ items,
+                                                            char* out_base, char* zero_base)
 {
     constexpr int CL = 256 / L;
     constexpr int STEPS = kFakeGroupsPerWg / CL;
@@ -405,13 +409,30 @@ __global__ __launch_bounds__(256) void int4_pack_asym_kernel(const uint16_t* __r
     if (slot >= total_items) return;
     const int64_t item = xcd_chunked_item(slot, total_items, kFakeItemsPerXcdRun);
     const int cl = threadIdx.x / L, ll = threadIdx.x % L;
-    const int64_t g0 = item * kFakeGroupsPerWg + cl;
+    int64_t g0 = item * kFakeGroupsPerWg + cl;
+    if (ITEMS) {
+        const wq_int4_pack_asym_item it = items[item];
+        x = (const uint16_t*)it.x;
+        packed = (uint32_t*)(out_base + (uintptr_t)it.packed);        // bases are null for absolute addresses
+        scale_out = (uint16_t*)(out_base + (uintptr_t)it.scale);
+        zero_out = (uint16_t*)(zero_base + (uintptr_t)it.zero);
+        n_groups = it.n_groups;
+        g0 = cl;
+        if (n_groups < 0) {                      // pass-through item: -n_groups bytes from x to packed
+            copy_item(x, packed, (int)-n_groups);
+            return;
+        }
+    }
     u32x4 v[STEPS];
 #pragma unroll
     for (int i = 0; i < STEPS; ++i) {
         const int64_t g = min(g0 + i * CL, n_groups - 1);
-        const int64_t row = g / groups_per_row, gc = g - row * groups_per_row;
-        v[i] = ldg_nt<u32x4>(x + row * sx_m + gc * (8 * L) + ll * 8);
+        if (ITEMS) {
+            v[i] = ldg_nt<u32x4>(x + g * (8 * L) + ll * 8);
+        } else {
+            const int64_t row = g / groups_per_row, gc = g - row * groups_per_row;
+            v[i] = ldg_nt<u32x4>(x + row * sx_m + gc * (8 * L) + ll * 8);
+        }
     }
 #pragma unroll
     for (int i = 0; i < STEPS; ++i) {
@@ -570,9 +591,67 @@ WQ_EXPORT int wq_int4_group_quant_pack_asym(const void* x, int64_t M, int64_t N,
     hipStream_t st = (hipStream_t)stream;
     const uint16_t* xp = (const uint16_t*)x;
     uint32_t* pp = (uint32_t*)packed;
-    if (group == 32) int4_pack_asym_kernel<4><<<g, 256, kFakeOccupancyPadBytes, st>>>(xp, sx_m, gpr, pp, (uint16_t*)scale, (uint16_t*)zero, n_groups, items);
-    else if (group == 64) int4_pack_asym_kernel<8><<<g, 256, kFakeOccupancyPadBytes, st>>>(xp, sx_m, gpr, pp, (uint16_t*)scale, (uint16_t*)zero, n_groups, items);
-    else int4_pack_asym_kernel<16><<<g, 256, kFakeOccupancyPadBytes, st>>>(xp, sx_m, gpr, pp, (uint16_t*)scale, (uint16_t*)zero, n_groups, items);
+    if (group == 32) int4_pack_asym_kernel<4, false><<<g, 256, kFakeOccupancyPadBytes, st>>>(xp, sx_m, gpr, pp, (uint16_t*)scale, (uint16_t*)zero, n_groups, items, nullptr, nullptr, nullptr);
+    else if (group == 64) int4_pack_asym_kernel<8, false><<<g, 256, kFakeOccupancyPadBytes, st>>>(xp, sx_m, gpr, pp, (uint16_t*)scale, (uint16_t*)zero, n_groups, items, nullptr, nullptr, nullptr);
+    else int4_pack_asym_kernel<16, false><<<g, 256, kFakeOccupancyPadBytes, st>>>(xp, sx_m, gpr, pp, (uint16_t*)scale, (uint16_t*)zero, n_groups, items, nullptr, nullptr, nullptr);
+    WQ_LAUNCH_CHECK();
+    return WQ_OK;
+}
+
+WQ_EXPORT int wq_int4_group_quant_pack_asym_items(const wq_int4_pack_asym_item* items, int64_t n_items, void* out_base,
+                                                  void* zero_base, int group, void* stream)
+{
+    if (n_items < 0) return WQ_ERR_SHAPE;
+    if (group != 32 && group != 64 && group != 128) return WQ_ERR_UNSUPPORTED;
+    if (n_items == 0) return WQ_OK;
+    if (!items) return WQ_ERR_NULL;
+    const dim3 g = grid_for_items(n_items);
+    hipStream_t st = (hipStream_t)stream;
+    char* ob = (char*)out_base;
+    char* zb = (char*)zero_base;
+    if (group == 32) int4_pack_asym_kernel<4, true><<<g, 256, kFakeOccupancyPadBytes, st>>>(nullptr, 0, 1, nullptr, nullptr, nullptr, 0, n_items, items, ob, zb);
+    else if (group == 64) int4_pack_asym_kernel<8, true><<<g, 256, kFakeOccupancyPadBytes, st>>>(nullptr, 0, 1, nullptr, nullptr, nullptr, 0, n_items, items, ob, zb);
+    else int4_pack_asym_kernel<16, true><<<g, 256, kFakeOccupancyPadBytes, st>>>(nullptr, 0, 1, nullptr, nullptr, nullptr, 0, n_items, items, ob, zb);
+    WQ_LAUNCH_CHECK();
+    return WQ_OK;
+}
+
+// Zero points of many tensors into the AWQ layout in one launch: zp bf16 [M, G] (integers 0..15) -> int32 [G, M/8],
+// word (g, r) = sum over k < 8 of zp[8r + k, g] << 4 * order[k], order = 0,4,1,5,2,6,3,7.  One lane per word.
+__global__ __launch_bounds__(256) void int4_zero_point_pack_kernel(const wq_int4_zp_desc* __restrict__ descs,
+                                                                  const int64_t* __restrict__ word_start, int n_desc,
+                                                                  int64_t total_words, const char* zero_base, char* out_base)
+{
+    const int64_t w = ((int64_t)blockIdx.x + (int64_t)blockIdx.y * gridDim.x) * 256 + threadIdx.x;
+    if (w >= total_words) return;
+    int lo = 0, hi = n_desc;                       // largest i with word_start[i] <= w
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (word_start[mid] <= w) lo = mid; else hi = mid;
+    }
+    const wq_int4_zp_desc d = descs[lo];
+    const int64_t local = w - word_start[lo];
+    const int64_t words_per_row = d.M / 8;
+    const int64_t g = local / words_per_row, r = local - g * words_per_row;
+    const uint16_t* zp = (const uint16_t*)(zero_base + (uintptr_t)d.zero);
+    uint32_t acc = 0;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        const int order = (k >> 1) + 4 * (k & 1);                       // 0,4,1,5,2,6,3,7
+        const float z = u2f((uint32_t)zp[(r * 8 + k) * d.G + g] << 16);
+        acc += (uint32_t)(int)z << (4 * order);
+    }
+    ((uint32_t*)(out_base + (uintptr_t)d.out))[local] = acc;
+}
+
+WQ_EXPORT int wq_int4_zero_point_pack_grouped(const wq_int4_zp_desc* descs, const int64_t* word_start, int n_desc,
+                                              int64_t total_words, const void* zero_base, void* out_base, void* stream)
+{
+    if (n_desc < 0 || total_words < 0) return WQ_ERR_SHAPE;
+    if (n_desc == 0 || total_words == 0) return WQ_OK;
+    if (!descs || !word_start) return WQ_ERR_NULL;
+    int4_zero_point_pack_kernel<<<grid_for_items(cdiv64(total_words, 256)), 256, 0, (hipStream_t)stream>>>(
+        descs, word_start, n_desc, total_words, (const char*)zero_base, (char*)out_base);
     WQ_LAUNCH_CHECK();
     return WQ_OK;
 }

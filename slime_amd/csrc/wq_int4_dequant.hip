@@ -117,9 +117,11 @@ __device__ __forceinline__ float ste_lanes_max(float v)
     return v;
 }
 
-template <int L>
+// ITEMS: one pre-resolved descriptor per work item (many tensors in one launch), pointing at the item's first group.
+template <int L, bool ITEMS>
 __global__ __launch_bounds__(256) void int4_fake_ste_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ y,
-                                                           int64_t n_groups, int64_t total_items, int div7)
+                                                           int64_t n_groups, int64_t total_items, int div7,
+                                                           const wq_int4_ste_item* __restrict__ items, char* y_base)
 {
     constexpr int CL = 256 / L;
     constexpr int STEPS = kSteGroupsPerWg / CL;
@@ -127,7 +129,14 @@ __global__ __launch_bounds__(256) void int4_fake_ste_kernel(const uint16_t* __re
     if (slot >= total_items) return;
     const int64_t item = xcd_chunked_item(slot, total_items, kSteItemsPerXcdRun);
     const int cl = threadIdx.x / L, ll = threadIdx.x % L;
-    const int64_t g0 = item * kSteGroupsPerWg + cl;
+    int64_t g0 = item * kSteGroupsPerWg + cl;
+    if (ITEMS) {
+        const wq_int4_ste_item it = items[item];
+        x = (const uint16_t*)it.x;
+        y = (uint16_t*)(y_base + (uintptr_t)it.y);       // y_base is null when the items hold addresses
+        n_groups = it.n_groups;
+        g0 = cl;
+    }
     u32x4 v[STEPS];
 #pragma unroll
     for (int i = 0; i < STEPS; ++i) {
@@ -246,9 +255,26 @@ WQ_EXPORT int wq_int4_fake_quant_ste(const void* x, void* y, int64_t M, int64_t 
     const int64_t items = cdiv64(n_groups, kSteGroupsPerWg);
     hipStream_t st = (hipStream_t)stream;
     const dim3 g = grid_for_items(items);
-    if (group == 32) int4_fake_ste_kernel<4><<<g, 256, kSteOccupancyPadBytes, st>>>((const uint16_t*)x, (uint16_t*)y, n_groups, items, div7);
-    else if (group == 64) int4_fake_ste_kernel<8><<<g, 256, kSteOccupancyPadBytes, st>>>((const uint16_t*)x, (uint16_t*)y, n_groups, items, div7);
-    else int4_fake_ste_kernel<16><<<g, 256, kSteOccupancyPadBytes, st>>>((const uint16_t*)x, (uint16_t*)y, n_groups, items, div7);
+    if (group == 32) int4_fake_ste_kernel<4, false><<<g, 256, kSteOccupancyPadBytes, st>>>((const uint16_t*)x, (uint16_t*)y, n_groups, items, div7, nullptr, nullptr);
+    else if (group == 64) int4_fake_ste_kernel<8, false><<<g, 256, kSteOccupancyPadBytes, st>>>((const uint16_t*)x, (uint16_t*)y, n_groups, items, div7, nullptr, nullptr);
+    else int4_fake_ste_kernel<16, false><<<g, 256, kSteOccupancyPadBytes, st>>>((const uint16_t*)x, (uint16_t*)y, n_groups, items, div7, nullptr, nullptr);
+    WQ_LAUNCH_CHECK();
+    return WQ_OK;
+}
+
+WQ_EXPORT int wq_int4_fake_quant_ste_items(const wq_int4_ste_item* items, int64_t n_items, void* y_base, int group, int div7,
+                                           void* stream)
+{
+    if (n_items < 0) return WQ_ERR_SHAPE;
+    if (div7 != WQ_DIV7_IEEE && div7 != WQ_DIV7_DEVICE) return WQ_ERR_MODE;
+    if (group != 32 && group != 64 && group != 128) return WQ_ERR_UNSUPPORTED;
+    if (n_items == 0) return WQ_OK;
+    if (!items) return WQ_ERR_NULL;
+    hipStream_t st = (hipStream_t)stream;
+    const dim3 g = grid_for_items(n_items);
+    if (group == 32) int4_fake_ste_kernel<4, true><<<g, 256, kSteOccupancyPadBytes, st>>>(nullptr, nullptr, 0, n_items, div7, items, (char*)y_base);
+    else if (group == 64) int4_fake_ste_kernel<8, true><<<g, 256, kSteOccupancyPadBytes, st>>>(nullptr, nullptr, 0, n_items, div7, items, (char*)y_base);
+    else int4_fake_ste_kernel<16, true><<<g, 256, kSteOccupancyPadBytes, st>>>(nullptr, nullptr, 0, n_items, div7, items, (char*)y_base);
     WQ_LAUNCH_CHECK();
     return WQ_OK;
 }

@@ -185,50 +185,93 @@ def item_table(rows, group: int):
     return table, owner, local
 
 
+def zero_point_rows(entries):
+    """Descriptor rows and prefix sums for ``wq_int4_zero_point_pack_grouped`` from ``(zero, out, M, G)`` tuples
+    (addresses or byte offsets).  -> (int64 [n, 4], int64 [n + 1], total words)."""
+    rows = torch.tensor([[z, o, M, G] for z, o, M, G in entries], dtype=torch.int64).reshape(-1, 4)
+    words = rows[:, 3] * (rows[:, 2] // 8)
+    start = torch.cat([torch.zeros(1, dtype=torch.int64), torch.cumsum(words, 0)])
+    return rows, start, int(start[-1])
+
+
 class Int4PackPlan:
-    """Symmetric quantise+pack of a fixed list of contiguous bf16 weights with one launch per ``run()``.
+    """Quantise+pack of a fixed list of contiguous bf16 weights with one launch per ``run()`` (symmetric) or two
+    (asymmetric: the pack kernel, then one kernel that packs every tensor's zero points in AWQ order).
 
-    ``outputs`` holds ``(weight_packed int32 [M,N/8], weight_scale bf16 [M,N/group])`` views into the
-    plan's flat buffers, in input order."""
+    ``outputs`` holds ``(weight_packed int32 [M,N/8], weight_scale bf16 [M,N/group])`` - plus
+    ``packed_zero_point int32 [N/group, M/8]`` when ``sym`` is false - views into the plan's flat buffers, in input
+    order: what ``pack_layer(w, group_size, sym)`` returns for each weight."""
 
-    def __init__(self, weights: Sequence[torch.Tensor], group_size: int = 128):
+    def __init__(self, weights: Sequence[torch.Tensor], group_size: int = 128, sym: bool = True):
         if not weights:
             raise ValueError("Int4PackPlan: empty weight list")
         if group_size not in (32, 64, 128):
             raise ValueError("Int4PackPlan: group_size must be 32, 64 or 128")
-        self.group = int(group_size)
+        self.group, self.sym = int(group_size), bool(sym)
         self.device = weights[0].device
         self.weights = list(weights)
-        p_off, s_off, p_total, s_total = [], [], 0, 0
+        p_off, s_off, z_off, p_total, s_total, z_total = [], [], [], 0, 0, 0
         for w in self.weights:
             _check_pack_input(w, self.group, "Int4PackPlan")
             if w.dtype != torch.bfloat16 or not w.is_contiguous() or w.data_ptr() % 16:
                 raise ValueError("Int4PackPlan: weights must be contiguous, 16-byte aligned bfloat16")
             M, N = w.shape
+            if not self.sym and M % 8:
+                # zero points are packed eight ROWS to a word (convert_hf_to_int4_direct.py:134-141); pack_layer itself
+                # takes such a weight through the reference's reshape, whatever that yields or raises
+                raise ValueError(f"Int4PackPlan(sym=False): {M} rows are not a multiple of 8")
             p_off.append(p_total)
             s_off.append(s_total)
+            z_off.append(z_total)
             p_total += (M * N // 8 + 63) // 64 * 64
             s_total += (M * N // self.group + 127) // 128 * 128
+            z_total += ((N // self.group) * (M // 8) + 63) // 64 * 64
         self.flat_packed = torch.empty(max(p_total, 1), dtype=torch.int32, device=self.device)
         self.flat_scale = torch.empty(max(s_total, 1), dtype=torch.bfloat16, device=self.device)
         rows, starts, work = [], [0], 0
         self.outputs = []
-        for w, po, so in zip(self.weights, p_off, s_off):
+        if not self.sym:
+            self._zero = torch.empty(max(s_total, 1), dtype=torch.bfloat16, device=self.device)     # [M, N/group] per tensor
+            self.flat_zp = torch.empty(max(z_total, 1), dtype=torch.int32, device=self.device)
+        zp_entries = []
+        for w, po, so, zo in zip(self.weights, p_off, s_off, z_off):
             M, N = w.shape
             n_groups = M * N // self.group
             packed = self.flat_packed[po:po + M * N // 8].view(M, N // 8)
             scale = self.flat_scale[so:so + n_groups].view(M, N // self.group)
-            self.outputs.append((packed, scale))
-            rows.append([w.data_ptr(), packed.data_ptr(), scale.data_ptr(), n_groups])
+            if self.sym:
+                self.outputs.append((packed, scale))
+                rows.append([w.data_ptr(), packed.data_ptr(), scale.data_ptr(), n_groups])
+            else:
+                G = N // self.group
+                zp = self.flat_zp[zo:zo + G * (M // 8)].view(G, M // 8)
+                zero = self._zero[so:so + n_groups]
+                self.outputs.append((packed, scale, zp))
+                rows.append([w.data_ptr(), packed.data_ptr(), scale.data_ptr(), zero.data_ptr(), n_groups])
+                zp_entries.append((zero.data_ptr(), zp.data_ptr(), M, G))
             work += -(-n_groups // _lib.INT4_GROUPS_PER_WG)
             starts.append(work)
         self.total_work = work
         self.bf16_bytes = sum(2 * w.numel() for w in self.weights)
-        # Many small tensors (the experts of a model): one pre-resolved descriptor per work item (32 bytes per 16 KiB of
-        # weights), so that the kernel needs a single scalar load instead of a search through the per-tensor prefix
-        # sums.  A handful of tensors keeps the search.
         self._items = None
-        if len(rows) >= _ITEM_TABLE_MIN_TENSORS:
+        if not self.sym:
+            # one descriptor per work item: x, packed, scale, zero advance with the item; n_groups is what is left
+            per = _lib.INT4_GROUPS_PER_WG
+            desc = torch.tensor(rows, dtype=torch.int64)
+            start = torch.tensor(starts, dtype=torch.int64)
+            owner = torch.repeat_interleave(torch.arange(len(rows)), start[1:] - start[:-1])
+            local = torch.arange(work, dtype=torch.int64) - start[owner]
+            d = desc[owner]
+            items = torch.stack([d[:, 0] + local * (per * self.group * 2), d[:, 1] + local * (per * self.group // 8 * 4),
+                                 d[:, 2] + local * (per * 2), d[:, 3] + local * (per * 2),
+                                 torch.clamp(d[:, 4] - local * per, max=per)], dim=1)
+            self._items = items.contiguous().to(self.device)
+            zrows, zstart, self._zp_words = zero_point_rows(zp_entries)
+            self._zp_rows, self._zp_start = zrows.to(self.device), zstart.to(self.device)
+        elif len(rows) >= _ITEM_TABLE_MIN_TENSORS:
+            # Many small tensors (the experts of a model): one pre-resolved descriptor per work item (32 bytes per 16 KiB
+            # of weights), so that the kernel needs a single scalar load instead of a search through the per-tensor
+            # prefix sums.  A handful of tensors keeps the search.
             items, _, _ = item_table(rows, self.group)
             self._items = items.contiguous().to(self.device)
         else:
@@ -237,14 +280,18 @@ class Int4PackPlan:
 
     def run(self):
         lib = _lib.load()
+        st = _lib.stream_ptr(self.device)
         with torch.cuda.device(self.device):
-            if self._items is not None:
-                rc = lib.wq_int4_group_quant_pack_items(self._items.data_ptr(), self.total_work, self.group,
-                                                        _lib.stream_ptr(self.device))
+            if not self.sym:
+                rc = lib.wq_int4_group_quant_pack_asym_items(self._items.data_ptr(), self.total_work, None, None, self.group, st)
+                if rc == 0:
+                    rc = lib.wq_int4_zero_point_pack_grouped(self._zp_rows.data_ptr(), self._zp_start.data_ptr(),
+                                                             len(self.weights), self._zp_words, None, None, st)
+            elif self._items is not None:
+                rc = lib.wq_int4_group_quant_pack_items(self._items.data_ptr(), self.total_work, self.group, st)
             else:
                 rc = lib.wq_int4_group_quant_pack_grouped(self._descs.data_ptr(), self._starts.data_ptr(),
-                                                          len(self.weights), self.total_work, self.group,
-                                                          _lib.stream_ptr(self.device))
+                                                          len(self.weights), self.total_work, self.group, st)
         _lib.check(rc, "Int4PackPlan.run")
         return self.outputs
 
@@ -383,3 +430,105 @@ def fake_int4_quantization_ste(x: torch.Tensor, group_size: int) -> torch.Tensor
     if hasattr(x, "main_grad"):
         out.main_grad = x.main_grad
     return out
+
+
+_STE_TABLES: "OrderedDict" = None
+
+
+def _ste_table(xs, group_size):
+    """Per-item table of the one-launch STE forward for these weights (y as offsets into one output buffer), cached on
+    the addresses and shapes of the weights: a layer that calls again with the same parameters builds nothing."""
+    global _STE_TABLES
+    from collections import OrderedDict
+
+    if _STE_TABLES is None:
+        _STE_TABLES = OrderedDict()
+    device = xs[0].device
+    key = (group_size, device.index, tuple((x.data_ptr(), x.shape[0], x.shape[1]) for x in xs))
+    entry = _STE_TABLES.get(key)
+    if entry is not None:
+        _STE_TABLES.move_to_end(key)
+        return entry
+    per = _lib.INT4_GROUPS_PER_WG
+    rows, offs, off = [], [], 0
+    for x in xs:
+        rows.append([x.data_ptr(), off, x.numel() // group_size])
+        offs.append(off // 2)
+        off += (2 * x.numel() + 15) // 16 * 16
+    desc = torch.tensor(rows, dtype=torch.int64)
+    counts = (desc[:, 2] + per - 1) // per
+    owner = torch.repeat_interleave(torch.arange(len(rows)), counts)
+    local = torch.arange(int(counts.sum()), dtype=torch.int64) - (torch.cumsum(counts, 0) - counts)[owner]
+    d = desc[owner]
+    step = per * group_size * 2
+    items = torch.stack([d[:, 0] + local * step, d[:, 1] + local * step, torch.clamp(d[:, 2] - local * per, max=per)], dim=1)
+    entry = (items.contiguous().to(device), items.shape[0], offs, off // 2)
+    _STE_TABLES[key] = entry
+    while len(_STE_TABLES) > 1024:
+        _STE_TABLES.popitem(last=False)
+    return entry
+
+
+class Int4StePlan:
+    """The QAT quantise-dequantise forward over a fixed list of contiguous bf16 weights with one launch per ``run()``;
+    ``outputs`` are views into the plan's flat buffer, in input order (no autograd: the inference-side / benchmark
+    form of ``fake_int4_quantization_ste_many``)."""
+
+    def __init__(self, weights: Sequence[torch.Tensor], group_size: int = 128):
+        if not weights or group_size not in (32, 64, 128):
+            raise ValueError("Int4StePlan: need at least one weight and a group size of 32, 64 or 128")
+        for w in weights:
+            _lib.require_gpu(w, "Int4StePlan")
+            if w.dim() != 2 or w.dtype != torch.bfloat16 or not w.is_contiguous() or w.data_ptr() % 16 or not w.numel() \
+                    or w.shape[1] % group_size:
+                raise ValueError("Int4StePlan: weights must be non-empty contiguous 16-byte aligned bfloat16 matrices "
+                                 "whose rows are whole groups")
+        self.group, self.device, self.weights = int(group_size), weights[0].device, list(weights)
+        self._items, self.n_items, offs, total = _ste_table(self.weights, self.group)
+        self.flat_y = torch.empty(total, dtype=torch.bfloat16, device=self.device)
+        self.outputs = [self.flat_y[o:o + w.numel()].view(w.shape) for o, w in zip(offs, self.weights)]
+        self.bf16_bytes = sum(2 * w.numel() for w in self.weights)
+
+    def run(self):
+        with torch.cuda.device(self.device):
+            rc = _lib.load().wq_int4_fake_quant_ste_items(self._items.data_ptr(), self.n_items, self.flat_y.data_ptr(),
+                                                          self.group, arith.div7_rule(), _lib.stream_ptr(self.device))
+        _lib.check(rc, "Int4StePlan.run")
+        return self.outputs
+
+
+class _FakeInt4QuantizationSTEMany(torch.autograd.Function):
+    """The same forward for a list of weights in ONE launch (identity backward per weight): the expert weights of a
+    grouped linear layer, which the patched forward quantises one after the other (megatron.patch:256-279)."""
+
+    @staticmethod
+    def forward(ctx, group_size, *xs):
+        device = xs[0].device
+        items, n_items, offs, total = _ste_table(xs, group_size)
+        flat = torch.empty(total, dtype=torch.bfloat16, device=device)
+        with torch.cuda.device(device):
+            rc = _lib.load().wq_int4_fake_quant_ste_items(items.data_ptr(), n_items, flat.data_ptr(), int(group_size),
+                                                          arith.div7_rule(), _lib.stream_ptr(device))
+        _lib.check(rc, "fake_int4_quantization_ste_many")
+        return tuple(flat[o:o + x.numel()].view(x.shape) for o, x in zip(offs, xs))
+
+    @staticmethod
+    def backward(ctx, *grads):
+        return (None,) + tuple(grads)
+
+
+def fake_int4_quantization_ste_many(xs: Sequence[torch.Tensor], group_size: int):
+    """``[fake_int4_quantization_ste(x, group_size) for x in xs]`` with one kernel launch when every weight is a
+    contiguous, 16-byte aligned bf16 matrix whose rows are whole groups of 32 / 64 / 128; otherwise one call per
+    weight.  Outputs are slices of one fresh allocation."""
+    xs = list(xs)
+    fast = xs and group_size in (32, 64, 128) and all(
+        x.is_cuda and x.dim() == 2 and x.dtype == torch.bfloat16 and x.is_contiguous() and x.data_ptr() % 16 == 0
+        and x.numel() and x.shape[1] % group_size == 0 and x.device == xs[0].device for x in xs)
+    if not fast:
+        return [fake_int4_quantization_ste(x, group_size) for x in xs]
+    outs = list(_FakeInt4QuantizationSTEMany.apply(group_size, *xs))
+    for x, o in zip(xs, outs):
+        if hasattr(x, "main_grad"):
+            o.main_grad = x.main_grad
+    return outs

@@ -161,7 +161,24 @@ def test_int4_bucket_asymmetric_and_other_groups(cuda):
     g256 = {**INT4_CFG, "config_groups": {"group_0": {"weights": {"group_size": 256, "symmetric": True}}}, "ignore": []}
     everything = {**INT4_CFG, "ignore": []}       # nothing ignored: the fp32 router goes through the per-tensor path
     for cfg in (asym, g32, everything):
-        _same_as_loop(B.BucketConverter(None, cfg).convert(params), B.per_param_loop(None, params, cfg))
+        conv = B.BucketConverter(None, cfg)
+        for _ in range(2):
+            out = conv.convert(params)
+            _same_as_loop(out, B.per_param_loop(None, params, cfg))
+        assert conv.plan_builds == 1
+        if cfg is asym:
+            assert out.launches == 2        # the pack kernel (with the pass-through copies) + the zero-point packer
+            assert [m.name.rsplit(".", 1)[1] for m in out.metadata if ".experts.0.gate_proj" in m.name] == [
+                "weight_zero_point", "weight_packed", "weight_scale", "weight_shape"]
+    # rows that are not a multiple of 8 under an asymmetric configuration go through the per-tensor path, with whatever
+    # the reference's zeros.reshape(-1, M // 8, 8) makes of them: a [3, 1] tensor for 12 x 256, an error for 12 x 128
+    odd = [(L.format(0) + "mlp.experts.linear_fc2.weight0", [("model.layers.0.mlp.experts.0.down_proj.weight", I.weights(12, 256, seed=3).to(cuda))])]
+    _same_as_loop(B.BucketConverter(None, asym).convert(odd), B.per_param_loop(None, odd, asym))
+    bad = [(L.format(0) + "mlp.experts.linear_fc2.weight0", [("model.layers.0.mlp.experts.0.down_proj.weight", I.weights(12, 128, seed=3).to(cuda))])]
+    with pytest.raises(RuntimeError, match="invalid for input of size"):
+        B.per_param_loop(None, bad, asym)
+    with pytest.raises(RuntimeError, match="invalid for input of size"):
+        B.BucketConverter(None, asym).convert(bad)
     one = [(L.format(0) + "mlp.experts.linear_fc2.weight0", [("model.layers.0.mlp.experts.0.down_proj.weight", I.weights(64, 512, seed=3).to(cuda))])]
     _same_as_loop(B.BucketConverter(None, g256).convert(one), B.per_param_loop(None, one, g256))
 
