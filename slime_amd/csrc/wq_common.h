@@ -185,22 +185,49 @@ __device__ __forceinline__ uint32_t row16_max_u32(uint32_t v)
     v = max(v, dpp_u32<0x140>(v));  // row_mirror
     return v;
 }
-__device__ __forceinline__ float row16_max_f32(float v)
+// fp32 max / min with the DPP-permuted copy of the same register in ONE instruction (v_max_f32_dpp).  Written as
+// inline assembly because the compiler, from fmaxf(v, dpp(v)), emits four (copy, DPP move, canonicalise, max) - and the
+// group-wise INT4 kernels, which run these reductions once per 8 elements, are bound by VALU issue.  A quiet NaN operand
+// is dropped, as fmaxf / fminf do; a signalling NaN (which no torch operation produces) becomes a quiet NaN result.
+// `s_nop 1`: a DPP read needs two wait states after the VALU write of its source.
+#define WQ_DPP_F32_OP(NAME, OP, CTRL)                                                                        \
+    __device__ __forceinline__ float NAME(float v)                                                           \
+    {                                                                                                        \
+        float r;                                                                                             \
+        asm("s_nop 1\n\t" OP " %0, %1, %1 " CTRL " row_mask:0xf bank_mask:0xf" : "=v"(r) : "v"(v));          \
+        return r;                                                                                            \
+    }
+WQ_DPP_F32_OP(max_f32_quad_1032, "v_max_f32_dpp", "quad_perm:[1,0,3,2]")
+WQ_DPP_F32_OP(max_f32_quad_2301, "v_max_f32_dpp", "quad_perm:[2,3,0,1]")
+WQ_DPP_F32_OP(max_f32_half_mirror, "v_max_f32_dpp", "row_half_mirror")
+WQ_DPP_F32_OP(max_f32_mirror, "v_max_f32_dpp", "row_mirror")
+WQ_DPP_F32_OP(min_f32_quad_1032, "v_min_f32_dpp", "quad_perm:[1,0,3,2]")
+WQ_DPP_F32_OP(min_f32_quad_2301, "v_min_f32_dpp", "quad_perm:[2,3,0,1]")
+WQ_DPP_F32_OP(min_f32_half_mirror, "v_min_f32_dpp", "row_half_mirror")
+WQ_DPP_F32_OP(min_f32_mirror, "v_min_f32_dpp", "row_mirror")
+#undef WQ_DPP_F32_OP
+
+// all-reduce over L = 4, 8 or 16 adjacent lanes (L = 16: a DPP row)
+template <int L>
+__device__ __forceinline__ float lanes_max_f32(float v)
 {
-    v = fmaxf(v, u2f(dpp_u32<0xB1>(f2u(v))));
-    v = fmaxf(v, u2f(dpp_u32<0x4E>(f2u(v))));
-    v = fmaxf(v, u2f(dpp_u32<0x141>(f2u(v))));
-    v = fmaxf(v, u2f(dpp_u32<0x140>(f2u(v))));
+    v = max_f32_quad_1032(v);
+    v = max_f32_quad_2301(v);
+    if (L >= 8) v = max_f32_half_mirror(v);
+    if (L >= 16) v = max_f32_mirror(v);
     return v;
 }
-__device__ __forceinline__ float row16_min_f32(float v)
+template <int L>
+__device__ __forceinline__ float lanes_min_f32(float v)
 {
-    v = fminf(v, u2f(dpp_u32<0xB1>(f2u(v))));
-    v = fminf(v, u2f(dpp_u32<0x4E>(f2u(v))));
-    v = fminf(v, u2f(dpp_u32<0x141>(f2u(v))));
-    v = fminf(v, u2f(dpp_u32<0x140>(f2u(v))));
+    v = min_f32_quad_1032(v);
+    v = min_f32_quad_2301(v);
+    if (L >= 8) v = min_f32_half_mirror(v);
+    if (L >= 16) v = min_f32_mirror(v);
     return v;
 }
+__device__ __forceinline__ float row16_max_f32(float v) { return lanes_max_f32<16>(v); }
+__device__ __forceinline__ float row16_min_f32(float v) { return lanes_min_f32<16>(v); }
 // NaN-propagating fp32 maximum over the wavefront
 __device__ __forceinline__ float wave64_max_nanprop_f32(float v)
 {
@@ -373,6 +400,36 @@ __device__ __forceinline__ float rcp_refined(float s)
 {
     const float r0 = __builtin_amdgcn_rcpf(s);
     return __builtin_fmaf(__builtin_fmaf(-s, r0, 1.0f), r0, r0);
+}
+
+// acc's byte BYTE <- low byte of (q + magic): v_add_f32_sdwa with the other bytes of the destination preserved.
+#define WQ_ADD_TO_BYTE(BYTE)                                                                                        \
+    __device__ __forceinline__ void add_magic_to_byte##BYTE(uint32_t& acc, float q, float magic)                    \
+    {                                                                                                               \
+        asm("v_add_f32_sdwa %0, %1, %2 dst_sel:BYTE_" #BYTE " dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD" \
+            : "+v"(acc) : "v"(q), "v"(magic));                                                                      \
+    }
+WQ_ADD_TO_BYTE(1)
+WQ_ADD_TO_BYTE(2)
+WQ_ADD_TO_BYTE(3)
+#undef WQ_ADD_TO_BYTE
+
+// Eight exact quotients -> one packed word, 9 instructions after the divisions: for |rintf(q)| <= 7 the low BYTE of
+// bits(q + kRoundMagic) is rintf(q) + 8 (its upper nibble is zero), so the even elements are gathered as the four
+// bytes of one register and the odd ones of another - each add writing its byte straight into place - and
+// even | odd << 4 is the word sum_j (q_j + 8) << 4j.
+__device__ __forceinline__ uint32_t pack8_sym_bytes(const float (&x)[8], float scale, float rcp)
+{
+    const float magic = kRoundMagic;
+    uint32_t even = f2u(div_by_scale(x[0], scale, rcp) + magic);      // byte 0; bytes 1-3 are overwritten below
+    uint32_t odd = f2u(div_by_scale(x[1], scale, rcp) + magic);
+    add_magic_to_byte1(even, div_by_scale(x[2], scale, rcp), magic);
+    add_magic_to_byte1(odd, div_by_scale(x[3], scale, rcp), magic);
+    add_magic_to_byte2(even, div_by_scale(x[4], scale, rcp), magic);
+    add_magic_to_byte2(odd, div_by_scale(x[5], scale, rcp), magic);
+    add_magic_to_byte3(even, div_by_scale(x[6], scale, rcp), magic);
+    add_magic_to_byte3(odd, div_by_scale(x[7], scale, rcp), magic);
+    return (odd << 4) | even;
 }
 
 // Eight exact quotients -> one packed word.  For |rintf(q)| <= 7 the float q + kRoundMagic has the bit

@@ -72,11 +72,20 @@ __device__ __forceinline__ void quant_tile_vec128(const wq_fp8_quant_desc& d, in
 #pragma unroll
         for (int i = 0; i < kTileLoads; ++i) v[i] = ldg_nt<u32x4>(xt + (xoff + i * xstep));
     } else {
+        // Edge tile: every lane loads from a valid address - its row and piece clamped into the tile - and the lanes
+        // outside the tensor are zeroed afterwards.  (Loads predicated per lane make the compiler wait for the earlier
+        // ones before it issues the next; this way all eight are in flight together, as in a full tile.)
+        const int rows = (int)min((int64_t)128, d.M - tm * 128);
+        const int pieces = (int)min((int64_t)16, (d.N - tn * 128) >> 3);
+        const uint32_t coff = (uint32_t)min(cc, pieces - 1) * 16u;
 #pragma unroll
         for (int i = 0; i < kTileLoads; ++i) {
-            v[i] = (u32x4){0u, 0u, 0u, 0u};
-            if (col_ok && kRowSlots * i < rows_left) v[i] = ldg_nt<u32x4>(xt + (xoff + i * xstep));
+            const uint32_t r = (uint32_t)min(rb + kRowSlots * i, rows - 1);
+            v[i] = ldg_nt<u32x4>(xt + (r * (uint32_t)d.sx_m * 2u + coff));
         }
+#pragma unroll
+        for (int i = 0; i < kTileLoads; ++i)
+            if (!(col_ok && kRowSlots * i < rows_left)) v[i] = (u32x4){0u, 0u, 0u, 0u};
     }
 
     uint32_t m = 0;

@@ -56,16 +56,6 @@ __device__ __forceinline__ float absmax8(const float (&x)[8])
     return m;
 }
 
-template <int L>
-__device__ __forceinline__ float lanes_max_f32(float v)
-{
-    v = fmaxf(v, u2f(dpp_u32<0xB1>(f2u(v))));
-    v = fmaxf(v, u2f(dpp_u32<0x4E>(f2u(v))));
-    if (L >= 8) v = fmaxf(v, u2f(dpp_u32<0x141>(f2u(v))));
-    if (L >= 16) v = fmaxf(v, u2f(dpp_u32<0x140>(f2u(v))));
-    return v;
-}
-
 typedef float f32x2_t __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 // fp32 -> bf16 bits, RNE, by v_cvt_pk_bf16_f32 (identical to the software rounding for all non-NaN inputs)
@@ -134,18 +124,23 @@ __global__ __launch_bounds__(256) void int4_pack_kernel(const Int4PackArgs a, co
         d = a.d;
     }
     const int cl = threadIdx.x / L, ll = threadIdx.x % L;
-    const int64_t g0 = local * kGroupsPerWg + cl;
-    const uint16_t* x = (const uint16_t*)d.x;
+    // Workgroup-uniform base of the item (scalar registers) and 32-bit per-lane byte offsets from it: an item is at
+    // most 64 groups = 16 KiB of input.
+    const int64_t base = local * kGroupsPerWg;
+    const int rem = (int)min((int64_t)kGroupsPerWg, d.n_groups - base);       // groups of the item, >= 1
+    const char* xb = (const char*)d.x + base * (16 * L);
+    char* pb = (char*)d.packed + base * (4 * L);
+    char* sb = (char*)d.scale + base * 2;
 
     // Rolling window: at most kPackWindow 16-byte loads per lane are in flight; the load of step i + window
     // is issued just before step i is processed.  More bytes in flight per CU than that lower the achieved
     // HBM bandwidth on this part, while a long work item amortises the per-workgroup start-up.
-    // Out-of-range groups re-read the tensor's last group instead of branching around the load (a
+    // Out-of-range groups re-read the item's last group instead of branching around the load (a
     // predicated load makes the compiler wait for earlier loads before issuing the next one).
     u32x4 v[STEPS];
     auto issue = [&](int i) {
-        const int64_t g = min(g0 + i * CL, d.n_groups - 1);
-        v[i] = ldg_nt<u32x4>(x + g * (8 * L) + ll * 8);
+        const int g = min(cl + i * CL, rem - 1);
+        v[i] = ldg_nt<u32x4>(xb + (uint32_t)(g * (16 * L) + ll * 16));
     };
 #pragma unroll
     for (int i = 0; i < kPackWindow && i < STEPS; ++i) issue(i);
@@ -153,16 +148,16 @@ __global__ __launch_bounds__(256) void int4_pack_kernel(const Int4PackArgs a, co
     for (int i = 0; i < STEPS; ++i) {
         if (i + kPackWindow < STEPS) issue(i + kPackWindow);
         __builtin_amdgcn_sched_barrier(0);
-        const int64_t g = g0 + i * CL;
+        const int g = cl + i * CL;
         float xs[8];
         unpack8(v[i], xs);
         const float scale = int4_scale_sym(lanes_max_f32<L>(absmax8(xs)));
-        uint32_t w = pack8_sym(xs, scale, rcp_refined(scale));
+        uint32_t w = pack8_sym_bytes(xs, scale, rcp_refined(scale));
         const uint32_t sb_bits = bf16_bits_hw(scale);
         if (sb_bits >= kLiteralChainScaleBits) w = pack8_literal(xs, scale, u2f(sb_bits << 16));
-        if (g < d.n_groups) {
-            stg_nt<uint32_t>((uint32_t*)d.packed + g * L + ll, w);
-            if (ll == 0) stg<uint16_t>((uint16_t*)d.scale + g, (uint16_t)sb_bits);
+        if (g < rem) {
+            stg_nt<uint32_t>(pb + (uint32_t)((g * L + ll) * 4), w);
+            if (ll == 0) stg<uint16_t>(sb + (uint32_t)(g * 2), (uint16_t)sb_bits);
         }
         __builtin_amdgcn_sched_barrier(0);
     }
@@ -284,16 +279,6 @@ __global__ __launch_bounds__(256) void int4_fake_quant_kernel(const T* __restric
 constexpr int kFakeGroupsPerWg = 64;
 constexpr int kFakeItemsPerXcdRun = 32;
 constexpr unsigned kFakeOccupancyPadBytes = 36 * 1024;
-
-template <int L>
-__device__ __forceinline__ float lanes_min_f32(float v)
-{
-    v = fminf(v, u2f(dpp_u32<0xB1>(f2u(v))));
-    v = fminf(v, u2f(dpp_u32<0x4E>(f2u(v))));
-    if (L >= 8) v = fminf(v, u2f(dpp_u32<0x141>(f2u(v))));
-    if (L >= 16) v = fminf(v, u2f(dpp_u32<0x140>(f2u(v))));
-    return v;
-}
 
 __device__ __forceinline__ uint32_t pack2_bf16_hw(float a, float b)
 {

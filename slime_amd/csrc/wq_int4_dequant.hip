@@ -107,16 +107,6 @@ constexpr int kSteGroupsPerWg = 64;
 constexpr int kSteItemsPerXcdRun = 32;
 constexpr int kSteOccupancyPadBytes = 36 * 1024;
 
-template <int L>
-__device__ __forceinline__ float ste_lanes_max(float v)
-{
-    v = fmaxf(v, u2f(dpp_u32<0xB1>(f2u(v))));
-    v = fmaxf(v, u2f(dpp_u32<0x4E>(f2u(v))));
-    if (L >= 8) v = fmaxf(v, u2f(dpp_u32<0x141>(f2u(v))));
-    if (L >= 16) v = fmaxf(v, u2f(dpp_u32<0x140>(f2u(v))));
-    return v;
-}
-
 // ITEMS: one pre-resolved descriptor per work item (many tensors in one launch), pointing at the item's first group.
 template <int L, bool ITEMS>
 __global__ __launch_bounds__(256) void int4_fake_ste_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ y,

@@ -67,8 +67,9 @@ __global__ __launch_bounds__(256) void selftest_int4_elem_kernel(uint32_t amax_l
         range_ok = range_ok && qi >= -7 && qi <= 7;
         want |= ((uint32_t)(qi + 8) & 0xFu) << (4 * j);
     }
-    const uint32_t got = pack8_sym(x, scale, rcp);
-    if (got != want || !range_ok) report(out, ((uint64_t)a << 16) | x0);
+    // both packers: the byte-gathering one the pack kernel uses and the shift-add one
+    const uint32_t got = pack8_sym_bytes(x, scale, rcp);
+    if (got != want || pack8_sym(x, scale, rcp) != want || !range_ok) report(out, ((uint64_t)a << 16) | x0);
 }
 
 // hardware fp32 -> e4m3fn vs software, both word positions of the packed conversion
