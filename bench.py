@@ -188,7 +188,7 @@ def bench_fp8_quant(dev, steps, warmup):
         q, s = plan.outputs[idx]
         qo, so = c_oracle.fp8_block_quant(weights[idx].cpu(), (128, 128), plan.mode)
         assert torch.equal(q.cpu().view(torch.uint8), qo) and torch.equal(s.cpu().view(torch.int32), so.view(torch.int32))
-    traffic, note = _traffic_from_profile("fp8_block_quant_qwen3_4b_pmc.txt", "fp8_block_quant")
+    traffic, note = _traffic_from_profile("fp8_block_quant_qwen3_4b.txt", "fp8_block_quant")
     out = {"workload": "Qwen3-4B-shaped bf16 state dict, block-FP8 128x128 quant of all 252 linear weights (36 layers x "
                        "q,k,v,o,gate,up,down), one grouped launch, block_fp8 arithmetic as torch evaluates it on GPU tensors",
            "tensors": len(weights), "bf16_GB": 2 * elements / 1e9, "kernel_ms": ev_ms, "kernel_ms_min": ev_min,

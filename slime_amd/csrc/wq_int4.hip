@@ -286,7 +286,9 @@ __device__ __forceinline__ uint32_t pack2_bf16_hw(float a, float b)
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
 }
 
-template <int L, bool SYM>
+// CONTIG: rows are back to back (row stride = row length), so a group's address is its flat index times the group
+// size; otherwise (row, group-in-row) come from a 32-bit division - the host checks that the group count fits.
+template <int L, bool SYM, bool CONTIG>
 __global__ __launch_bounds__(256) void int4_fake_quant_vec_kernel(const uint16_t* __restrict__ x, int64_t sx_m,
                                                                  int groups_per_row, uint16_t* __restrict__ q,
                                                                  uint16_t* __restrict__ scale_out,
@@ -304,8 +306,12 @@ __global__ __launch_bounds__(256) void int4_fake_quant_vec_kernel(const uint16_t
 #pragma unroll
     for (int i = 0; i < STEPS; ++i) {
         const int64_t g = min(g0 + i * CL, n_groups - 1);
-        const int64_t row = g / groups_per_row, gc = g - row * groups_per_row;
-        v[i] = ldg_nt<u32x4>(x + row * sx_m + gc * (8 * L) + ll * 8);
+        if (CONTIG) {
+            v[i] = ldg_nt<u32x4>(x + g * (8 * L) + ll * 8);
+        } else {
+            const uint32_t row = (uint32_t)g / (uint32_t)groups_per_row, gc = (uint32_t)g - row * (uint32_t)groups_per_row;
+            v[i] = ldg_nt<u32x4>(x + (int64_t)row * sx_m + gc * (8 * L) + ll * 8);
+        }
     }
 #pragma unroll
     for (int i = 0; i < STEPS; ++i) {
@@ -333,16 +339,18 @@ __global__ __launch_bounds__(256) void int4_fake_quant_vec_kernel(const uint16_t
             vmax = lanes_max_f32<L>(vmax);
             vmin = lanes_min_f32<L>(vmin);
             scale = fmaxf((vmax - vmin) * (1.0f / 15.0f), 1e-5f);
-            zero = fminf(fmaxf(-__builtin_rintf(vmin / scale), 0.0f), 15.0f) + 0.0f;
             // x / scale by the correctly rounded reciprocal (one division per lane) and the two-FMA correction, which
             // yields the correctly rounded quotient for any fp32 divisor as long as the reciprocal is a normal number and
             // nothing overflows (Markstein's theorem); groups holding huge or non-finite values divide element by element.
+            // The zero point's min / scale is one more such quotient.
             const float r = 1.0f / scale;
             const bool safe = scale < 0x1p100f && fmaxf(fabsf(vmax), fabsf(vmin)) * r < 0x1p60f;
             if (__builtin_amdgcn_ballot_w64(!safe) == 0) {
+                zero = fminf(fmaxf(-__builtin_rintf(div_by_scale(vmin, scale, r)), 0.0f), 15.0f) + 0.0f;
 #pragma unroll
                 for (int j = 0; j < 8; ++j) o[j] = __builtin_rintf(div_by_scale(xs[j], scale, r)) + zero;
             } else {
+                zero = fminf(fmaxf(-__builtin_rintf(vmin / scale), 0.0f), 15.0f) + 0.0f;
 #pragma unroll
                 for (int j = 0; j < 8; ++j) o[j] = __builtin_rintf(xs[j] / scale) + zero;
             }
@@ -414,9 +422,11 @@ __global__ __launch_bounds__(256) void int4_pack_asym_kernel(const uint16_t* __r
         const int64_t g = min(g0 + i * CL, n_groups - 1);
         if (ITEMS) {
             v[i] = ldg_nt<u32x4>(x + g * (8 * L) + ll * 8);
+        } else if (sx_m == (int64_t)groups_per_row * (8 * L)) {     // contiguous rows (uniform branch)
+            v[i] = ldg_nt<u32x4>(x + g * (8 * L) + ll * 8);
         } else {
-            const int64_t row = g / groups_per_row, gc = g - row * groups_per_row;
-            v[i] = ldg_nt<u32x4>(x + row * sx_m + gc * (8 * L) + ll * 8);
+            const uint32_t row = (uint32_t)g / (uint32_t)groups_per_row, gc = (uint32_t)g - row * (uint32_t)groups_per_row;
+            v[i] = ldg_nt<u32x4>(x + (int64_t)row * sx_m + gc * (8 * L) + ll * 8);
         }
     }
 #pragma unroll
@@ -429,16 +439,18 @@ __global__ __launch_bounds__(256) void int4_pack_asym_kernel(const uint16_t* __r
         vmax = lanes_max_f32<L>(vmax);
         vmin = lanes_min_f32<L>(vmin);
         const float scale = fmaxf((vmax - vmin) * (1.0f / 15.0f), 1e-5f);
-        const float zero = fminf(fmaxf(-__builtin_rintf(vmin / scale), 0.0f), 15.0f) + 0.0f;
         const uint32_t sb_bits = f32_to_bf16_bits(scale);
-        float q[8];
-        // x / scale by the correctly rounded reciprocal and the two-FMA correction (see int4_fake_quant_vec_kernel)
+        float q[8], zero;
+        // x / scale (and min / scale of the zero point) by the correctly rounded reciprocal and the two-FMA correction
+        // (see int4_fake_quant_vec_kernel)
         const float r = 1.0f / scale;
         const bool safe = scale < 0x1p100f && fmaxf(fabsf(vmax), fabsf(vmin)) * r < 0x1p60f;
         if (__builtin_amdgcn_ballot_w64(!safe) == 0) {
+            zero = fminf(fmaxf(-__builtin_rintf(div_by_scale(vmin, scale, r)), 0.0f), 15.0f) + 0.0f;
 #pragma unroll
             for (int j = 0; j < 8; ++j) q[j] = __builtin_rintf(div_by_scale(xs[j], scale, r)) + zero;
         } else {
+            zero = fminf(fmaxf(-__builtin_rintf(vmin / scale), 0.0f), 15.0f) + 0.0f;
 #pragma unroll
             for (int j = 0; j < 8; ++j) q[j] = __builtin_rintf(xs[j] / scale) + zero;
         }
@@ -472,9 +484,15 @@ static bool launch_fake_vec(const uint16_t* x, int64_t M, int64_t N, int64_t sx_
     const int64_t items = cdiv64(n_groups, kFakeGroupsPerWg);
     const dim3 g = grid_for_items(items);
     const int gpr = (int)(N / bn);
-    if (bn == 32) int4_fake_quant_vec_kernel<4, SYM><<<g, 256, kFakeOccupancyPadBytes, st>>>(x, sx_m, gpr, q, sc, zp, n_groups, items);
-    else if (bn == 64) int4_fake_quant_vec_kernel<8, SYM><<<g, 256, kFakeOccupancyPadBytes, st>>>(x, sx_m, gpr, q, sc, zp, n_groups, items);
-    else int4_fake_quant_vec_kernel<16, SYM><<<g, 256, kFakeOccupancyPadBytes, st>>>(x, sx_m, gpr, q, sc, zp, n_groups, items);
+    if (sx_m == N) {
+        if (bn == 32) int4_fake_quant_vec_kernel<4, SYM, true><<<g, 256, kFakeOccupancyPadBytes, st>>>(x, sx_m, gpr, q, sc, zp, n_groups, items);
+        else if (bn == 64) int4_fake_quant_vec_kernel<8, SYM, true><<<g, 256, kFakeOccupancyPadBytes, st>>>(x, sx_m, gpr, q, sc, zp, n_groups, items);
+        else int4_fake_quant_vec_kernel<16, SYM, true><<<g, 256, kFakeOccupancyPadBytes, st>>>(x, sx_m, gpr, q, sc, zp, n_groups, items);
+    } else {
+        if (bn == 32) int4_fake_quant_vec_kernel<4, SYM, false><<<g, 256, kFakeOccupancyPadBytes, st>>>(x, sx_m, gpr, q, sc, zp, n_groups, items);
+        else if (bn == 64) int4_fake_quant_vec_kernel<8, SYM, false><<<g, 256, kFakeOccupancyPadBytes, st>>>(x, sx_m, gpr, q, sc, zp, n_groups, items);
+        else int4_fake_quant_vec_kernel<16, SYM, false><<<g, 256, kFakeOccupancyPadBytes, st>>>(x, sx_m, gpr, q, sc, zp, n_groups, items);
+    }
     return true;
 }
 
@@ -542,7 +560,8 @@ WQ_EXPORT int wq_int4_fake_quant(const void* x, int dtype, int64_t M, int64_t N,
     const int64_t groups = cdiv64(M, bm) * cdiv64(N, bn);
     hipStream_t st = (hipStream_t)stream;
     const bool vec = dtype == WQ_DTYPE_BF16 && bm == 1 && (bn == 32 || bn == 64 || bn == 128) && sx_n == 1 && N % bn == 0 &&
-                     (sx_m & 7) == 0 && N / bn < (1ll << 31) && ((uintptr_t)x & 15) == 0 && ((uintptr_t)q & 15) == 0;
+                     (sx_m & 7) == 0 && N / bn < (1ll << 31) && ((uintptr_t)x & 15) == 0 && ((uintptr_t)q & 15) == 0 &&
+                     (sx_m == N || groups < (1ll << 32));
     if (vec) {
         if (sym) launch_fake_vec<true>((const uint16_t*)x, M, N, sx_m, bn, (uint16_t*)q, (uint16_t*)scale, (uint16_t*)zero, st);
         else launch_fake_vec<false>((const uint16_t*)x, M, N, sx_m, bn, (uint16_t*)q, (uint16_t*)scale, (uint16_t*)zero, st);
@@ -570,6 +589,7 @@ WQ_EXPORT int wq_int4_group_quant_pack_asym(const void* x, int64_t M, int64_t N,
         return WQ_ERR_ALIGN;
     if (N / group >= (1ll << 31)) return WQ_ERR_TOO_LARGE;
     const int64_t n_groups = M * (N / group);
+    if (sx_m != N && n_groups >= (1ll << 32)) return WQ_ERR_TOO_LARGE;      // strided rows: 32-bit group index
     const int64_t items = cdiv64(n_groups, kFakeGroupsPerWg);
     const dim3 g = grid_for_items(items);
     const int gpr = (int)(N / group);
