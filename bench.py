@@ -849,6 +849,8 @@ def main():
             extras["weight_sync_bucket"] = bench_bucket(dev, args.steps, args.warmup, args.int4_layers)
         extras["delta_xor"] = bench_delta(dev, args.steps, args.warmup)
         extras["single_tensor_forms"] = bench_single_tensor_forms(dev, args.steps, args.warmup)
+        # the practical ceiling of a 1:1 read:write stream on this very box, measured in this very run
+        extras["copy_kernel_calibration"] = bench_copy(dev, args.steps, args.warmup)
         line["other_workloads"] = extras
     print(json.dumps(line))
 
