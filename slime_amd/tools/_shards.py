@@ -90,6 +90,66 @@ def to_device(t: torch.Tensor, dev: torch.device) -> torch.Tensor:
     return t.to(dev, non_blocking=True)
 
 
+class _HostStage(threading.local):
+    """This thread's pinned staging memory for results on their way to a shard file.  A fresh pageable destination
+    (``tensor.cpu()``) costs a page fault per 4 KiB and a bounce copy: 4 GB/s on a machine whose link does 55 GB/s into
+    pinned memory.  The memory is a bump allocator over grow-only chunks; ``reset`` (start of the next shard on this
+    thread) rewinds it and folds the chunks into one, so from the second shard on a worker allocates nothing."""
+
+    chunk_bytes = 256 << 20
+
+    def __init__(self):
+        self.chunks, self.used, self.cur = [], 0, 0
+
+    def reset(self):
+        total = sum(c.numel() for c in self.chunks)
+        if len(self.chunks) > 1:
+            self.chunks = []                  # release before asking for the sum of them in one piece
+            self.chunks = [self._alloc(total)]
+        self.used = self.cur = 0
+
+    @staticmethod
+    def _alloc(nbytes: int) -> torch.Tensor:
+        try:
+            return torch.empty(nbytes, dtype=torch.uint8, pin_memory=True)
+        except RuntimeError:                  # the host refuses to lock more memory: pageable staging still works
+            return torch.empty(nbytes, dtype=torch.uint8)
+
+    def take(self, nbytes: int) -> torch.Tensor:
+        nbytes_al = -(-max(nbytes, 1) // 256) * 256
+        while self.cur < len(self.chunks) and self.used + nbytes_al > self.chunks[self.cur].numel():
+            self.cur, self.used = self.cur + 1, 0
+        if self.cur == len(self.chunks):
+            self.chunks.append(self._alloc(max(nbytes_al, self.chunk_bytes)))
+            self.used = 0
+        piece = self.chunks[self.cur][self.used:self.used + nbytes]
+        self.used += nbytes_al
+        return piece
+
+
+_stage = _HostStage()
+
+
+def begin_shard() -> None:
+    """Call at the start of every shard: host tensors handed out by ``to_host`` for the previous shard of this thread
+    are dead from here on (their memory is reused)."""
+    _stage.reset()
+
+
+def to_host(*tensors: torch.Tensor):
+    """Device tensors -> host tensors of the same shape and dtype inside this thread's pinned staging memory; one
+    synchronisation for all of them.  Valid until this thread's next ``begin_shard``."""
+    out = []
+    for t in tensors:
+        t = t.contiguous()
+        h = _stage.take(t.numel() * t.element_size()).view(t.dtype).view(t.shape)
+        h.copy_(t, non_blocking=True)
+        out.append(h)
+    if tensors:
+        torch.cuda.current_stream(tensors[0].device).synchronize()
+    return out[0] if len(out) == 1 else tuple(out)
+
+
 def copy_matching_files(input_path: str, output_path: str, keep, skip=()) -> None:
     """Copies (with metadata) the plain files of a checkpoint directory for which ``keep(name)`` holds."""
     for name in os.listdir(input_path):

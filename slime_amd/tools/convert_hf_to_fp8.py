@@ -68,6 +68,7 @@ def process_file(input_path, output_path, filename, strategy, block_size, result
 
 def _process_file(input_path, output_path, filename, strategy, block_size, result_collector):
     dev = _shards.device()
+    _shards.begin_shard()
     weights = _shards.read_shard(os.path.join(input_path, filename))
     out, skipped = {}, []
     todo = [k for k in weights if is_converted(k)]
@@ -83,12 +84,11 @@ def _process_file(input_path, output_path, filename, strategy, block_size, resul
             planned = [i for i, w in enumerate(on_gpu) if w.dtype == torch.bfloat16 and w.dim() == 2]
             for i, (k, w) in enumerate(zip(todo, on_gpu)):
                 if i not in planned:
-                    q, s = block_fp8(w, block_size)
-                    out[k], out[scale_name(k, block_size)] = q.cpu(), s.cpu()
+                    out[k], out[scale_name(k, block_size)] = _shards.to_host(*block_fp8(w, block_size))
             if planned:
                 plan = Fp8QuantPlan([on_gpu[i] for i in planned], block_size)
                 plan.run()
-                flat_q, flat_s = plan.flat_q.cpu(), plan.flat_s.cpu()     # two copies for the whole shard
+                flat_q, flat_s = _shards.to_host(plan.flat_q, plan.flat_s)     # two copies for the whole shard
                 qbase, sbase = plan.flat_q.data_ptr(), plan.flat_s.data_ptr()
                 for i, (q, s) in zip(planned, plan.outputs):
                     k = todo[i]
@@ -99,8 +99,7 @@ def _process_file(input_path, output_path, filename, strategy, block_size, resul
         else:
             fn = tensor_fp8 if strategy == "tensor" else channel_fp8
             for k, w in zip(todo, on_gpu):
-                q, s = fn(w)
-                out[k], out[scale_name(k, block_size)] = q.cpu(), s.cpu()
+                out[k], out[scale_name(k, block_size)] = _shards.to_host(*fn(w))
     # keep the reference's key order: converted weight followed by its scale, in shard order
     ordered = {}
     for k in weights:

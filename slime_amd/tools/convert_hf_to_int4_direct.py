@@ -48,6 +48,7 @@ def int4_quantization_config(group_size: int, is_symmetric: bool, ignore_rules) 
 
 def process_file(input_path, output_path, filename, group_size, is_symmetric, ignore_rules, result_collector):
     dev = _shards.device()
+    _shards.begin_shard()
     weights = _shards.read_shard(os.path.join(input_path, filename))
     todo = [n for n, w in weights.items()
             if not is_ignored(n, ignore_rules) and n.endswith(".weight") and w.dim() >= 2]
@@ -59,7 +60,7 @@ def process_file(input_path, output_path, filename, group_size, is_symmetric, ig
         if fused:
             plan = Int4PackPlan([w.contiguous() for w in on_gpu], group_size)
             plan.run()
-            flat_p, flat_s = plan.flat_packed.cpu(), plan.flat_scale.cpu()
+            flat_p, flat_s = _shards.to_host(plan.flat_packed, plan.flat_scale)
             pbase, sbase = plan.flat_packed.data_ptr(), plan.flat_scale.data_ptr()
             for n, (p, s) in zip(todo, plan.outputs):
                 po, so = (p.data_ptr() - pbase) // 4, (s.data_ptr() - sbase) // 2
@@ -67,7 +68,7 @@ def process_file(input_path, output_path, filename, group_size, is_symmetric, ig
         else:
             for n, w in zip(todo, on_gpu):
                 p, s, zp = pack_layer(w, group_size, is_symmetric)
-                results[n] = (p.cpu(), s.cpu(), None if zp is None else zp.cpu())
+                results[n] = (*_shards.to_host(p, s), None if zp is None else _shards.to_host(zp))
     out = {}
     for n, w in weights.items():
         if n not in results:

@@ -51,6 +51,7 @@ def convert_file(input_path: str, output_path: str, group_size: int, skip_existi
     if skip_existing and os.path.exists(output_path):
         return
     dev = _shards.device()
+    _shards.begin_shard()
     shard = _shards.read_shard(input_path)
     modules = {}                                  # module name -> {part: tensor}, in shard order
     for key, tensor in shard.items():
@@ -69,11 +70,11 @@ def convert_file(input_path: str, output_path: str, group_size: int, skip_existi
         if one_launch and scale.dtype == torch.bfloat16:
             bucket.append((f"{name}.weight", packed, scale, parts["weight_shape"]))
         else:       # fp16 / fp32 scales, per-element scales, odd group sizes: one launch per tensor
-            tensors[f"{name}.weight"] = _dequantize_tensor(packed, scale, parts["weight_shape"], group_size).cpu()
+            tensors[f"{name}.weight"] = _shards.to_host(_dequantize_tensor(packed, scale, parts["weight_shape"], group_size))
     if bucket:
         plan = Int4DequantPlan([b[1] for b in bucket], [b[2] for b in bucket], [b[3] for b in bucket], group_size)
         plan.run()                                # one launch and one copy for the shard
-        flat, base = plan.flat_y.cpu(), plan.flat_y.data_ptr()
+        flat, base = _shards.to_host(plan.flat_y), plan.flat_y.data_ptr()
         for (name, *_), y in zip(bucket, plan.outputs):
             off = (y.data_ptr() - base) // 2
             tensors[name] = flat[off:off + y.numel()].view(y.shape)

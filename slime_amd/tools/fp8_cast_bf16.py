@@ -47,6 +47,7 @@ def main(fp8_path, bf16_path, block_size: int = 128):
     for path in sorted(glob.glob(os.path.join(fp8_path, "*.safetensors"))):
         file_name = os.path.basename(path)
         print(f"Handling file: {path}")
+        _shards.begin_shard()
         current = shard(file_name)
         out, codes, scales, names = {}, [], [], []
         for name, t in current.items():
@@ -65,7 +66,7 @@ def main(fp8_path, bf16_path, block_size: int = 128):
         if names:
             plan = Fp8DequantPlan(codes, scales, block_size, 0, torch.bfloat16)
             plan.run()
-            flat = plan.flat_y.cpu()        # one copy for the whole shard
+            flat = _shards.to_host(plan.flat_y)        # one copy for the whole shard
             base = plan.flat_y.data_ptr()
             for name, y in zip(names, plan.outputs):
                 off = (y.data_ptr() - base) // 2

@@ -72,3 +72,26 @@ def test_int4_to_bf16_key_rule():
     assert all(K2._is_quantized_weight_key(k) for k in yes) and not any(K2._is_quantized_weight_key(k) for k in no)
     args = K2.parse_args(["--model-dir", "m", "--files", "a.safetensors", "b.safetensors", "--overwrite"])
     assert args.files == ["a.safetensors", "b.safetensors"] and args.overwrite and args.output_dir is None
+
+
+def test_host_stage_bump_allocator_reuses_and_coalesces():
+    """The staging area of the converters' device-to-host copies: aligned disjoint pieces, growth by chunks, one
+    chunk of the combined size after the next shard begins, and no allocation from then on."""
+    from slime_amd.tools._shards import _HostStage
+
+    st = _HostStage()
+    st.chunk_bytes = 4096
+    a, b = st.take(1000), st.take(3500)          # second piece does not fit behind the first: new chunk
+    c = st.take(10000)                           # bigger than a chunk
+    assert [x.numel() for x in (a, b, c)] == [1000, 3500, 10000]
+    assert len(st.chunks) == 3 and all(x.data_ptr() % 64 == 0 for x in (a, b, c))
+    a.fill_(1), b.fill_(2), c.fill_(3)
+    assert (int(a.sum()), int(b.sum()), int(c.sum())) == (1000, 7000, 30000)      # disjoint
+    st.reset()
+    assert len(st.chunks) == 1 and st.chunks[0].numel() == 4096 + 4096 + 10240
+    base = st.chunks[0].data_ptr()
+    pieces = [st.take(n) for n in (1000, 3500, 10000)]
+    assert len(st.chunks) == 1 and pieces[0].data_ptr() == base
+    assert pieces[1].data_ptr() == base + 1024 and pieces[2].data_ptr() == base + 1024 + 3584
+    st.reset()
+    assert st.take(0).numel() == 0 and st.take(5).data_ptr() == base + 256
