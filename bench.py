@@ -529,7 +529,11 @@ def bench_single_tensor_forms(dev, steps, warmup):
     cases = (("fp8_channel_quant", lambda: slime_amd.channel_fp8(w), 3 * el + 4 * w.shape[0]),
              ("fp8_tensor_quant", lambda: slime_amd.tensor_fp8(w), 5 * el),
              ("int4_fake_quant_sym", lambda: slime_amd.fake_int4_quant_cuda(w, (1, 128), True), 4 * el + 4 * el // 128),
-             ("int4_fake_quant_asym", lambda: slime_amd.fake_int4_quant_cuda(w, (1, 128), False), 4 * el + 4 * el // 128))
+             ("int4_fake_quant_asym", lambda: slime_amd.fake_int4_quant_cuda(w, (1, 128), False), 4 * el + 4 * el // 128),
+             # FP8-aligned weight: quantise + expand in one pass (4 bytes per element), and the two kernels it replaces
+             ("fp8_aligned_weight", lambda: slime_amd.fp8_aligned_weight(w), 4 * el),
+             ("fp8_quant_then_dequant", lambda: slime_amd.block_quant_dequant(
+                 *slime_amd.blockwise_cast_to_fp8_triton(w, (128, 128)), [128, 128], torch.bfloat16), 6 * el))
     for name, fn, algo in cases:
         wall_ms, ev_ms, ev_min = _time_launches(fn, steps, warmup)
         out[name] = {"kernel_ms": ev_ms, "bf16_GBps": 2 * el / ev_ms / 1e6, "algo_GBps": algo / ev_ms / 1e6,
@@ -543,8 +547,12 @@ def bench_single_tensor_forms(dev, steps, warmup):
         assert torch.equal(q[:512].cpu().view(torch.int16), qo.view(torch.int16))
         assert torch.equal(s[:512].cpu().view(torch.int16), so.view(torch.int16))
         assert torch.equal(z[:512].cpu().view(torch.int16), zo.view(torch.int16))
+    y = slime_amd.fp8_aligned_weight(w)
+    qo, so = c_oracle.fp8_block_quant(head, (128, 128), 1)
+    assert torch.equal(y[:512].cpu().view(torch.int16), c_oracle.fp8_block_dequant(qo, so, 128, 0).view(torch.int16))
     out["workload"] = ("one bf16 [151936, 2560] tensor (778 MB); algorithmic bytes per element: channel 3, tensor 5 (two "
-                       "reads), fake INT4 4; parity checked on the first 512 rows")
+                       "reads), fake INT4 4, FP8-aligned weight 4 (the quantiser followed by the dequantiser: 6); parity "
+                       "checked on the first 512 rows")
     del w
     torch.cuda.empty_cache()
     return out

@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define WQ_ABI_VERSION 12
+#define WQ_ABI_VERSION 13
 
 enum {
     WQ_OK = 0,
@@ -136,6 +136,18 @@ int wq_fp8_row_quant(const void *x, int64_t M, int64_t N, int64_t sx_m, int64_t 
                      void *y, int64_t sy_m, float *s, int mode, void *stream);
 int wq_fp8_tensor_quant(const void *x, int64_t M, int64_t N, int64_t sx_m, int64_t sx_n,
                         void *y, int64_t sy_m, float *s, uint32_t *workspace, int mode, void *stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * bf16 [M,N] -> bf16 [M,N] carrying the values the weight has after block-FP8 quantisation: per block
+ * the codes of wq_fp8_block_quant (same `mode`, all four accepted) are formed in registers and expanded
+ * again as wq_fp8_block_dequant does (f32(code) * scale, one RNE rounding to bf16), in ONE pass of
+ * 2 + 2 bytes per element.  Replaces the pair blockwise_cast_to_fp8_triton / quant_weight_ue8m0 ->
+ * block_quant_dequant of _get_fp8_aligned_absorb_weight (slime_plugins/models/glm5/glm5.py:105-165;
+ * modes WQ_FP8_MODE_TRITON and WQ_FP8_MODE_UE8M0 there) and is bit-identical to the two calls.
+ * Strides in elements (y: unit column stride); `s` [ceil(M/bm), ceil(N/bn)] contiguous receives the
+ * block scales, or NULL. */
+int wq_fp8_block_quant_dequant(const void *x, int64_t M, int64_t N, int64_t sx_m, int64_t sx_n, void *y,
+                               int64_t sy_m, float *s, int bm, int bn, int mode, void *stream);
 
 /* ---------------------------------------------------------------------------------------------
  * e4m3fn [M,N] contiguous + fp32 scale [ceil(M/block), ceil(N/block)] contiguous -> y [M,N]

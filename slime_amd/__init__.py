@@ -7,6 +7,7 @@ of ``slime_amd/lib/libslime_amd_wq.so``; there is no CPU or pure-torch fallback.
 """
 
 from . import _lib, arith, delta
+from .aligned import get_fp8_aligned_absorb_weight
 from .bucket import BucketConverter, FlattenedBucket, FlattenedTensorMetadata, quantize_bucket
 from .arith import get_torch_arithmetic, set_torch_arithmetic, torch_arithmetic
 from .fp8 import (
@@ -14,8 +15,10 @@ from .fp8 import (
     Fp8QuantPlan,
     block_fp8,
     block_fp8_many,
+    block_quant_dequant,
     blockwise_cast_to_fp8_triton,
     channel_fp8,
+    fp8_aligned_weight,
     quant_fp8,
     quant_weight_ue8m0,
     tensor_fp8,
@@ -48,6 +51,7 @@ from .processors import (
 quantize_weight = blockwise_cast_to_fp8_triton
 
 __all__ = [
+    "block_quant_dequant", "fp8_aligned_weight", "get_fp8_aligned_absorb_weight",
     "Int4StePlan", "fake_int4_quantization_ste_many", "BucketConverter", "FlattenedBucket", "FlattenedTensorMetadata", "quantize_bucket", "quant_weight_ue8m0",
     "set_ue8m0_requant", "transform_scale_ue8m0",
     "Fp8DequantPlan", "Fp8QuantPlan", "Int4DequantPlan", "Int4PackPlan", "block_fp8", "block_fp8_many",

@@ -181,6 +181,44 @@ def weight_dequant(x: torch.Tensor, s: torch.Tensor, block_size: int = 128) -> t
     return _dequant(x, s, block_size, _lib.DEQ_MODE_F32SCALE, torch.get_default_dtype(), "weight_dequant")
 
 
+def block_quant_dequant(x_q_block: torch.Tensor, x_s: torch.Tensor, block_size, dtype: torch.dtype) -> torch.Tensor:
+    """Name and arguments of the sglang helper the reference calls at slime_plugins/models/glm5/glm5.py:144-161
+    (``block_quant_dequant(qweight, scale_inv, [128, 128], torch.bfloat16)``): e4m3fn codes times their block scale in
+    fp32, rounded once to ``dtype`` (bfloat16 or float32) - ``weight_dequant``'s arithmetic with an explicit output
+    type.  Square blocks only (the dequantiser's contract)."""
+    bm, bn = int(block_size[0]), int(block_size[1])
+    if bm != bn:
+        raise ValueError(f"block_quant_dequant: square blocks only, got {bm}x{bn}")
+    return _dequant(x_q_block, x_s, bm, _lib.DEQ_MODE_F32SCALE, dtype, "block_quant_dequant")
+
+
+def fp8_aligned_weight(weight: torch.Tensor, block_size=(128, 128), use_ue8m0: bool = False,
+                       return_scale: bool = False):
+    """bf16 weight -> bf16 weight holding the values it has after block-FP8 quantisation, in ONE pass (2 + 2 bytes per
+    element instead of 3 + 3 and no code tensor).  Bit-identical to the pair the reference runs in
+    ``_get_fp8_aligned_absorb_weight`` (slime_plugins/models/glm5/glm5.py:105-165)::
+
+        block_quant_dequant(*blockwise_cast_to_fp8_triton(w.contiguous(), (128, 128)), [128, 128], torch.bfloat16)
+        block_quant_dequant(*quant_weight_ue8m0(w.contiguous(), [128, 128]), [128, 128], torch.bfloat16)   # use_ue8m0
+
+    Any row / column strides; ``return_scale`` also returns the float32 block scales."""
+    _check_weight(weight, "fp8_aligned_weight")
+    bm, bn = int(block_size[0]), int(block_size[1])
+    if bm <= 0 or bn <= 0:
+        raise ValueError(f"fp8_aligned_weight: block size must be positive, got {block_size}")
+    M, N = weight.shape
+    y = torch.empty((M, N), dtype=torch.bfloat16, device=weight.device)
+    s = torch.empty((ceildiv(M, bm), ceildiv(N, bn)), dtype=torch.float32, device=weight.device) if return_scale else None
+    if M and N:
+        with torch.cuda.device(weight.device):
+            rc = _lib.load().wq_fp8_block_quant_dequant(
+                weight.data_ptr(), M, N, weight.stride(0), weight.stride(1), y.data_ptr(), N,
+                s.data_ptr() if return_scale else None, bm, bn,
+                _lib.FP8_MODE_UE8M0 if use_ue8m0 else _lib.FP8_MODE_TRITON, _lib.stream_ptr(weight.device))
+        _lib.check(rc, "fp8_aligned_weight")
+    return (y, s) if return_scale else y
+
+
 def weight_dequant_bf16_scale(x: torch.Tensor, s: torch.Tensor, block_size: int = 128) -> torch.Tensor:
     """Dequant-on-read of the HF->Megatron loader (hf_to_megatron/common.py:42-56): the scale is
     rounded to bf16 before the multiply; result bf16."""
