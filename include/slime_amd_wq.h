@@ -9,7 +9,9 @@
  *     as void*; NULL selects the default stream.  Launches are asynchronous and are ordered
  *     on `stream` only; the library keeps no mutable global state and every entry point may
  *     be called concurrently from several host threads (one exception, documented there:
- *     wq_delta_xor_noalloc works in a device array owned by the library).
+ *     wq_delta_xor_noalloc works in a device array owned by the library).  No entry point
+ *     allocates, frees, clears memory with a memset node or synchronises, so every call may be
+ *     recorded into a HIP graph (stream capture) and replayed on updated inputs.
  *   - Return value: 0 on success, a negative WQ_ERR_* for rejected arguments (nothing was
  *     launched), or a positive hipError_t reported by the launch.  wq_error_string() names any
  *     of them.
