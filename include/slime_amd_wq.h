@@ -32,7 +32,7 @@
 extern "C" {
 #endif
 
-#define WQ_ABI_VERSION 13
+#define WQ_ABI_VERSION 14
 
 enum {
     WQ_OK = 0,
@@ -138,6 +138,12 @@ int wq_fp8_row_quant(const void *x, int64_t M, int64_t N, int64_t sx_m, int64_t 
                      void *y, int64_t sy_m, float *s, int mode, void *stream);
 int wq_fp8_tensor_quant(const void *x, int64_t M, int64_t N, int64_t sx_m, int64_t sx_n,
                         void *y, int64_t sy_m, float *s, uint32_t *workspace, int mode, void *stream);
+/* tensor_fp8 for the other floating dtypes the reference function takes (dtype: WQ_DTYPE_BF16 / F32 / F16): the
+ * quotient is rounded to the weight's dtype before the clamp, as torch's type promotion with a 0-dim scale makes it;
+ * plain two-pass kernels.  (channel_fp8 on those dtypes is wq_fp8_block_quant_any with bm = 1, bn = N: a row is a
+ * block, and both divide by a dimensioned fp32 scale.) */
+int wq_fp8_tensor_quant_any(const void *x, int dtype, int64_t M, int64_t N, int64_t sx_m, int64_t sx_n,
+                            void *y, int64_t sy_m, float *s, uint32_t *workspace, int mode, void *stream);
 
 /* ---------------------------------------------------------------------------------------------
  * bf16 [M,N] -> bf16 [M,N] carrying the values the weight has after block-FP8 quantisation: per block

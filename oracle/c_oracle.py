@@ -35,13 +35,16 @@ def lib() -> ctypes.CDLL:
         L.wqo_fp8_block_quant_any.argtypes = [_vp, _int, _i64, _i64, _i64, _i64, _i64, _i64, _int, _vp, _vp]
         L.wqo_fp8_channel_quant.argtypes = [_vp, _i64, _i64, _i64, _i64, _int, _vp, _vp]
         L.wqo_fp8_tensor_quant.argtypes = [_vp, _i64, _i64, _i64, _i64, _int, _vp, _vp]
+        L.wqo_fp8_tensor_quant_any.argtypes = [_vp, _int, _i64, _i64, _i64, _i64, _int, _vp, _vp]
+        L.wqo_f32_to_f16.argtypes = [ctypes.c_float]
+        L.wqo_f32_to_f16.restype = ctypes.c_uint16
         L.wqo_fp8_block_dequant.argtypes = [_vp, _vp, _i64, _i64, _i64, _int, _vp]
         L.wqo_int4_fake_quant.argtypes = [_vp, _int, _i64, _i64, _i64, _i64, _i64, _i64, _int, _vp, _vp, _vp]
         L.wqo_int4_pack_layer.argtypes = [_vp, _i64, _i64, _i64, _int, _vp, _vp, _vp]
         L.wqo_int4_dequant.argtypes = [_vp, _vp, _i64, _i64, _i64, _vp]
         L.wqo_int4_dequant_any.argtypes = [_vp, _vp, _int, _i64, _i64, _i64, _vp]
         L.wqo_int4_fake_ste.argtypes = [_vp, _i64, _i64, _i64, _int, _vp]
-        for n in ("wqo_f32_to_e4m3fn_n", "wqo_e4m3fn_to_f32_n", "wqo_f32_to_bf16_n"):
+        for n in ("wqo_f32_to_e4m3fn_n", "wqo_e4m3fn_to_f32_n", "wqo_f32_to_bf16_n", "wqo_f32_to_f16_n"):
             getattr(L, n).argtypes = [_vp, _vp, _i64]
             getattr(L, n).restype = None
         L.wqo_num_threads.restype = _int
@@ -85,6 +88,13 @@ def f32_to_bf16(x: torch.Tensor) -> torch.Tensor:
     return y
 
 
+def f32_to_f16(x: torch.Tensor) -> torch.Tensor:
+    x = _cpu(x).contiguous().to(torch.float32)
+    y = torch.empty(x.shape, dtype=torch.float16)
+    lib().wqo_f32_to_f16_n(x.data_ptr(), y.data_ptr(), x.numel())
+    return y
+
+
 def fp8_block_quant(w: torch.Tensor, block_size=(128, 128), mode: int = 0):
     """-> (uint8 [M,N] holding e4m3fn codes, float32 [cdiv(M,bm), cdiv(N,bn)])."""
     assert _cpu(w).dim() == 2
@@ -102,8 +112,13 @@ def fp8_block_quant(w: torch.Tensor, block_size=(128, 128), mode: int = 0):
     return y, s
 
 
+_ANY_DTYPE = {torch.bfloat16: 0, torch.float32: 1, torch.float16: 2}
+
+
 def fp8_channel_quant(w: torch.Tensor, mode: int = 0):
-    assert _cpu(w).dtype == torch.bfloat16 and w.dim() == 2
+    assert _cpu(w).dim() == 2
+    if w.dtype != torch.bfloat16:        # a row is a block of shape (1, N): same arithmetic (dimensioned fp32 scale)
+        return fp8_block_quant(w, (1, max(w.shape[1], 1)), mode)
     M, N = w.shape
     y = torch.empty(M, N, dtype=torch.uint8)
     s = torch.empty(M, 1, dtype=torch.float32)
@@ -114,10 +129,14 @@ def fp8_channel_quant(w: torch.Tensor, mode: int = 0):
 
 
 def fp8_tensor_quant(w: torch.Tensor, mode: int = 0):
-    assert _cpu(w).dtype == torch.bfloat16 and w.dim() == 2
+    assert _cpu(w).dim() == 2
     M, N = w.shape
     y = torch.empty(M, N, dtype=torch.uint8)
     s = torch.empty(1, dtype=torch.float32)
+    if w.dtype != torch.bfloat16:
+        _check(lib().wqo_fp8_tensor_quant_any(w.data_ptr(), _ANY_DTYPE[w.dtype], M, N, w.stride(0), w.stride(1), mode,
+                                              y.data_ptr(), s.data_ptr()), "fp8_tensor_quant")
+        return y, s
     _check(lib().wqo_fp8_tensor_quant(w.data_ptr(), M, N, w.stride(0), w.stride(1), mode, y.data_ptr(),
                                       s.data_ptr()),
            "fp8_tensor_quant")

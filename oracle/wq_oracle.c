@@ -17,6 +17,8 @@
  *   wqo_fp8_channel_quant tools/convert_hf_to_fp8.py:78-83 (channel_fp8)
  *   wqo_fp8_tensor_quant  tools/convert_hf_to_fp8.py:86-91 (tensor_fp8), same arithmetic as
  *                         megatron_to_hf/processors/quantizer_fp8.py:114-116
+ *   wqo_fp8_tensor_quant_any  the same function on fp16 / fp32 weights (channel_fp8 on those dtypes is
+ *                         wqo_fp8_block_quant_any with blocks of one row)
  *   wqo_fp8_block_dequant mode 0: tools/fp8_cast_bf16.py:16-41 (weight_dequant)
  *                         mode 1: slime/backends/megatron_utils/hf_to_megatron/common.py:42-56
  *   wqo_int4_fake_quant   slime/backends/megatron_utils/kernels/int4_qat/fake_int4_quant_cuda.cu:37-267
@@ -352,6 +354,67 @@ WQO_API int wqo_fp8_tensor_quant(const uint16_t *x, int64_t M, int64_t N, int64_
     for (int64_t i = 0; i < M; ++i)
         for (int64_t j = 0; j < N; ++j)
             y[i * N + j] = quant_elem_tensor(wqo_bf16_to_f32(x[i * sx_m + j * sx_n]), divisor);
+    return 0;
+}
+
+/* fp32 -> fp16 bits, round-to-nearest-even, subnormals kept, overflow to infinity, NaN stays NaN (quiet). */
+WQO_API uint16_t wqo_f32_to_f16(float f)
+{
+    uint32_t u = f2u(f), sign = (u >> 16) & 0x8000u, a = u & 0x7FFFFFFFu;
+    if (a > 0x7F800000u) return (uint16_t)(sign | 0x7E00u | ((a >> 13) & 0x3FFu));      /* NaN */
+    if (a >= 0x47800000u) return (uint16_t)(sign | 0x7C00u);                               /* >= 2^16 (and inf): inf */
+    if (a < 0x33000000u) return (uint16_t)sign;                                            /* < 2^-25: zero */
+    if (a < 0x38800000u) {
+        /* below 2^-14: subnormal result = RNE(|f| * 2^24), an integer of at most 11 bits (1024 = the smallest normal) */
+        int e = (int)(a >> 23);                                /* biased exponent, 102..112 */
+        uint32_t m = (a & 0x7FFFFFu) | 0x800000u;              /* 24-bit significand: |f| = m * 2^(e-150) */
+        int shift = 126 - e;                                   /* |f| * 2^24 = m >> shift, shift in 14..24 */
+        uint32_t q = m >> shift, rem = m & ((1u << shift) - 1u), half = 1u << (shift - 1);
+        if (rem > half || (rem == half && (q & 1u))) ++q;
+        return (uint16_t)(sign | q);
+    }
+    /* normal: drop 13 bits of the significand with RNE; the carry walks into the exponent (up to infinity) */
+    uint32_t r = a - 0x38000000u;                              /* rebias 127 -> 15 */
+    uint32_t q = r >> 13, rem = r & 0x1FFFu;
+    if (rem > 0x1000u || (rem == 0x1000u && (q & 1u))) ++q;
+    return (uint16_t)(sign | q);
+}
+
+WQO_API void wqo_f32_to_f16_n(const float *x, uint16_t *y, int64_t n)
+{ for (int64_t i = 0; i < n; ++i) y[i] = wqo_f32_to_f16(x[i]); }
+
+/* value rounded to the weight dtype and widened again: what a torch op with that result dtype leaves behind */
+static inline float round_to_dtype(float v, int dtype)
+{
+    if (dtype == 1) return v;
+    if (dtype == 2) return wqo_f16_to_f32(wqo_f32_to_f16(v));
+    return wqo_bf16_to_f32(wqo_f32_to_bf16(v));
+}
+
+/* tensor_fp8 for the other floating dtypes the reference function takes (convert_hf_to_fp8.py:86-91; dtype as in
+ * load_any).  `weight / scale` has the weight's dtype (the 0-dim fp32 scale does not take part in type promotion): the
+ * fp32 quotient is rounded to it - no second rounding for fp32 weights - and on GPU tensors (mode 2) the divisor is
+ * converted to it first. */
+WQO_API int wqo_fp8_tensor_quant_any(const void *x, int dtype, int64_t M, int64_t N, int64_t sx_m, int64_t sx_n,
+                                     int mode, uint8_t *y, float *s)
+{
+    if (M < 0 || N < 0 || (mode != 0 && mode != 2) || dtype < 0 || dtype > 2) return 1;
+    volatile float inv448 = 1.0f / FP8_MAX;
+    float amax = 0.0f;
+    for (int64_t i = 0; i < M; ++i)
+        for (int64_t j = 0; j < N; ++j)
+            amax = max_nanprop(amax, fabsf(load_any(x, dtype, i * sx_m + j * sx_n)));
+    float a = amax;
+    if (a == a && a < torch_floor(dtype)) a = torch_floor(dtype);
+    float scale = mode == 2 ? a * inv448 : a / FP8_MAX;
+    float divisor = mode == 2 ? round_to_dtype(scale, dtype) : scale;
+    s[0] = scale;
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < M; ++i)
+        for (int64_t j = 0; j < N; ++j) {
+            float q = round_to_dtype(load_any(x, dtype, i * sx_m + j * sx_n) / divisor, dtype);
+            y[i * N + j] = wqo_f32_to_e4m3fn(clamp_nanprop(q, -FP8_MAX, FP8_MAX));
+        }
     return 0;
 }
 

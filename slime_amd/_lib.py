@@ -15,7 +15,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libslime_amd_wq.so")
 
-ABI_VERSION = 13
+ABI_VERSION = 14
 
 # selectors (mirrors of the header's enums)
 DTYPE_BF16, DTYPE_F32, DTYPE_F16, DTYPE_F64 = 0, 1, 2, 3
@@ -41,6 +41,7 @@ SIGNATURES = {
     "wq_fp8_block_quant_any": [_vp, _int, _i64, _i64, _i64, _i64, _vp, _i64, _vp, _int, _int, _int, _vp],
     "wq_fp8_row_quant": [_vp, _i64, _i64, _i64, _i64, _vp, _i64, _vp, _int, _vp],
     "wq_fp8_tensor_quant": [_vp, _i64, _i64, _i64, _i64, _vp, _i64, _vp, _vp, _int, _vp],
+    "wq_fp8_tensor_quant_any": [_vp, _int, _i64, _i64, _i64, _i64, _vp, _i64, _vp, _vp, _int, _vp],
     "wq_fp8_block_dequant": [_vp, _vp, _vp, _int, _i64, _i64, _int, _int, _vp],
     "wq_fp8_block_quant_dequant": [_vp, _i64, _i64, _i64, _i64, _vp, _i64, _vp, _int, _int, _int, _vp],
     "wq_fp8_block_dequant_grouped": [_vp, _vp, _int, _i64, _int, _int, _int, _vp],

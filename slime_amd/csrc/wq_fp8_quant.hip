@@ -571,6 +571,61 @@ static void launch_block_quant_any(const void* x, int64_t M, int64_t N, int64_t 
         fp8_block_quant_any_kernel<T, WQ_FP8_MODE_TRITON><<<g, 256, 0, st>>>(x, M, N, sx_m, sx_n, y, sy_m, s, bm, bn, tiles);
 }
 
+// tensor_fp8 on the other floating dtypes: `weight / scale` has the weight's dtype (the 0-dim fp32 scale does not take part
+// in type promotion), so the fp32 quotient is rounded to it before the clamp - no second rounding for fp32 weights - and on
+// GPU tensors the divisor is converted to it first.  Workspace: the fp32 bits of the NaN-propagating max |x| (for
+// non-negative floats and NaNs the unsigned order of the bits is the order torch.max uses).
+template <typename T> __device__ __forceinline__ float round_to(float v);
+template <> __device__ __forceinline__ float round_to<float>(float v) { return v; }
+template <> __device__ __forceinline__ float round_to<_Float16>(float v) { return (float)(_Float16)v; }
+template <> __device__ __forceinline__ float round_to<uint16_t>(float v) { return u2f(f32_to_bf16_bits(v) << 16); }
+
+template <typename T>
+__global__ __launch_bounds__(256) void fp8_tensor_amax_any_kernel(const void* __restrict__ x, int64_t M, int64_t N,
+                                                                 int64_t sx_m, int64_t sx_n, uint32_t* __restrict__ ws)
+{
+    __shared__ uint32_t lds[4];
+    const int64_t total = M * N;
+    uint32_t m = 0;
+    for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < total; e += (int64_t)gridDim.x * 256) {
+        const int64_t i = e / N, j = e - i * N;
+        m = max(m, f2u(load_any<T>(x, i * sx_m + j * sx_n)) & 0x7FFFFFFFu);
+    }
+    m = wave64_max_u32(m);
+    if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6] = m;
+    __syncthreads();
+    if (threadIdx.x == 0) atomicMax(ws, max(max(lds[0], lds[1]), max(lds[2], lds[3])));
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void fp8_tensor_apply_any_kernel(const void* __restrict__ x, int64_t M, int64_t N,
+                                                                  int64_t sx_m, int64_t sx_n, uint8_t* __restrict__ y,
+                                                                  int64_t sy_m, float* __restrict__ s,
+                                                                  const uint32_t* __restrict__ ws, int mode)
+{
+    const float m = u2f(*ws);
+    const float a = m != m ? m : fmaxf(m, torch_floor_1em12<T>());
+    const float scale = mode == WQ_FP8_MODE_TORCH_DEVICE ? a * (1.0f / kFp8Max) : a / kFp8Max;
+    if (blockIdx.x == 0 && threadIdx.x == 0) s[0] = scale;
+    const float divisor = mode == WQ_FP8_MODE_TORCH_DEVICE ? round_to<T>(scale) : scale;
+    const int64_t total = M * N;
+    for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < total; e += (int64_t)gridDim.x * 256) {
+        const int64_t i = e / N, j = e - i * N;
+        float q = round_to<T>(load_any<T>(x, i * sx_m + j * sx_n) / divisor);
+        if (q == q) q = fminf(fmaxf(q, -kFp8Max), kFp8Max);
+        y[i * sy_m + j] = (uint8_t)f32_to_e4m3fn_sw(q);
+    }
+}
+
+template <typename T>
+static void launch_tensor_quant_any(const void* x, int64_t M, int64_t N, int64_t sx_m, int64_t sx_n, uint8_t* y,
+                                    int64_t sy_m, float* s, uint32_t* ws, int mode, hipStream_t st)
+{
+    const int blocks = (int)min((int64_t)(256 * 16), max((int64_t)1, cdiv64(M * N, 256 * 8)));
+    fp8_tensor_amax_any_kernel<T><<<blocks, 256, 0, st>>>(x, M, N, sx_m, sx_n, ws);
+    fp8_tensor_apply_any_kernel<T><<<blocks, 256, 0, st>>>(x, M, N, sx_m, sx_n, y, sy_m, s, ws, mode);
+}
+
 static bool known_mode(int mode)
 {
     return mode == WQ_FP8_MODE_TORCH || mode == WQ_FP8_MODE_TRITON || mode == WQ_FP8_MODE_TORCH_DEVICE ||
@@ -709,6 +764,21 @@ WQ_EXPORT int wq_fp8_block_quant_any(const void* x, int dtype, int64_t M, int64_
     if (dtype == WQ_DTYPE_F32) launch_block_quant_any<float>(x, M, N, sx_m, sx_n, (uint8_t*)y, sy_m, s, bm, bn, mode, st);
     else if (dtype == WQ_DTYPE_F16) launch_block_quant_any<_Float16>(x, M, N, sx_m, sx_n, (uint8_t*)y, sy_m, s, bm, bn, mode, st);
     else launch_block_quant_any<uint16_t>(x, M, N, sx_m, sx_n, (uint8_t*)y, sy_m, s, bm, bn, mode, st);
+    WQ_LAUNCH_CHECK();
+    return WQ_OK;
+}
+
+WQ_EXPORT int wq_fp8_tensor_quant_any(const void* x, int dtype, int64_t M, int64_t N, int64_t sx_m, int64_t sx_n, void* y,
+                                      int64_t sy_m, float* s, uint32_t* workspace, int mode, void* stream)
+{
+    if (dtype == WQ_DTYPE_BF16) return wq_fp8_tensor_quant(x, M, N, sx_m, sx_n, y, sy_m, s, workspace, mode, stream);
+    if (dtype != WQ_DTYPE_F32 && dtype != WQ_DTYPE_F16) return WQ_ERR_MODE;
+    if (M < 0 || N < 0) return WQ_ERR_SHAPE;
+    if (mode != WQ_FP8_MODE_TORCH && mode != WQ_FP8_MODE_TORCH_DEVICE) return WQ_ERR_MODE;
+    if (!s || !workspace || (M * N > 0 && (!x || !y))) return WQ_ERR_NULL;
+    hipStream_t st = (hipStream_t)stream;
+    if (dtype == WQ_DTYPE_F32) launch_tensor_quant_any<float>(x, M, N, sx_m, sx_n, (uint8_t*)y, sy_m, s, workspace, mode, st);
+    else launch_tensor_quant_any<_Float16>(x, M, N, sx_m, sx_n, (uint8_t*)y, sy_m, s, workspace, mode, st);
     WQ_LAUNCH_CHECK();
     return WQ_OK;
 }

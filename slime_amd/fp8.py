@@ -78,7 +78,11 @@ def block_fp8(weight: torch.Tensor, block_size) -> tuple[torch.Tensor, torch.Ten
 
 
 def channel_fp8(weight: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
-    """Per-row scaling, tools/convert_hf_to_fp8.py:78-83 -> (qweight [M,N], scale float32 [M,1])."""
+    """Per-row scaling, tools/convert_hf_to_fp8.py:78-83 -> (qweight [M,N], scale float32 [M,1]).  bf16 rows take the
+    bandwidth-tuned kernels; fp16 / fp32 weights are quantised as blocks of one row (the same arithmetic: both
+    divide by a dimensioned float32 scale)."""
+    if weight.dtype in _OTHER_FLOAT_DTYPES and weight.dim() == 2:
+        return _block_quant(weight, 1, max(int(weight.shape[1]), 1), arith.fp8_torch_mode(), "channel_fp8")
     _check_weight(weight, "channel_fp8")
     M, N = weight.shape
     q = torch.empty((M, N), dtype=FP8_DTYPE, device=weight.device)
@@ -93,16 +97,27 @@ def channel_fp8(weight: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
 
 
 def tensor_fp8(weight: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
-    """Per-tensor scaling, tools/convert_hf_to_fp8.py:86-91 -> (qweight [M,N], scale float32 [1])."""
-    _check_weight(weight, "tensor_fp8")
+    """Per-tensor scaling, tools/convert_hf_to_fp8.py:86-91 -> (qweight [M,N], scale float32 [1]).  The quotient is
+    rounded to the weight's dtype before the clamp, as torch's type promotion with a 0-dim scale makes it (bf16 and
+    fp16 weights round twice, fp32 weights once); fp16 / fp32 weights take plain two-pass kernels."""
+    other = weight.dtype in _OTHER_FLOAT_DTYPES and weight.dim() == 2
+    if other:
+        _lib.require_gpu(weight, "tensor_fp8")
+    else:
+        _check_weight(weight, "tensor_fp8")
     M, N = weight.shape
     q = torch.empty((M, N), dtype=FP8_DTYPE, device=weight.device)
     s = torch.empty((1,), dtype=torch.float32, device=weight.device)
     ws = torch.zeros((1,), dtype=torch.int32, device=weight.device)
     with torch.cuda.device(weight.device):
-        rc = _lib.load().wq_fp8_tensor_quant(weight.data_ptr(), M, N, weight.stride(0), weight.stride(1),
-                                             q.data_ptr(), N, s.data_ptr(), ws.data_ptr(), arith.fp8_torch_mode(),
-                                             _lib.stream_ptr(weight.device))
+        if other:
+            rc = _lib.load().wq_fp8_tensor_quant_any(weight.data_ptr(), _OTHER_FLOAT_DTYPES[weight.dtype], M, N,
+                                                     weight.stride(0), weight.stride(1), q.data_ptr(), N, s.data_ptr(),
+                                                     ws.data_ptr(), arith.fp8_torch_mode(), _lib.stream_ptr(weight.device))
+        else:
+            rc = _lib.load().wq_fp8_tensor_quant(weight.data_ptr(), M, N, weight.stride(0), weight.stride(1),
+                                                 q.data_ptr(), N, s.data_ptr(), ws.data_ptr(), arith.fp8_torch_mode(),
+                                                 _lib.stream_ptr(weight.device))
     _lib.check(rc, "tensor_fp8")
     return q, s
 

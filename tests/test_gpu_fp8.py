@@ -448,6 +448,44 @@ def test_block_quant_other_dtypes_match_torch_ops_on_the_gpu(cuda, dt):
     assert torch.equal(_bits32(s), _bits32(sr)) and torch.equal(_codes(q), _codes(qr))
 
 
+@pytest.mark.parametrize("dt", [torch.float16, torch.float32])
+@pytest.mark.parametrize("mode", [0, 2])
+def test_channel_and_tensor_quant_other_dtypes(cuda, dt, mode):
+    """fp16 / fp32 weights through the per-row and per-tensor forms, against the oracle: the per-tensor quotient is
+    rounded to the weight's dtype (twice-rounded for fp16, once for fp32), rows are blocks of one row."""
+    g = torch.Generator().manual_seed(7)
+    for shape in ((256, 384), (300, 200), (7, 7168), (129, 127)):
+        w = I.weights(*shape, seed=sum(shape))
+        x = (w.float() * (1 + 1e-3 * torch.randn(shape, generator=g))).to(dt)
+        x[3] = 0                                            # an all-zero row: 0 / 0 for fp16 (its clamp bound rounds to 0)
+        for view in (lambda t: t, lambda t: t.t(), lambda t: t[::2, 1:]):
+            xc, xg = view(x), view(x.to(cuda))
+            with slime_amd.torch_arithmetic(ARITH[mode]):
+                q, s = slime_amd.channel_fp8(xg)
+                qt, st = slime_amd.tensor_fp8(xg)
+            for (got, sc), (qo, so) in (((q, s), C.fp8_channel_quant(xc, mode)), ((qt, st), C.fp8_tensor_quant(xc, mode))):
+                qc = _codes(got)
+                nan = (qo & 0x7F) == 0x7F
+                assert torch.equal((qc & 0x7F) == 0x7F, nan) and torch.equal(qc[~nan], qo[~nan]), (shape, dt, mode)
+                snan = so.isnan()
+                assert torch.equal(sc.cpu().isnan().view(-1), snan.view(-1))
+                assert torch.equal(_bits32(sc).view(-1)[~snan.view(-1)], _bits32(so).view(-1)[~snan.view(-1)])
+            assert s.shape == (xg.shape[0], 1) and st.shape == (1,)
+
+
+@pytest.mark.parametrize("dt", [torch.float16, torch.float32])
+def test_channel_and_tensor_quant_other_dtypes_match_torch_ops_on_the_gpu(cuda, dt):
+    # torch's own GPU kernels running the reference's lines: the witness for the dtype of the quotient and of the divisor
+    g = torch.Generator().manual_seed(8)
+    for shape, std in (((512, 640), 0.02), ((300, 200), 1.0), ((64, 4096), 1e-3)):
+        w = I.weights(*shape, seed=9, std=std)
+        x = (w.float() * (1 + 1e-3 * torch.randn(shape, generator=g))).to(dt).to(cuda)
+        for ref, mine in ((T.channel_fp8_ref, slime_amd.channel_fp8), (T.tensor_fp8_ref, slime_amd.tensor_fp8)):
+            qr, sr = ref(x)
+            q, s = mine(x)
+            assert torch.equal(_bits32(s), _bits32(sr)) and torch.equal(_codes(q), _codes(qr)), (shape, dt)
+
+
 def test_int8_weights_are_refused(cuda):
     with pytest.raises(TypeError):
         slime_amd.block_fp8(torch.zeros(128, 128, dtype=torch.int8, device=cuda), (128, 128))

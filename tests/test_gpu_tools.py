@@ -112,6 +112,27 @@ def test_convert_hf_to_fp8_other_strategies(ckpt, tmp_path, cuda, strategy):
     assert (q["quant_method"] == "fp8") == (strategy == "tensor")
 
 
+@pytest.mark.parametrize("strategy", ["block", "tensor", "channel"])
+def test_convert_hf_to_fp8_half_and_single_precision_checkpoints(tmp_path, cuda, strategy):
+    """The reference's quant_fp8 takes whatever float dtype the checkpoint holds; so does the converter."""
+    src, out = tmp_path / "mixed", tmp_path / f"mixed_{strategy}"
+    src.mkdir()
+    tensors = {"model.layers.0.self_attn.q_proj.weight": I.weights(300, 256, seed=2).to(torch.float16),
+               "model.layers.0.self_attn.o_proj.weight": I.weights(256, 384, seed=3).float() * 1.001,
+               "model.layers.0.mlp.down_proj.weight": I.weights(128, 256, seed=4)}
+    save_file(tensors, str(src / "model.safetensors"), metadata={"format": "pt"})
+    json.dump({"architectures": ["X"]}, open(src / "config.json", "w"))
+    F8.main(["--model-dir", str(src), "--save-dir", str(out), "--strategy", strategy] +
+            (["--block-size", "128", "128"] if strategy == "block" else []))
+    got = load_file(str(out / "model.safetensors"))
+    for k, w in tensors.items():
+        qo, so = {"block": lambda t: C.fp8_block_quant(t, (128, 128), 2), "tensor": lambda t: C.fp8_tensor_quant(t, 2),
+                  "channel": lambda t: C.fp8_channel_quant(t, 2)}[strategy](w)
+        s = got[k.replace(".weight", ".weight_scale_inv" if strategy == "block" else ".weight_scale")]
+        assert got[k].dtype == torch.float8_e4m3fn and torch.equal(got[k].view(torch.uint8), qo), k
+        assert s.shape == so.shape and torch.equal(s.view(torch.int32), so.view(torch.int32)), k
+
+
 @pytest.mark.parametrize("group,sym", [(128, True), (32, True), (128, False)])
 def test_convert_hf_to_int4_direct(ckpt, tmp_path, cuda, group, sym):
     src, tensors = ckpt

@@ -69,3 +69,19 @@ def test_f32_to_bf16_sweep():
     x = x[~x.isnan()]
     want = x.to(torch.bfloat16).view(torch.int16)
     assert torch.equal(C.f32_to_bf16(x).view(torch.int16), want)
+
+
+def test_f32_to_f16_sweep_and_every_boundary():
+    g = torch.Generator().manual_seed(2)
+    bits = torch.randint(-2 ** 31, 2 ** 31 - 1, (1 << 22,), generator=g, dtype=torch.int64).to(torch.int32)
+    # every finite fp16 value, the midpoint to its upper neighbour, and one fp32 ulp either side of both:
+    # all rounding boundaries, the subnormal range, the step to infinity at 65520
+    h = torch.arange(0, 0x7C00, dtype=torch.int32).to(torch.int16).view(torch.float16).to(torch.float32)
+    nxt = torch.cat([h[1:], torch.tensor([65536.0])])
+    pts = torch.cat([h, (h + nxt) / 2, torch.tensor([2.0 ** -25, 2.0 ** -26, 65519.99, 65520.0, 1e30, float("inf")])])
+    b = pts.view(torch.int32)
+    pts = torch.cat([pts, (b + 1).view(torch.float32), (b - 1).clamp(min=0).view(torch.float32)])
+    x = torch.cat([bits.view(torch.float32), pts, -pts])
+    x = x[~x.isnan()]
+    assert torch.equal(C.f32_to_f16(x).view(torch.int16), x.to(torch.float16).view(torch.int16))
+    assert C.f32_to_f16(torch.tensor([float("nan")])).isnan().all()

@@ -8,7 +8,7 @@ import torch
 from oracle import c_oracle as C
 from oracle import torch_ref as T
 from tests import wq_inputs as I
-from tests.exact_arith import (BF16_1EM12, F32_1EM10, Fraction, e4m3_code, rn_bf16, rn_e4m3, rn_f32)
+from tests.exact_arith import (BF16_1EM12, F32_1EM10, Fraction, e4m3_code, rn_bf16, rn_e4m3, rn_f32, round_to_format)
 
 E4M3 = torch.float8_e4m3fn
 
@@ -417,3 +417,40 @@ def test_ue8m0_differs_from_the_plain_block_scale():
     _, s0 = C.fp8_block_quant(w, (128, 128), 1)
     _, s3 = C.fp8_block_quant(w, (128, 128), 3)
     assert (s3 >= s0).all() and not torch.equal(s0, s3)
+
+
+@pytest.mark.parametrize("dt", [torch.float16, torch.float32])
+@pytest.mark.parametrize("device_arith", [False, True])
+def test_channel_and_tensor_forms_other_dtypes(dt, device_arith):
+    """fp16 / fp32 weights: the C oracle against the op-for-op torch restatement - the per-tensor quotient takes the
+    weight's dtype (and, in the GPU evaluation, so does the divisor); rows are blocks of one row."""
+    g = torch.Generator().manual_seed(3)
+    for shape, std in (((37, 200), 0.05), ((128, 130), 1.0), ((5, 1000), 1e-3)):
+        w = (torch.randn(shape, generator=g) * std).to(dt)
+        for view in (lambda t: t, lambda t: t.t()):
+            x = view(w)
+            q, s = C.fp8_tensor_quant(x, 2 if device_arith else 0)
+            qr, sr = T.tensor_fp8_ref(x, device_arith)
+            assert torch.equal(q, qr.view(torch.uint8)) and torch.equal(s.view(torch.int32), sr.view(torch.int32))
+            q, s = C.fp8_channel_quant(x, 2 if device_arith else 0)
+            qr, sr = T.channel_fp8_ref(x, device_arith)
+            assert torch.equal(q, qr.view(torch.uint8)) and torch.equal(s.view(torch.int32), sr.view(torch.int32))
+    # fp32 weights round once: the per-tensor form equals one block spanning the tensor
+    w = (torch.randn(64, 96, generator=g) * 0.3)
+    q, s = C.fp8_tensor_quant(w, 0)
+    qb, sb = C.fp8_block_quant(w, (64, 96), 0)
+    assert torch.equal(q, qb) and torch.equal(s.view(torch.int32), sb.view(-1).view(torch.int32))
+    # fp16 weights round twice.  Exact rational arithmetic on every element: scale = RN32(amax / 448),
+    # code = e4m3(RN16(RN32(x / scale))); the sample must contain elements on which one rounding would differ
+    f16 = lambda v: round_to_format(v, 11, -14)
+    h = (torch.randn(1, 3000, generator=g) * 30).clamp(-100, 100).to(torch.float16)
+    h[0, 0] = 100.25                                            # amax
+    q, sc = C.fp8_tensor_quant(h, 0)
+    scale = rn_f32(Fraction(100.25) / 448)
+    assert Fraction(sc.item()) == scale
+    differ = 0
+    for v, code in zip(h[0].tolist(), q[0].tolist()):
+        q32 = rn_f32(Fraction(v) / scale)
+        assert code == e4m3_code(rn_e4m3(f16(q32)), negative_zero=(v < 0 and f16(q32) == 0)), v
+        differ += rn_e4m3(f16(q32)) != rn_e4m3(q32)
+    assert differ > 0
