@@ -159,8 +159,8 @@ int wq_fp8_block_quant_dequant(const void *x, int64_t M, int64_t N, int64_t sx_m
 
 /* ---------------------------------------------------------------------------------------------
  * e4m3fn [M,N] contiguous + fp32 scale [ceil(M/block), ceil(N/block)] contiguous -> y [M,N]
- * contiguous, of type out_dtype: WQ_DTYPE_BF16 (product rounded once, RNE) or WQ_DTYPE_F32 (the fp32
- * product itself).  Replaces weight_dequant (tools/fp8_cast_bf16.py:31-41), which asserts the same
+ * contiguous, of type out_dtype: WQ_DTYPE_BF16 or WQ_DTYPE_F16 (product rounded once, RNE; fp16 with
+ * mode WQ_DEQ_MODE_F32SCALE only) or WQ_DTYPE_F32 (the fp32 product itself).  Replaces weight_dequant (tools/fp8_cast_bf16.py:31-41), which asserts the same
  * contiguity and writes torch's default dtype (bf16 in the tool, :45). */
 int wq_fp8_block_dequant(const void *x, const float *s, void *y, int out_dtype, int64_t M, int64_t N,
                          int block, int mode, void *stream);

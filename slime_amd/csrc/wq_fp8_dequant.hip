@@ -62,6 +62,27 @@ __device__ __forceinline__ u32x2 dequant4(uint32_t codes, float sc)
     return o;
 }
 
+// RNE fp32 -> fp16 for two values packed in a dword (two v_cvt_f16_f32; the packed conversion rounds toward zero).
+// The empty asm keeps the fp32 product a value of its own: left alone, the compiler folds "convert(a * b)" into
+// v_fma_mixlo_f16 a, b, 0, which rounds the exact product once (the reference rounds it to fp32 first) and turns a
+// product of -0 into +0.
+__device__ __forceinline__ uint32_t pack_f16x2(float a, float b)
+{
+    asm volatile("" : "+v"(a), "+v"(b));
+    const _Float16 ha = (_Float16)a, hb = (_Float16)b;
+    return (uint32_t)__builtin_bit_cast(uint16_t, ha) | ((uint32_t)__builtin_bit_cast(uint16_t, hb) << 16);
+}
+
+__device__ __forceinline__ u32x2 dequant4_f16(uint32_t codes, float sc)
+{
+    f32x2 lo = __builtin_amdgcn_cvt_pk_f32_fp8((int)codes, false);
+    f32x2 hi = __builtin_amdgcn_cvt_pk_f32_fp8((int)codes, true);
+    u32x2 o;
+    o.x = pack_f16x2(lo.x * sc, lo.y * sc);
+    o.y = pack_f16x2(hi.x * sc, hi.y * sc);
+    return o;
+}
+
 __device__ __forceinline__ f32x4 dequant4_f32(uint32_t codes, float sc)
 {
     f32x2 lo = __builtin_amdgcn_cvt_pk_f32_fp8((int)codes, false);
@@ -69,7 +90,8 @@ __device__ __forceinline__ f32x4 dequant4_f32(uint32_t codes, float sc)
     return (f32x4){lo.x * sc, lo.y * sc, hi.x * sc, hi.y * sc};
 }
 
-// OUT: WQ_DTYPE_BF16 (the reference tool's default dtype) or WQ_DTYPE_F32 (the un-rounded product).
+// OUT: WQ_DTYPE_BF16 (the reference tool's default dtype), WQ_DTYPE_F16 (product rounded once to fp16) or WQ_DTYPE_F32
+// (the un-rounded product).
 // GROUPED: 0 = one tensor in the kernel arguments, 1 = descriptor array + prefix sums (the owner of a work item is
 // searched), 2 = one pre-resolved descriptor per work item (a single scalar load, no search)
 template <int MODE, int GROUPED, int OUT>
@@ -131,8 +153,9 @@ __global__ __launch_bounds__(256) void fp8_block_dequant_kernel(const DeqArgs a,
             if (!ok[i]) continue;
             if (MODE == WQ_DEQ_MODE_BF16SCALE) sc[i] = u2f(f32_to_bf16_bits(sc[i]) << 16);
             const uint64_t off = (uint64_t)row[i] * N + col[i];
-            if (OUT == WQ_DTYPE_BF16) {
-                const u32x2 a0 = dequant4(v[i].x, sc[i]), a1 = dequant4(v[i].y, sc[i]);
+            if (OUT == WQ_DTYPE_BF16 || OUT == WQ_DTYPE_F16) {
+                const u32x2 a0 = OUT == WQ_DTYPE_BF16 ? dequant4(v[i].x, sc[i]) : dequant4_f16(v[i].x, sc[i]);
+                const u32x2 a1 = OUT == WQ_DTYPE_BF16 ? dequant4(v[i].y, sc[i]) : dequant4_f16(v[i].y, sc[i]);
                 const u32x4 o = {a0.x, a0.y, a1.x, a1.y};
                 stg_nt<u32x4>((uint16_t*)d.y + off, o);
             } else {
@@ -155,6 +178,7 @@ __global__ __launch_bounds__(256) void fp8_block_dequant_kernel(const DeqArgs a,
                 const uint32_t code = x[off];
                 const f32x2 f = __builtin_amdgcn_cvt_pk_f32_fp8((int)code, false);
                 if (OUT == WQ_DTYPE_BF16) ((uint16_t*)d.y)[off] = (uint16_t)(pack_bf16x2(f.x * sc, 0.0f) & 0xFFFFu);
+                else if (OUT == WQ_DTYPE_F16) ((uint16_t*)d.y)[off] = (uint16_t)(pack_f16x2(f.x * sc, 0.0f) & 0xFFFFu);
                 else ((float*)d.y)[off] = f.x * sc;
             }
             c += 4;
@@ -178,6 +202,7 @@ static int launch_deq(const DeqArgs& a, int64_t work, int mode, int out_dtype, h
     const dim3 g = grid_for_items(work);
     if (mode == WQ_DEQ_MODE_F32SCALE) {
         if (out_dtype == WQ_DTYPE_BF16) fp8_block_dequant_kernel<WQ_DEQ_MODE_F32SCALE, GROUPED, WQ_DTYPE_BF16><<<g, 256, kDeqOccupancyPadBytes, st>>>(a, work);
+        else if (out_dtype == WQ_DTYPE_F16) fp8_block_dequant_kernel<WQ_DEQ_MODE_F32SCALE, GROUPED, WQ_DTYPE_F16><<<g, 256, kDeqOccupancyPadBytes, st>>>(a, work);
         else fp8_block_dequant_kernel<WQ_DEQ_MODE_F32SCALE, GROUPED, WQ_DTYPE_F32><<<g, 256, kDeqOccupancyPadBytes, st>>>(a, work);
     } else {
         if (out_dtype == WQ_DTYPE_BF16) fp8_block_dequant_kernel<WQ_DEQ_MODE_BF16SCALE, GROUPED, WQ_DTYPE_BF16><<<g, 256, kDeqOccupancyPadBytes, st>>>(a, work);
@@ -191,7 +216,8 @@ static int check_deq(int64_t block, int mode, int out_dtype)
 {
     if (block <= 0) return WQ_ERR_SHAPE;
     if (mode != WQ_DEQ_MODE_F32SCALE && mode != WQ_DEQ_MODE_BF16SCALE) return WQ_ERR_MODE;
-    if (out_dtype != WQ_DTYPE_BF16 && out_dtype != WQ_DTYPE_F32) return WQ_ERR_MODE;
+    if (out_dtype != WQ_DTYPE_BF16 && out_dtype != WQ_DTYPE_F32 && out_dtype != WQ_DTYPE_F16) return WQ_ERR_MODE;
+    if (out_dtype == WQ_DTYPE_F16 && mode != WQ_DEQ_MODE_F32SCALE) return WQ_ERR_UNSUPPORTED;   // the loader's variant is bf16
     return WQ_OK;
 }
 

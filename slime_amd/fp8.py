@@ -166,6 +166,9 @@ def transform_scale_ue8m0(sf: torch.Tensor, mn: int) -> torch.Tensor:
         "call with transform_ue8m0=False to get the power-of-two scales as float32 (the form hf_checkpoint_saver uses)")
 
 
+_DEQ_OUT_DTYPES = {torch.bfloat16: _lib.DTYPE_BF16, torch.float32: _lib.DTYPE_F32, torch.float16: _lib.DTYPE_F16}
+
+
 def _dequant(x: torch.Tensor, s: torch.Tensor, block_size: int, mode: int, out_dtype: torch.dtype, what: str):
     _lib.require_gpu(x, what)
     assert x.is_contiguous() and s.is_contiguous()
@@ -174,8 +177,8 @@ def _dequant(x: torch.Tensor, s: torch.Tensor, block_size: int, mode: int, out_d
         raise TypeError(f"{what}: x must hold one-byte e4m3fn codes, got {x.dtype}")
     if s.dtype != torch.float32:
         raise TypeError(f"{what}: scale must be float32, got {s.dtype}")
-    if out_dtype not in (torch.bfloat16, torch.float32):
-        raise TypeError(f"{what}: output dtype {out_dtype} is not supported (bfloat16 or float32)")
+    if out_dtype not in _DEQ_OUT_DTYPES or (out_dtype == torch.float16 and mode != _lib.DEQ_MODE_F32SCALE):
+        raise TypeError(f"{what}: output dtype {out_dtype} is not supported (bfloat16, float16 or float32)")
     M, N = x.shape
     if tuple(s.shape) != (ceildiv(M, block_size), ceildiv(N, block_size)):
         raise ValueError(f"{what}: scale shape {tuple(s.shape)} does not match x {tuple(x.shape)} / {block_size}")
@@ -184,15 +187,14 @@ def _dequant(x: torch.Tensor, s: torch.Tensor, block_size: int, mode: int, out_d
         with torch.cuda.device(x.device):
             rc = _lib.load().wq_fp8_block_dequant(
                 x.data_ptr(), s.data_ptr(), y.data_ptr(),
-                _lib.DTYPE_BF16 if out_dtype == torch.bfloat16 else _lib.DTYPE_F32,
-                M, N, int(block_size), mode, _lib.stream_ptr(x.device))
+                _DEQ_OUT_DTYPES[out_dtype], M, N, int(block_size), mode, _lib.stream_ptr(x.device))
         _lib.check(rc, what)
     return y
 
 
 def weight_dequant(x: torch.Tensor, s: torch.Tensor, block_size: int = 128) -> torch.Tensor:
     """y = (f32(x) * s[block]) in torch's default dtype (tools/fp8_cast_bf16.py:31-41; the tool sets the
-    default dtype to bfloat16 at :45, callers that have not get float32, as with the reference)."""
+    default dtype to bfloat16 at :45, callers that have not get float32 - or float16 -, as with the reference)."""
     return _dequant(x, s, block_size, _lib.DEQ_MODE_F32SCALE, torch.get_default_dtype(), "weight_dequant")
 
 

@@ -198,3 +198,24 @@ def test_ue8m0_requests_are_not_ignored():
 
 def lib_rc(name, *args):
     return getattr(_lib.load(), name)(*args)
+
+
+def test_no_mixed_precision_fma_in_the_dequantiser(tmp_path):
+    """`(half)(a * b)` invites the compiler to emit v_fma_mixlo_f16 a, b, 0: one rounding of the exact product where the
+    reference rounds to fp32 first, and +0 for a product of -0.  The kernel source blocks that fusion; this compiles the
+    file to assembly with the library's own flags and checks that none of it came back."""
+    import re
+    import shutil
+    import subprocess
+
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(hipcc):
+        pytest.skip("no hipcc")
+    csrc = os.path.join(ROOT, "slime_amd", "csrc")
+    flags = re.search(r"^HIPFLAGS \?= (.*?)\n(?!\s)", open(os.path.join(csrc, "Makefile")).read(), re.S | re.M).group(1)
+    flags = flags.replace("\\\n", " ").replace("$(ARCH)", "gfx950").split()
+    out = tmp_path / "deq.s"
+    subprocess.check_call([hipcc, *flags, "-I", os.path.join(ROOT, "include"), "-S", "--cuda-device-only", "-o", str(out),
+                           os.path.join(csrc, "wq_fp8_dequant.hip")], stderr=subprocess.DEVNULL)
+    asm = out.read_text()
+    assert "v_cvt_f16_f32" in asm and "fma_mix" not in asm and "mad_mix" not in asm

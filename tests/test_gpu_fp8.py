@@ -222,6 +222,27 @@ def test_dequant_shapes(cuda, shape):
     assert I.same_bits(y32.cpu(), x.view(E4M3).float() * T._expand_scale(s, shape[0], shape[1], 128))
 
 
+def test_dequant_into_half_precision(cuda):
+    """torch's default dtype float16: the reference stores the fp32 product to an fp16 tensor - one RNE rounding, with
+    overflow to infinity and gradual underflow (scales up to 1e3 and down to 1e-9 reach both ends)."""
+    for shape in ((256, 256), (300, 200), (17, 1040), (5, 1000)):
+        x = I.fp8_codes(*shape, seed=shape[0] + 1)
+        s = I.log_uniform_scales(-(-shape[0] // 128), -(-shape[1] // 128), seed=shape[1], lo=1e-9, hi=1e3)
+        s[0, 0], s[-1, -1] = 1e3, 3e-7                       # overflow to infinity / fp16 subnormals for certain
+        torch.set_default_dtype(torch.float16)
+        try:
+            y = slime_amd.weight_dequant(x.to(cuda).view(E4M3), s.to(cuda))
+        finally:
+            torch.set_default_dtype(torch.float32)
+        want = C.f32_to_f16(C.e4m3fn_to_f32(x) * T._expand_scale(s, shape[0], shape[1], 128))
+        assert y.dtype == torch.float16 and I.same_bits(y.cpu(), want)
+        assert want.isinf().any() and (want.float().abs() < 6e-5).any()
+        # torch's own conversion on the GPU as a second witness
+        assert I.same_bits(y, (x.to(cuda).view(E4M3).float() * T._expand_scale(s, shape[0], shape[1], 128).to(cuda)).half())
+    with pytest.raises(TypeError):
+        slime_amd.fp8._dequant(x.to(cuda).view(E4M3), s.to(cuda), 128, 1, torch.float16, "t")
+
+
 def test_dequant_reference_kat(cuda):
     # tests/test_hf_to_megatron.py:345-358 of the reference
     w = torch.linspace(-2, 2, 128 * 128).view(128, 128).to(E4M3)
