@@ -87,6 +87,7 @@ KERNEL_SOURCES = {
     "fp8_block_dequant": ("wq_fp8_dequant.hip", "wq_common.h"),
     "int4_dequant": ("wq_int4_dequant.hip", "wq_common.h"),
     "delta_xor": ("wq_delta.hip", "wq_common.h"),
+    "fp8_fake_quant": ("wq_fp8_fake.hip", "wq_common.h"),
 }
 
 
