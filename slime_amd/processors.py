@@ -138,8 +138,11 @@ def quantize_params_fp8(args, megatron_name, converted_named_params, quantizatio
 
 _GROUP_TABLES: OrderedDict = OrderedDict()
 _GROUP_LOCK = threading.Lock()
-_GROUP_STATS = {"builds": 0, "hits": 0}
-_GROUP_MAX = 4096
+_GROUP_STATS = {"builds": 0, "hits": 0, "bytes": 0}
+# The cache is bounded by the device memory its tables take, not by a count: an MoE model presents one gate/up pair per
+# expert and layer (6 144 for 48 x 128 experts, 12 KiB of table each) in the same order on every sync, and a
+# least-recently-used list shorter than that cycle would miss every time.
+_GROUP_MAX_BYTES = 512 << 20
 
 
 def plan_cache_info() -> dict:
@@ -172,10 +175,13 @@ def _group_cast(weights, block_size):
         table, _, _ = tile_table(rows, bm, bn)
         entry = (table.contiguous().to(device), table.shape[0], layout, off)
         with _GROUP_LOCK:
+            if key not in _GROUP_TABLES:
+                _GROUP_STATS["bytes"] += entry[0].numel() * 8
             _GROUP_TABLES[key] = entry
             _GROUP_STATS["builds"] += 1
-            while len(_GROUP_TABLES) > _GROUP_MAX:
-                _GROUP_TABLES.popitem(last=False)
+            while _GROUP_STATS["bytes"] > _GROUP_MAX_BYTES and len(_GROUP_TABLES) > 1:
+                _, old = _GROUP_TABLES.popitem(last=False)
+                _GROUP_STATS["bytes"] -= old[0].numel() * 8
     table, n_tiles, layout, total = entry
     flat = torch.empty(total, dtype=torch.uint8, device=device)
     with torch.cuda.device(device):
