@@ -505,7 +505,9 @@ def bench_delta(dev, steps, warmup):
     assert np.array_equal(diffs[5].cpu().numpy(), want) and np.array_equal(olds[5].cpu().numpy(), check_new)
     assert results[5].tolist() == [changed, int(delta_ref.adler32_ref(check_new), 16)] and changed == 4096
     nbytes = sum(nw.numel() for nw in news)
-    out = {"workload": "Qwen3-4B-shaped state dict (252 bf16 tensors, 7.27 GB) against its snapshot in HBM: xor diff, "
+    xxh3 = _bench_xxh3(news, steps, warmup)
+    out = {"xxh3_128": xxh3,
+           "workload": "Qwen3-4B-shaped state dict (252 bf16 tensors, 7.27 GB) against its snapshot in HBM: xor diff, "
                        "changed-byte count, adler32, snapshot update; two launches for the whole bucket",
            "tensors": len(news), "weight_GB": nbytes / 1e9, "kernel_ms": ev_ms, "wall_ms": wall_ms,
            "weight_GBps": nbytes / ev_ms / 1e6, "algo_GBps": 4 * nbytes / ev_ms / 1e6,
@@ -513,6 +515,36 @@ def bench_delta(dev, steps, warmup):
     del news, olds, plan
     torch.cuda.empty_cache()
     return out
+
+
+def _bench_xxh3(news, steps, warmup):
+    """The digest the reference's delta publisher attaches by default, over the same state dict: two launches (block sums
+    at memory speed, then one scramble chain per tensor), against the xxhash package on the host for one tensor."""
+    import torch
+
+    from slime_amd import delta
+
+    def run():
+        delta.xxh3_128_many(news)           # includes the table upload and the read-back of 252 digests
+
+    wall_ms, ev_ms, _ = _time_launches(run, max(steps // 4, 3), 1)
+    nbytes = sum(nw.numel() for nw in news)
+    rec = {"workload": "xxh3-128 of every tensor of the same state dict (read once; 64 bytes of block sums per KiB, then a "
+                       "sequential chain of 48 640 blocks for the largest tensor)",
+           "ms": ev_ms, "wall_ms": wall_ms, "weight_GBps": nbytes / ev_ms / 1e6, "hbm_frac": (nbytes * 17 / 16) / ev_ms / 1e6 / HBM_PEAK_GBS}
+    try:
+        import xxhash
+
+        got = delta.xxh3_128(news[4])
+        host = news[4].cpu().numpy().tobytes()
+        t0 = time.perf_counter()
+        want = xxhash.xxh3_128(host).hexdigest()
+        rec["host_one_thread_GBps"] = len(host) / (time.perf_counter() - t0) / 1e9
+        assert got == want
+        rec["parity"] = "digest of a 49.8 MB tensor equals xxhash.xxh3_128 on the host"
+    except ImportError:
+        rec["parity"] = "xxhash package not installed: not checked in this run"
+    return rec
 
 
 def bench_single_tensor_forms(dev, steps, warmup):

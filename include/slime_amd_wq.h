@@ -32,7 +32,7 @@
 extern "C" {
 #endif
 
-#define WQ_ABI_VERSION 14
+#define WQ_ABI_VERSION 15
 
 enum {
     WQ_OK = 0,
@@ -397,6 +397,29 @@ typedef struct wq_delta_chunk_item {
 } wq_delta_chunk_item;
 int wq_delta_xor_items(const wq_delta_chunk_item *items, int64_t n_items, const wq_delta_desc *descs, int n_desc,
                        int write_diff, int update_old, void *stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * XXH3-128 (seed 0) of n > 240 bytes in device memory: the digest checksum("xxh3-128", new) attaches to every
+ * changed tensor of a published delta (slime/utils/disk_delta.py:40-58; the default of
+ * --update-weight-delta-checksum, slime/utils/arguments.py:186-188), computed where the tensor lives instead of
+ * after a copy to the host.  digest: DEVICE uint64[2] = {low64, high64}; the reference's hexdigest() is
+ * high64 then low64, most significant byte first.  workspace: DEVICE, wq_xxh3_workspace_bytes(n) bytes
+ * (64 per KiB of input), 16-byte aligned, overwritten.  Any alignment of `data` (16-byte aligned inputs take
+ * the fast path).  n <= 240 (XXH3's short-input forms) returns WQ_ERR_UNSUPPORTED: hash those on the host. */
+int64_t wq_xxh3_workspace_bytes(int64_t n);
+int wq_xxh3_128(const void *data, int64_t n, uint64_t *workspace, uint64_t *digest, void *stream);
+
+/* Many tensors, two launches.  `descs` DEVICE array; item_start DEVICE int64[n_desc+1], exclusive prefix sum of
+ * ceil(((n - 1) / 1024) / 16) per tensor (work items of 16 KiB).  Tensors of 240 bytes or less are skipped
+ * (their digest slot is left untouched). */
+typedef struct wq_xxh3_desc {
+    const void *data;
+    int64_t n;
+    uint64_t *sums;    /* this tensor's workspace: wq_xxh3_workspace_bytes(n) bytes, 16-byte aligned */
+    uint64_t *digest;  /* uint64[2] */
+} wq_xxh3_desc;
+int wq_xxh3_128_grouped(const wq_xxh3_desc *descs, const int64_t *item_start, int n_desc, int64_t total_items,
+                        void *stream);
 
 /* ---------------------------------------------------------------------------------------------
  * Self-checks and calibration helpers (used by the test-suite and the benchmark, not by callers).

@@ -15,7 +15,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libslime_amd_wq.so")
 
-ABI_VERSION = 14
+ABI_VERSION = 15
 
 # selectors (mirrors of the header's enums)
 DTYPE_BF16, DTYPE_F32, DTYPE_F16, DTYPE_F64 = 0, 1, 2, 3
@@ -41,6 +41,9 @@ SIGNATURES = {
     "wq_fp8_block_quant_any": [_vp, _int, _i64, _i64, _i64, _i64, _vp, _i64, _vp, _int, _int, _int, _vp],
     "wq_fp8_row_quant": [_vp, _i64, _i64, _i64, _i64, _vp, _i64, _vp, _int, _vp],
     "wq_fp8_tensor_quant": [_vp, _i64, _i64, _i64, _i64, _vp, _i64, _vp, _vp, _int, _vp],
+    "wq_xxh3_workspace_bytes": [_i64],
+    "wq_xxh3_128": [_vp, _i64, _vp, _vp, _vp],
+    "wq_xxh3_128_grouped": [_vp, _vp, _int, _i64, _vp],
     "wq_fp8_tensor_quant_any": [_vp, _int, _i64, _i64, _i64, _i64, _vp, _i64, _vp, _vp, _int, _vp],
     "wq_fp8_block_dequant": [_vp, _vp, _vp, _int, _i64, _i64, _int, _int, _vp],
     "wq_fp8_block_quant_dequant": [_vp, _i64, _i64, _i64, _i64, _vp, _i64, _vp, _int, _int, _int, _vp],
@@ -100,7 +103,7 @@ def load() -> ctypes.CDLL:
                 raise WqLibraryError(f"{LIB_PATH} does not export {name}; rebuild the library") from exc
             fn.argtypes = argtypes
             fn.restype = (ctypes.c_char_p if name == "wq_error_string"
-                          else _i64 if name == "wq_delta_workspace_bytes" else _int)
+                          else _i64 if name in ("wq_delta_workspace_bytes", "wq_xxh3_workspace_bytes") else _int)
         if lib.wq_abi_version() != ABI_VERSION:
             raise WqLibraryError(f"ABI mismatch: library {lib.wq_abi_version()}, binding {ABI_VERSION}; rebuild")
         _lib = lib

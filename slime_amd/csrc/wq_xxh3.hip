@@ -1,0 +1,288 @@
+// XXH3-128 (seed 0, default secret) of tensors in HBM, for gfx950: the digest the delta publisher attaches to every
+// changed tensor (checksum("xxh3-128", new), slime/utils/disk_delta.py:40-58 - the default of
+// --update-weight-delta-checksum).  The reference hashes on the host, which means copying every changed tensor there;
+// here the tensor stays where it is and sixteen bytes come back.
+//
+// XXH3's long-input form keeps eight 64-bit accumulators.  A 1 KiB block adds, for each of its sixteen 64-byte
+// stripes, lo32(d ^ k) * hi32(d ^ k) of the stripe's word i to accumulator i and word i ^ 1 itself to it - a plain sum
+// mod 2^64, in any order - and only then are the accumulators scrambled (xor-shift, xor, multiply): the one step that
+// makes blocks sequential.  So the work splits in two:
+//   xxh3_block_sums_kernel   the eight sums of every block, at memory speed: a wavefront takes a block with one
+//                            16-byte load per lane (lane l holds words 2j, 2j+1 of stripe l / 4, j = l % 4), multiplies
+//                            in place and adds across the sixteen lanes that share j; 64 bytes of sums per KiB.
+//   xxh3_chain_kernel        per tensor, eight lanes walk acc <- scramble(acc + sums[k]) (about 60 clocks a block), add
+//                            the tail - the stripes of the last partial block and the last 64 bytes, read straight from
+//                            the tensor - and one lane folds the accumulators into the two 64-bit halves.
+// Inputs of 240 bytes or less use XXH3's short forms, which are not provided (the caller hashes those on the host).
+
+#include "wq_common.h"
+
+namespace wq {
+
+__constant__ uint8_t kXxh3Secret[192] = {
+    0xb8, 0xfe, 0x6c, 0x39, 0x23, 0xa4, 0x4b, 0xbe, 0x7c, 0x01, 0x81, 0x2c, 0xf7, 0x21, 0xad, 0x1c,
+    0xde, 0xd4, 0x6d, 0xe9, 0x83, 0x90, 0x97, 0xdb, 0x72, 0x40, 0xa4, 0xa4, 0xb7, 0xb3, 0x67, 0x1f,
+    0xcb, 0x79, 0xe6, 0x4e, 0xcc, 0xc0, 0xe5, 0x78, 0x82, 0x5a, 0xd0, 0x7d, 0xcc, 0xff, 0x72, 0x21,
+    0xb8, 0x08, 0x46, 0x74, 0xf7, 0x43, 0x24, 0x8e, 0xe0, 0x35, 0x90, 0xe6, 0x81, 0x3a, 0x26, 0x4c,
+    0x3c, 0x28, 0x52, 0xbb, 0x91, 0xc3, 0x00, 0xcb, 0x88, 0xd0, 0x65, 0x8b, 0x1b, 0x53, 0x2e, 0xa3,
+    0x71, 0x64, 0x48, 0x97, 0xa2, 0x0d, 0xf9, 0x4e, 0x38, 0x19, 0xef, 0x46, 0xa9, 0xde, 0xac, 0xd8,
+    0xa8, 0xfa, 0x76, 0x3f, 0xe3, 0x9c, 0x34, 0x3f, 0xf9, 0xdc, 0xbb, 0xc7, 0xc7, 0x0b, 0x4f, 0x1d,
+    0x8a, 0x51, 0xe0, 0x4b, 0xcd, 0xb4, 0x59, 0x31, 0xc8, 0x9f, 0x7e, 0xc9, 0xd9, 0x78, 0x73, 0x64,
+    0xea, 0xc5, 0xac, 0x83, 0x34, 0xd3, 0xeb, 0xc3, 0xc5, 0x81, 0xa0, 0xff, 0xfa, 0x13, 0x63, 0xeb,
+    0x17, 0x0d, 0xdd, 0x51, 0xb7, 0xf0, 0xda, 0x49, 0xd3, 0x16, 0x55, 0x26, 0x29, 0xd4, 0x68, 0x9e,
+    0x2b, 0x16, 0xbe, 0x58, 0x7d, 0x47, 0xa1, 0xfc, 0x8f, 0xf8, 0xb8, 0xd1, 0x7a, 0xd0, 0x31, 0xce,
+    0x45, 0xcb, 0x3a, 0x8f, 0x95, 0x16, 0x04, 0x28, 0xaf, 0xd7, 0xfb, 0xca, 0xbb, 0x4b, 0x40, 0x7e,
+};
+
+constexpr uint64_t kP32_1 = 0x9E3779B1ull, kP32_2 = 0x85EBCA77ull, kP32_3 = 0xC2B2AE3Dull;
+constexpr uint64_t kP64_1 = 0x9E3779B185EBCA87ull, kP64_2 = 0xC2B2AE3D27D4EB4Full, kP64_3 = 0x165667B19E3779F9ull;
+constexpr uint64_t kP64_4 = 0x85EBCA77C2B2AE63ull, kP64_5 = 0x27D4EB2F165667C5ull, kMx1 = 0x165667919E3779F9ull;
+constexpr int kXxhBlock = 1024, kXxhStripe = 64;
+constexpr int kXxhBlocksPerItem = 16;      // a work item of the sums kernel: 16 KiB, four blocks per wavefront
+constexpr int kXxhItemsPerXcdRun = 32;
+
+struct Xxh3Args {
+    wq_xxh3_desc d;
+    const wq_xxh3_desc* descs;
+    const int64_t* item_start;
+    int32_t n_desc;
+};
+
+// little-endian u64 of the secret at any byte offset
+__device__ __forceinline__ uint64_t secret64(int off)
+{
+    uint64_t v = 0;
+#pragma unroll
+    for (int b = 0; b < 8; ++b) v |= (uint64_t)kXxh3Secret[off + b] << (8 * b);
+    return v;
+}
+
+__device__ __forceinline__ uint64_t load64_bytes(const uint8_t* p)
+{
+    uint64_t v = 0;
+#pragma unroll
+    for (int b = 0; b < 8; ++b) v |= (uint64_t)p[b] << (8 * b);
+    return v;
+}
+
+__device__ __forceinline__ uint64_t mul_halves(uint64_t x) { return (x & 0xFFFFFFFFull) * (x >> 32); }
+
+__device__ __forceinline__ uint64_t shfl_xor_u64(uint64_t v, int mask)
+{
+    const uint32_t lo = (uint32_t)__shfl_xor((int)(uint32_t)v, mask), hi = (uint32_t)__shfl_xor((int)(uint32_t)(v >> 32), mask);
+    return ((uint64_t)hi << 32) | lo;
+}
+
+// v + (v of the lane 4 further on in the 16-lane row) + ... : the sum over the four lanes of a row that share lane % 4,
+// by two rotations of the row (DPP row_ror:4, row_ror:8)
+__device__ __forceinline__ uint64_t row_sum_stride4_u64(uint64_t v)
+{
+    uint32_t lo = (uint32_t)v, hi = (uint32_t)(v >> 32);
+    v += ((uint64_t)dpp_u32<0x124>(hi) << 32) | dpp_u32<0x124>(lo);
+    lo = (uint32_t)v, hi = (uint32_t)(v >> 32);
+    v += ((uint64_t)dpp_u32<0x128>(hi) << 32) | dpp_u32<0x128>(lo);
+    return v;
+}
+
+__device__ __forceinline__ int64_t scrambled_blocks(int64_t n) { return (n - 1) / kXxhBlock; }
+
+template <int GROUPED>
+__global__ __launch_bounds__(256) void xxh3_block_sums_kernel(const Xxh3Args a, const int64_t total_items)
+{
+    const int64_t slot = (int64_t)blockIdx.x + (int64_t)blockIdx.y * gridDim.x;
+    if (slot >= total_items) return;
+    const int64_t item = xcd_chunked_item(slot, total_items, kXxhItemsPerXcdRun);
+    wq_xxh3_desc d;
+    int64_t local = item;
+    if (GROUPED) {
+        const int di = find_owner(a.item_start, a.n_desc, item, total_items);
+        d = a.descs[di];
+        local = item - a.item_start[di];
+    } else {
+        d = a.d;
+    }
+    const int64_t nb = scrambled_blocks(d.n);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const int stripe = lane >> 2, pair = lane & 3;
+    // stripe s reads the secret at 8 s: word i of the stripe meets the secret's u64 number s + i
+    const uint64_t k0 = secret64(8 * (stripe + 2 * pair)), k1 = secret64(8 * (stripe + 2 * pair + 1));
+    const uint8_t* base = (const uint8_t*)d.data;
+    const bool aligned = ((uintptr_t)base & 15) == 0;
+    constexpr int PER_WAVE = kXxhBlocksPerItem / 4;
+
+    uint64_t d0[PER_WAVE], d1[PER_WAVE];
+#pragma unroll
+    for (int i = 0; i < PER_WAVE; ++i) {
+        // blocks past the end re-read the tensor's first block instead of branching around the load
+        const int64_t b = local * kXxhBlocksPerItem + wave + 4 * i;
+        const uint8_t* p = base + (b < nb ? b : 0) * kXxhBlock + lane * 16;
+        if (aligned) {
+            const u32x4 v = ldg_nt<u32x4>(p);
+            d0[i] = ((uint64_t)v.y << 32) | v.x;
+            d1[i] = ((uint64_t)v.w << 32) | v.z;
+        } else {
+            d0[i] = load64_bytes(p);
+            d1[i] = load64_bytes(p + 8);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < PER_WAVE; ++i) {
+        const int64_t b = local * kXxhBlocksPerItem + wave + 4 * i;
+        uint64_t s0 = d1[i] + mul_halves(d0[i] ^ k0);      // into accumulator 2 * pair
+        uint64_t s1 = d0[i] + mul_halves(d1[i] ^ k1);      // into accumulator 2 * pair + 1
+        s0 = row_sum_stride4_u64(s0);                       // stripes 4r .. 4r+3 of row r
+        s1 = row_sum_stride4_u64(s1);
+#pragma unroll
+        for (int m = 16; m < 64; m <<= 1) {                 // the four rows
+            s0 += shfl_xor_u64(s0, m);
+            s1 += shfl_xor_u64(s1, m);
+        }
+        if (lane < 4 && b < nb) {
+            uint64_t* out = d.sums + b * 8 + 2 * lane;
+            out[0] = s0;
+            out[1] = s1;
+        }
+    }
+}
+
+__device__ __forceinline__ uint64_t mul128_fold64(uint64_t x, uint64_t y) { return (x * y) ^ __umul64hi(x, y); }
+
+__device__ __forceinline__ uint64_t avalanche(uint64_t h)
+{
+    h ^= h >> 37;
+    h *= kMx1;
+    return h ^ (h >> 32);
+}
+
+// one wavefront per tensor; lanes 0..7 own one accumulator each
+__global__ __launch_bounds__(64) void xxh3_chain_kernel(const wq_xxh3_desc single, const wq_xxh3_desc* __restrict__ descs,
+                                                        int n_desc)
+{
+    const int t = blockIdx.x;
+    if (t >= n_desc) return;
+    const wq_xxh3_desc d = descs ? descs[t] : single;
+    if (d.n <= 240) return;                   // short forms: not provided (rejected on the host for the single form)
+    const int lane = threadIdx.x, i = lane & 7;
+    const uint64_t init[8] = {kP32_3, kP64_1, kP64_2, kP64_3, kP64_4, kP32_2, kP64_5, kP32_1};
+    uint64_t acc = init[0];
+#pragma unroll
+    for (int k = 1; k < 8; ++k) acc = i == k ? init[k] : acc;
+    const uint64_t scramble_key = secret64(192 - kXxhStripe + 8 * i);
+    const int64_t nb = scrambled_blocks(d.n);
+    const uint64_t* s = d.sums + i;
+
+    // The walk.  A block costs about 55 clocks of dependent arithmetic and a load from HBM takes well over a thousand,
+    // so the sums are fetched 32 blocks ahead: four batches of eight are in flight, and the batch just consumed is
+    // refilled at once with the blocks 32 further on.
+    constexpr int U = 8, DEPTH = 4;
+    uint64_t ring[DEPTH][U];
+    int64_t k = 0;
+    if (nb >= DEPTH * U) {
+#pragma unroll
+        for (int b = 0; b < DEPTH; ++b)
+#pragma unroll
+            for (int u = 0; u < U; ++u) ring[b][u] = s[(b * U + u) * 8];
+        for (; k + 2 * DEPTH * U <= nb; k += DEPTH * U) {
+#pragma unroll
+            for (int b = 0; b < DEPTH; ++b) {
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    acc += ring[b][u];
+                    acc = ((acc ^ (acc >> 47)) ^ scramble_key) * kP32_1;
+                }
+#pragma unroll
+                for (int u = 0; u < U; ++u) ring[b][u] = s[(k + (DEPTH + b) * U + u) * 8];
+            }
+        }
+#pragma unroll
+        for (int b = 0; b < DEPTH; ++b)
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                acc += ring[b][u];
+                acc = ((acc ^ (acc >> 47)) ^ scramble_key) * kP32_1;
+            }
+        k += DEPTH * U;
+    }
+    for (; k < nb; ++k) {
+        acc += s[k * 8];
+        acc = ((acc ^ (acc >> 47)) ^ scramble_key) * kP32_1;
+    }
+
+    // the last partial block: its whole stripes, then the last 64 bytes of the input under their own key
+    const uint8_t* data = (const uint8_t*)d.data;
+    const int64_t tail = nb * kXxhBlock;
+    const int n_stripes = (int)(((d.n - 1) - tail) / kXxhStripe);
+    for (int st = 0; st <= n_stripes; ++st) {
+        const bool last = st == n_stripes;
+        const uint8_t* p = last ? data + d.n - kXxhStripe : data + tail + (int64_t)st * kXxhStripe;
+        const uint64_t w = load64_bytes(p + 8 * i);
+        const uint64_t key = secret64(last ? 192 - kXxhStripe - 7 + 8 * i : 8 * st + 8 * i);
+        acc += shfl_xor_u64(w, 1) + mul_halves(w ^ key);
+    }
+
+    // fold: lane 0 collects the eight accumulators
+    uint64_t all[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const uint32_t lo = (uint32_t)__shfl((int)(uint32_t)acc, j), hi = (uint32_t)__shfl((int)(uint32_t)(acc >> 32), j);
+        all[j] = ((uint64_t)hi << 32) | lo;
+    }
+    if (lane == 0) {
+        uint64_t low = (uint64_t)d.n * kP64_1, high = ~((uint64_t)d.n * kP64_2);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            low += mul128_fold64(all[2 * j] ^ secret64(11 + 16 * j), all[2 * j + 1] ^ secret64(11 + 16 * j + 8));
+            high += mul128_fold64(all[2 * j] ^ secret64(192 - kXxhStripe - 11 + 16 * j),
+                                  all[2 * j + 1] ^ secret64(192 - kXxhStripe - 11 + 16 * j + 8));
+        }
+        d.digest[0] = avalanche(low);
+        d.digest[1] = avalanche(high);
+    }
+}
+
+static inline int64_t xxh3_items(int64_t n) { return cdiv64(n > 0 ? (n - 1) / kXxhBlock : 0, kXxhBlocksPerItem); }
+
+}  // namespace wq
+
+using namespace wq;
+
+WQ_EXPORT int64_t wq_xxh3_workspace_bytes(int64_t n) { return n > 0 ? ((n - 1) / kXxhBlock) * 64 + 64 : 64; }
+
+WQ_EXPORT int wq_xxh3_128(const void* data, int64_t n, uint64_t* workspace, uint64_t* digest, void* stream)
+{
+    if (n < 0) return WQ_ERR_SHAPE;
+    if (n <= 240) return WQ_ERR_UNSUPPORTED;
+    if (!data || !workspace || !digest) return WQ_ERR_NULL;
+    if (((uintptr_t)workspace & 15) || ((uintptr_t)digest & 7)) return WQ_ERR_ALIGN;
+    hipStream_t st = (hipStream_t)stream;
+    Xxh3Args a{};
+    a.d = wq_xxh3_desc{data, n, workspace, digest};
+    const int64_t items = xxh3_items(n);
+    if (items) {
+        xxh3_block_sums_kernel<0><<<grid_for_items(items), 256, 0, st>>>(a, items);
+        WQ_LAUNCH_CHECK();
+    }
+    xxh3_chain_kernel<<<1, 64, 0, st>>>(a.d, nullptr, 1);
+    WQ_LAUNCH_CHECK();
+    return WQ_OK;
+}
+
+WQ_EXPORT int wq_xxh3_128_grouped(const wq_xxh3_desc* descs, const int64_t* item_start, int n_desc, int64_t total_items,
+                                  void* stream)
+{
+    if (n_desc < 0 || total_items < 0) return WQ_ERR_SHAPE;
+    if (n_desc == 0) return WQ_OK;
+    if (!descs || !item_start) return WQ_ERR_NULL;
+    hipStream_t st = (hipStream_t)stream;
+    Xxh3Args a{};
+    a.descs = descs;
+    a.item_start = item_start;
+    a.n_desc = n_desc;
+    if (total_items) {
+        xxh3_block_sums_kernel<1><<<grid_for_items(total_items), 256, 0, st>>>(a, total_items);
+        WQ_LAUNCH_CHECK();
+    }
+    xxh3_chain_kernel<<<n_desc, 64, 0, st>>>(wq_xxh3_desc{}, descs, n_desc);
+    WQ_LAUNCH_CHECK();
+    return WQ_OK;
+}

@@ -9,7 +9,9 @@ only the diff of a tensor that did change has to cross PCIe for compression.
 
 ``xor_diff`` / ``overwrite_encode`` / ``checksum`` are the per-tensor operations, ``DeltaEncoder`` the
 snapshot-keeping loop body (``diff_and_compress`` + ``collect`` without the zstd step, which stays on the
-host).  Only the ``adler32`` checksum is computed on the GPU: xxh3-128 and blake3 are sequential by design.
+host).  ``adler32`` comes out of the diff pass itself; ``xxh3-128`` - the reference's default - is computed on the GPU
+too (its per-block sums at memory speed, the sequential scramble chain by eight lanes per tensor: ``xxh3_128`` /
+``xxh3_128_many``), so a changed tensor's bytes never cross PCIe for their digest.  ``blake3`` is a host digest.
 """
 
 from __future__ import annotations
@@ -172,11 +174,63 @@ def overwrite_encode(new: torch.Tensor, old: torch.Tensor) -> torch.Tensor:
     return out
 
 
+XXH3_SHORT = 240     # inputs up to this size use XXH3's short forms: hashed on the host (a few hundred bytes to copy)
+
+
+def _hex128(low: int, high: int) -> str:
+    return f"{high & 0xFFFFFFFFFFFFFFFF:016x}{low & 0xFFFFFFFFFFFFFFFF:016x}"
+
+
+def xxh3_128_many(tensors) -> list:
+    """``xxhash.xxh3_128(bytes of t).hexdigest()`` for every tensor, computed on the GPU with two launches and one
+    synchronisation (tensors of 240 bytes or less: on the host).  -> list of 32-digit hex strings."""
+    flats = [_as_bytes(t, "xxh3_128") for t in tensors]
+    out = [None] * len(flats)
+    big = [i for i, f in enumerate(flats) if f.numel() > XXH3_SHORT]
+    if big:
+        device = flats[big[0]].device
+        lib = _lib.load()
+        ws_off, total_ws, items, n_items = [], 0, [0], 0
+        for i in big:
+            n = flats[i].numel()
+            ws_off.append(total_ws)
+            total_ws += (lib.wq_xxh3_workspace_bytes(n) + 255) // 256 * 256
+            n_items += -(-((n - 1) // 1024) // 16)
+            items.append(n_items)
+        ws = torch.empty(total_ws // 8, dtype=torch.int64, device=device)
+        digests = torch.empty((len(big), 2), dtype=torch.int64, device=device)
+        rows = [[flats[i].data_ptr(), flats[i].numel(), ws.data_ptr() + o, digests.data_ptr() + 16 * k]
+                for k, (i, o) in enumerate(zip(big, ws_off))]
+        descs = torch.tensor(rows, dtype=torch.int64).to(device)
+        starts = torch.tensor(items, dtype=torch.int64).to(device)
+        with torch.cuda.device(device):
+            rc = lib.wq_xxh3_128_grouped(descs.data_ptr(), starts.data_ptr(), len(big), n_items, _lib.stream_ptr(device))
+        _lib.check(rc, "xxh3_128")
+        for i, (low, high) in zip(big, digests.tolist()):
+            out[i] = _hex128(low, high)
+    for i, f in enumerate(flats):
+        if out[i] is None:
+            from .delta_host import host_checksum
+
+            out[i] = host_checksum("xxh3-128", f)
+    return out
+
+
+def xxh3_128(buf: torch.Tensor) -> str:
+    """``checksum("xxh3-128", buf)`` of slime/utils/disk_delta.py:55-58 with the tensor left in device memory."""
+    return xxh3_128_many([buf])[0]
+
+
 def checksum(algorithm: str, buf: torch.Tensor) -> str:
-    """``checksum("adler32", tensor)`` of slime/utils/disk_delta.py:55-58 on the GPU -> 8 hex digits.
-    Other algorithms raise KeyError, as the reference does for unknown names: they are host-side digests."""
+    """``checksum(algorithm, tensor)`` of slime/utils/disk_delta.py:55-58 on the GPU: "adler32" -> 8 hex digits,
+    "xxh3-128" -> 32.  "blake3" is hashed on the host (it needs the ``blake3`` package, as in the reference); unknown
+    names raise KeyError as the reference does."""
+    if algorithm == "xxh3-128":
+        return xxh3_128(buf)
     if algorithm != "adler32":
-        raise KeyError(f"checksum algorithm {algorithm!r} is not computed on the GPU (adler32 only)")
+        from .delta_host import host_checksum
+
+        return host_checksum(algorithm, buf)
     nw = _as_bytes(buf, "checksum")
     result = torch.empty(2, dtype=torch.int64, device=nw.device)
     _xor_pass(nw, nw, None, False, _workspace(nw.numel(), nw.device), result)
@@ -192,7 +246,7 @@ class DeltaEncoder:
     changed; the snapshot is updated either way (``collect``: ``snapshot[name] = new``).  ``changed_bytes`` /
     ``total_bytes`` accumulate as in the reference."""
 
-    def __init__(self, delta_encoding: str = "xor", checksum_algorithm: str = "adler32"):
+    def __init__(self, delta_encoding: str = "xor", checksum_algorithm: str = "xxh3-128"):
         if delta_encoding not in ("xor", "overwrite"):
             raise ValueError(f"unknown delta encoding {delta_encoding!r}")
         self.delta_encoding = delta_encoding
@@ -211,8 +265,13 @@ class DeltaEncoder:
         named_tensors = list(named_tensors)
         diffs, results = xor_diff_many([t for _, t in named_tensors], [self.snapshot[n] for n, _ in named_tensors],
                                        update_snapshot=True)
+        results = results.tolist()
+        digests = {}
+        if self.checksum_algorithm == "xxh3-128":       # one grouped digest pass over the tensors that changed
+            moved = [i for i, (changed, _) in enumerate(results) if changed]
+            digests = dict(zip(moved, xxh3_128_many([named_tensors[i][1] for i in moved])))
         out = []
-        for (name, t), diff, (changed, adler) in zip(named_tensors, diffs, results.tolist()):
+        for i, ((name, t), diff, (changed, adler)) in enumerate(zip(named_tensors, diffs, results)):
             self.total_bytes += diff.numel()
             if not changed:
                 out.append((name, None, None, 0))
@@ -220,10 +279,10 @@ class DeltaEncoder:
             self.changed_bytes += changed
             if self.checksum_algorithm == "adler32":
                 digest = f"{adler:08x}"
+            elif i in digests:
+                digest = digests[i]
             else:
-                from .delta_host import host_checksum
-
-                digest = host_checksum(self.checksum_algorithm, t)
+                digest = checksum(self.checksum_algorithm, t)
             out.append((name, diff, digest, changed))
         return out
 
@@ -253,10 +312,5 @@ class DeltaEncoder:
         if not changed:
             return None, None, 0
         self.changed_bytes += changed
-        if self.checksum_algorithm == "adler32":
-            digest = f"{adler:08x}"
-        else:
-            from .delta_host import host_checksum
-
-            digest = host_checksum(self.checksum_algorithm, nw)
+        digest = f"{adler:08x}" if self.checksum_algorithm == "adler32" else checksum(self.checksum_algorithm, nw)
         return diff, digest, changed

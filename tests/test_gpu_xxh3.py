@@ -1,0 +1,94 @@
+"""XXH3-128 on the GPU against the ``xxhash`` package the reference calls, and against the numpy restatement."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import xxh3_ref as X
+from slime_amd import _lib, delta
+
+pytestmark = pytest.mark.gpu
+xxhash = pytest.importorskip("xxhash")
+
+
+def _lib_hex(t):
+    return xxhash.xxh3_128(t.contiguous().view(torch.uint8).numpy().tobytes()).hexdigest()
+
+
+def _bytes(n, seed):
+    return torch.from_numpy(np.random.default_rng(seed).integers(0, 256, n, dtype=np.uint8))
+
+
+@pytest.mark.parametrize("n", [241, 256, 305, 1023, 1024, 1025, 1088, 1089, 2047, 2048, 2049, 16383, 16384, 16385, 16384 * 3 + 1,
+                               65536 + 64, (1 << 20) - 2, 1 << 20, (1 << 20) + 2, 5 * (1 << 20) + 777])
+def test_every_boundary_against_the_library(cuda, n):
+    x = _bytes(n, n)
+    got = delta.xxh3_128(x.to(cuda))
+    assert got == _lib_hex(x) and got == X.hexdigest(x.numpy())
+
+
+def test_many_tensors_two_launches(cuda):
+    sizes = [0, 5, 240, 241, 1024, 1025, 100000, 49152, 1, (1 << 20) + 3, 16384 * 40, 2 * 2560 * 9728]
+    xs = [_bytes(n, 50 + i) for i, n in enumerate(sizes)]
+    got = delta.xxh3_128_many([x.to(cuda) for x in xs])
+    assert got == [_lib_hex(x) for x in xs]
+    # bf16 weights and views: the digest is over the bytes of the contiguous tensor, as tensor.contiguous().view(uint8) gives
+    g = torch.Generator().manual_seed(1)
+    w = (torch.randn(300, 520, generator=g) * 0.02).to(torch.bfloat16)
+    for view in (lambda t: t, lambda t: t[:, 8:], lambda t: t.t(), lambda t: t[1:]):
+        assert delta.checksum("xxh3-128", view(w.to(cuda))) == _lib_hex(view(w).contiguous())
+
+
+def test_special_contents_and_unaligned_base(cuda):
+    for x in (torch.zeros(70000, dtype=torch.uint8), torch.full((70000,), 255, dtype=torch.uint8),
+              torch.arange(70000, dtype=torch.int32).view(torch.uint8)):
+        assert delta.xxh3_128(x.to(cuda)) == _lib_hex(x)
+    # through the C ABI at byte offsets 1..15 from an aligned base (the Python layer would copy to an aligned buffer)
+    lib = _lib.load()
+    x = _bytes(40000, 9)
+    xg = x.to(cuda)
+    for off in (1, 2, 7, 8, 15):
+        n = 40000 - off - 3
+        ws = torch.empty(lib.wq_xxh3_workspace_bytes(n) // 8, dtype=torch.int64, device=cuda)
+        out = torch.zeros(2, dtype=torch.int64, device=cuda)
+        assert lib.wq_xxh3_128(xg.data_ptr() + off, n, ws.data_ptr(), out.data_ptr(), _lib.stream_ptr(cuda)) == 0
+        low, high = out.tolist()
+        assert delta._hex128(low, high) == _lib_hex(x[off:off + n]), off
+    out = torch.zeros(2, dtype=torch.int64, device=cuda)
+    ws = torch.empty(64, dtype=torch.int64, device=cuda)
+    assert lib.wq_xxh3_128(xg.data_ptr(), 240, ws.data_ptr(), out.data_ptr(), _lib.stream_ptr(cuda)) == -4     # short forms
+    assert lib.wq_xxh3_128(xg.data_ptr(), -1, ws.data_ptr(), out.data_ptr(), _lib.stream_ptr(cuda)) == -2
+    assert lib.wq_xxh3_128(None, 1000, ws.data_ptr(), out.data_ptr(), _lib.stream_ptr(cuda)) == -1
+
+
+def test_large_tensor(cuda):
+    # 1.5 GiB: 1.5 M blocks in one chain; compared with the library on the host
+    g = torch.Generator(device=cuda).manual_seed(3)
+    x = torch.randint(0, 256, (3 << 29,), dtype=torch.uint8, device=cuda, generator=g)
+    assert delta.xxh3_128(x) == _lib_hex(x.cpu())
+
+
+def test_delta_encoder_uses_the_gpu_digest_by_default(cuda, monkeypatch):
+    from slime_amd import delta_host
+
+    def no_host(*a, **k):
+        raise AssertionError("the digest of a long tensor must not be computed on the host")
+
+    monkeypatch.setattr(delta_host, "host_checksum", no_host)
+    g = torch.Generator().manual_seed(9)
+    state = {f"l{i}.weight": torch.randn(64 + i, 96, generator=g).to(torch.bfloat16) for i in range(6)}
+    enc = delta.DeltaEncoder()
+    assert enc.checksum_algorithm == "xxh3-128"            # --update-weight-delta-checksum default
+    for n, t in state.items():
+        enc.capture(n, t.to(cuda))
+    state["l2.weight"] = state["l2.weight"] * 2
+    state["l5.weight"] = state["l5.weight"] + 1
+    out = enc.encode_bucket([(n, t.to(cuda)) for n, t in state.items()])
+    for name, diff, digest, changed in out:
+        if name in ("l2.weight", "l5.weight"):
+            assert changed and digest == _lib_hex(state[name])
+        else:
+            assert diff is None and digest is None and changed == 0
+    state["l0.weight"] = state["l0.weight"] - 1
+    _, digest, changed = enc.encode("l0.weight", state["l0.weight"].to(cuda))
+    assert changed and digest == _lib_hex(state["l0.weight"])
