@@ -16,6 +16,8 @@ fake-quant kernel and then the reference's own chain of tensor ops on the GPU.
 from __future__ import annotations
 
 import math
+import threading
+from collections import OrderedDict
 from typing import Sequence
 
 import torch
@@ -432,23 +434,20 @@ def fake_int4_quantization_ste(x: torch.Tensor, group_size: int) -> torch.Tensor
     return out
 
 
-_STE_TABLES: "OrderedDict" = None
+_STE_TABLES: OrderedDict = OrderedDict()
+_STE_LOCK = threading.Lock()
 
 
 def _ste_table(xs, group_size):
     """Per-item table of the one-launch STE forward for these weights (y as offsets into one output buffer), cached on
     the addresses and shapes of the weights: a layer that calls again with the same parameters builds nothing."""
-    global _STE_TABLES
-    from collections import OrderedDict
-
-    if _STE_TABLES is None:
-        _STE_TABLES = OrderedDict()
     device = xs[0].device
     key = (group_size, device.index, tuple((x.data_ptr(), x.shape[0], x.shape[1]) for x in xs))
-    entry = _STE_TABLES.get(key)
-    if entry is not None:
-        _STE_TABLES.move_to_end(key)
-        return entry
+    with _STE_LOCK:
+        entry = _STE_TABLES.get(key)
+        if entry is not None:
+            _STE_TABLES.move_to_end(key)
+            return entry
     per = _lib.INT4_GROUPS_PER_WG
     rows, offs, off = [], [], 0
     for x in xs:
@@ -463,9 +462,10 @@ def _ste_table(xs, group_size):
     step = per * group_size * 2
     items = torch.stack([d[:, 0] + local * step, d[:, 1] + local * step, torch.clamp(d[:, 2] - local * per, max=per)], dim=1)
     entry = (items.contiguous().to(device), items.shape[0], offs, off // 2)
-    _STE_TABLES[key] = entry
-    while len(_STE_TABLES) > 1024:
-        _STE_TABLES.popitem(last=False)
+    with _STE_LOCK:
+        _STE_TABLES[key] = entry
+        while len(_STE_TABLES) > 1024:
+            _STE_TABLES.popitem(last=False)
     return entry
 
 
