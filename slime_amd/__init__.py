@@ -8,6 +8,7 @@ of ``slime_amd/lib/libslime_amd_wq.so``; there is no CPU or pure-torch fallback.
 
 from . import _lib, arith, delta
 from .aligned import get_fp8_aligned_absorb_weight
+from .hf_reader import SafetensorReader
 from .bucket import BucketConverter, FlattenedBucket, FlattenedTensorMetadata, quantize_bucket
 from .arith import get_torch_arithmetic, set_torch_arithmetic, torch_arithmetic
 from .fp8 import (
@@ -51,7 +52,7 @@ from .processors import (
 quantize_weight = blockwise_cast_to_fp8_triton
 
 __all__ = [
-    "block_quant_dequant", "fp8_aligned_weight", "get_fp8_aligned_absorb_weight",
+    "block_quant_dequant", "fp8_aligned_weight", "get_fp8_aligned_absorb_weight", "SafetensorReader",
     "Int4StePlan", "fake_int4_quantization_ste_many", "BucketConverter", "FlattenedBucket", "FlattenedTensorMetadata", "quantize_bucket", "quant_weight_ue8m0",
     "set_ue8m0_requant", "transform_scale_ue8m0",
     "Fp8DequantPlan", "Fp8QuantPlan", "Int4DequantPlan", "Int4PackPlan", "block_fp8", "block_fp8_many",
