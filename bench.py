@@ -374,6 +374,42 @@ def bench_bucket(dev, steps, warmup, layers):
     return out
 
 
+def bench_grouped_experts(dev, steps, warmup, experts=128):
+    """The stacked expert weights of one MoE layer's grouped linears (fc1 = gate+up [1536, 2048], fc2 [2048, 768]) as the
+    FP8-aligned MoE forward quantises them on every step: one launch per grouped linear against the loop it replaces."""
+    import torch
+
+    import slime_amd
+
+    fc1 = [_gen_bf16((1536, 2048), dev, outliers=True) for _ in range(experts)]
+    fc2 = [_gen_bf16((2048, 768), dev, outliers=True) for _ in range(experts)]
+
+    def one_launch():
+        slime_amd.quantize_grouped_weights(fc1, (128, 128))
+        slime_amd.quantize_grouped_weights(fc2, (128, 128))
+
+    def loop():
+        for ws, shape in ((fc1, (1536, 2048)), (fc2, (2048, 768))):
+            q = torch.empty((experts, *shape), dtype=torch.float8_e4m3fn, device=dev)
+            s = torch.empty((experts, shape[0] // 128, shape[1] // 128), dtype=torch.float32, device=dev)
+            for e, w in enumerate(ws):
+                qe, se = slime_amd.blockwise_cast_to_fp8_triton(w, (128, 128))
+                q[e].copy_(qe)
+                s[e].copy_(se)
+
+    wall1, ev1, _ = _time_launches(one_launch, steps, warmup)
+    wall2, ev2, _ = _time_launches(loop, max(steps // 4, 2), 1)
+    q, s = slime_amd.quantize_grouped_weights(fc1, (128, 128))
+    qe, se = slime_amd.blockwise_cast_to_fp8_triton(fc1[7], (128, 128))
+    assert torch.equal(q[7].view(torch.uint8), qe.view(torch.uint8)) and torch.equal(s[7], se)
+    el = experts * (1536 * 2048 + 2048 * 768)
+    algo = 3 * el + 4 * el // 16384
+    return {"workload": f"{experts} experts x (fc1 [1536,2048], fc2 [2048,768]) bf16 -> stacked e4m3 [E,N,K] + fp32 scales, "
+                        "one launch per grouped linear (table cached on the weight addresses)",
+            "ms": ev1, "wall_ms": wall1, "hbm_frac": algo / ev1 / 1e6 / HBM_PEAK_GBS,
+            "per_expert_loop_ms": ev2, "per_expert_loop_wall_ms": wall2, "launches": 2, "loop_launches": 6 * experts}
+
+
 def bench_int4_pack(dev, steps, warmup, layers):
     import torch
 
@@ -779,7 +815,7 @@ def main():
     ap.add_argument("--dequant-experts", type=int, default=256)
     ap.add_argument("--no-extras", action="store_true", help="headline step only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
-    ap.add_argument("--only", choices=["fp8", "cfg1", "bucket", "fp8moe", "int4", "dequant", "int4deq", "ste", "delta", "forms", "copy", "stream", "hashes"], default=None,
+    ap.add_argument("--only", choices=["fp8", "cfg1", "bucket", "fp8moe", "int4", "dequant", "int4deq", "ste", "delta", "forms", "experts", "copy", "stream", "hashes"], default=None,
                     help="run just one of the other legs and print its record: a kernel for profiling, the plain copy "
                          "kernel that hardware counters are calibrated against, or the host-resident streaming run "
                          "(64 x 1 GiB buckets, PCIe-bound)")
@@ -824,6 +860,9 @@ def main():
         return
     if args.only in ("int4deq", "ste"):
         print(json.dumps(bench_int4_inverse(dev, args.steps, args.warmup, min(args.int4_layers, 8), args.only)))
+        return
+    if args.only == "experts":
+        print(json.dumps(bench_grouped_experts(dev, args.steps, args.warmup)))
         return
     if args.only == "forms":
         print(json.dumps(bench_single_tensor_forms(dev, args.steps, args.warmup)))
@@ -890,6 +929,7 @@ def main():
             extras["weight_sync_bucket"] = bench_bucket(dev, args.steps, args.warmup, args.int4_layers)
         extras["delta_xor"] = bench_delta(dev, args.steps, args.warmup)
         extras["single_tensor_forms"] = bench_single_tensor_forms(dev, args.steps, args.warmup)
+        extras["grouped_expert_weights"] = bench_grouped_experts(dev, args.steps, args.warmup)
         # the practical ceiling of a 1:1 read:write stream on this very box, measured in this very run
         extras["copy_kernel_calibration"] = bench_copy(dev, args.steps, args.warmup)
         line["other_workloads"] = extras

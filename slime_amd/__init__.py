@@ -43,6 +43,7 @@ from .processors import (
     _quantize_param,
     quantize_params,
     quantize_params_compressed_tensors,
+    quantize_grouped_weights,
     quantize_params_fp8,
     set_ue8m0_requant,
 )
@@ -52,7 +53,7 @@ from .processors import (
 quantize_weight = blockwise_cast_to_fp8_triton
 
 __all__ = [
-    "block_quant_dequant", "fp8_aligned_weight", "get_fp8_aligned_absorb_weight", "SafetensorReader",
+    "quantize_grouped_weights", "block_quant_dequant", "fp8_aligned_weight", "get_fp8_aligned_absorb_weight", "SafetensorReader",
     "Int4StePlan", "fake_int4_quantization_ste_many", "BucketConverter", "FlattenedBucket", "FlattenedTensorMetadata", "quantize_bucket", "quant_weight_ue8m0",
     "set_ue8m0_requant", "transform_scale_ue8m0",
     "Fp8DequantPlan", "Fp8QuantPlan", "Int4DequantPlan", "Int4PackPlan", "block_fp8", "block_fp8_many",

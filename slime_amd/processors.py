@@ -192,6 +192,64 @@ def _group_cast(weights, block_size):
             for q0, M, N, s0, tm, tn in layout]
 
 
+def quantize_grouped_weights(weights, block_size=(128, 128), use_ue8m0: bool = False):
+    """The expert weights of one grouped linear quantised by ONE launch straight into the stacked tensors a grouped GEMM
+    reads: -> (qweight e4m3fn [E, N, K], scale float32 [E, ceil(N/bm), ceil(K/bn)]).
+
+    Replaces the loop of ``_quantize_grouped_weights`` (slime/backends/megatron_utils/alignment/
+    deepgemm_moe_forward.py:1383-1428), which calls ``ops.quantize_weight(weight, (128, 128))`` - that is
+    ``blockwise_cast_to_fp8_triton``, or sglang's ``quant_weight_ue8m0`` with ``use_ue8m0`` - once per expert and copies
+    every result into the stacked tensors: E launches, 2 E copies and a second pass over the quantised bytes.  Same
+    bytes; the per-tile table is cached on the addresses of the weights (a training step presents the same parameters
+    again).  All weights: 2-D bf16 on one GPU, one shape.  The reference's later ``requant_weight_ue8m0`` of the stacked
+    tensors (sglang, Blackwell only) is not provided."""
+    weights = list(weights)
+    if not weights:
+        raise ValueError("quantize_grouped_weights: no weights")
+    bm, bn = int(block_size[0]), int(block_size[1])
+    shape, device = tuple(weights[0].shape), weights[0].device
+    for i, w in enumerate(weights):
+        if w.dtype != torch.bfloat16:
+            raise RuntimeError(f"weight{i} must be BF16, got {w.dtype}")
+        if not w.is_cuda or w.device != device:
+            raise RuntimeError(f"weight{i} must be on {device}, got {w.device}")
+        if w.dim() != 2 or tuple(w.shape) != shape:
+            raise RuntimeError(f"weight{i} has shape {tuple(w.shape)}, expected {shape}")
+    E, (M, N) = len(weights), shape
+    tm, tn = ceildiv(M, bm), ceildiv(N, bn)
+    mode = _lib.FP8_MODE_UE8M0 if use_ue8m0 else _lib.FP8_MODE_TRITON
+    if E * M * N == 0:
+        return (torch.empty((E, M, N), dtype=FP8_DTYPE, device=device),
+                torch.empty((E, tm, tn), dtype=torch.float32, device=device))
+    key = ("stacked", bm, bn, device.index, tuple((w.data_ptr(), w.stride()) for w in weights), shape)
+    with _GROUP_LOCK:
+        entry = _GROUP_TABLES.get(key)
+        if entry is not None:
+            _GROUP_TABLES.move_to_end(key)
+            _GROUP_STATS["hits"] += 1
+    s_base = (E * M * N + 15) // 16 * 16
+    if entry is None:
+        rows = [[w.data_ptr(), e * M * N, s_base + 4 * e * tm * tn, M, N, w.stride(0), w.stride(1), N]
+                for e, w in enumerate(weights)]
+        table, _, _ = tile_table(rows, bm, bn)
+        entry = (table.contiguous().to(device), table.shape[0], None, s_base + 4 * E * tm * tn)
+        with _GROUP_LOCK:
+            if key not in _GROUP_TABLES:
+                _GROUP_STATS["bytes"] += entry[0].numel() * 8
+            _GROUP_TABLES[key] = entry
+            _GROUP_STATS["builds"] += 1
+            while _GROUP_STATS["bytes"] > _GROUP_MAX_BYTES and len(_GROUP_TABLES) > 1:
+                _, old = _GROUP_TABLES.popitem(last=False)
+                _GROUP_STATS["bytes"] -= old[0].numel() * 8
+    table, n_tiles, _, total = entry
+    flat = torch.empty(total, dtype=torch.uint8, device=device)
+    with torch.cuda.device(device):
+        rc = _lib.load().wq_fp8_bucket_convert(table.data_ptr(), n_tiles, flat.data_ptr(), bm, bn, mode, _lib.stream_ptr(device))
+    _lib.check(rc, "quantize_grouped_weights")
+    return (flat[:E * M * N].view(FP8_DTYPE).view(E, M, N),
+            flat[s_base:s_base + 4 * E * tm * tn].view(torch.float32).view(E, tm, tn))
+
+
 def _is_ignored(name: str, ignore_rules) -> bool:
     """``re:<regex>`` rules use re.match, others match exactly or as a prefix
     (quantizer_compressed_tensors.py:277-279)."""
@@ -239,4 +297,4 @@ def quantize_params(args, megatron_name, converted_named_params, quantization_co
 
 
 __all__ = ["quantize_params", "quantize_params_fp8", "_quantize_param", "quantize_params_compressed_tensors",
-           "set_ue8m0_requant", "ue8m0_requant_enabled", "plan_cache_info", "FP8_DTYPE"]
+           "set_ue8m0_requant", "ue8m0_requant_enabled", "plan_cache_info", "quantize_grouped_weights", "FP8_DTYPE"]

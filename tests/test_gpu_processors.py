@@ -5,6 +5,7 @@ import torch
 
 import slime_amd
 from oracle import c_oracle as C
+from slime_amd import processors
 from tests import wq_inputs as I
 
 pytestmark = pytest.mark.gpu
@@ -65,3 +66,42 @@ def test_shim_module_and_hook(cuda):
     assert I.same_bits(q.cpu(), qo) and I.same_bits(s.cpu(), so)
     qw, sc = slime_amd.quantize_weight(w.to(cuda), (128, 128))
     assert tuple(qw.shape) == (8, 256) and tuple(sc.shape) == (1, 2) and sc.dtype == torch.float32
+
+
+@pytest.mark.parametrize("shape", [(768, 2048), (300, 200), (129, 127)])
+@pytest.mark.parametrize("ue8m0", [False, True])
+def test_quantize_grouped_weights_equals_the_per_expert_loop(cuda, shape, ue8m0):
+    """The stacked [E, N, K] codes and [E, n, k] scales of the alignment forward's grouped weights, one launch, against
+    the loop it replaces (quantise each expert, copy into the stack) and the oracle."""
+    E = 5
+    fc = I.weights(E * shape[0], shape[1], seed=shape[0]).to(cuda)
+    views = list(fc.chunk(E, dim=0))                                  # expert weights as views of one parameter
+    views[2] = views[2].clone().t().contiguous().t()                  # one of them column-major
+    q, s = slime_amd.quantize_grouped_weights(views, (128, 128), use_ue8m0=ue8m0)
+    tm, tn = -(-shape[0] // 128), -(-shape[1] // 128)
+    assert q.shape == (E, *shape) and q.dtype == torch.float8_e4m3fn and s.shape == (E, tm, tn) and s.dtype == torch.float32
+    assert q.is_contiguous() and s.is_contiguous()
+    one = slime_amd.quant_weight_ue8m0 if ue8m0 else slime_amd.blockwise_cast_to_fp8_triton
+    for e, w in enumerate(views):
+        qe, se = one(w.contiguous(), [128, 128])
+        assert I.same_bits(q[e].view(torch.uint8), qe.view(torch.uint8)) and I.same_bits(s[e], se), e
+        qo, so = C.fp8_block_quant(w.cpu().contiguous(), (128, 128), 3 if ue8m0 else 1)
+        assert torch.equal(q[e].cpu().view(torch.uint8), qo) and I.same_bits(s[e].cpu(), so), e
+    builds = processors.plan_cache_info()["builds"]
+    q2, _ = slime_amd.quantize_grouped_weights(views, (128, 128), use_ue8m0=ue8m0)
+    assert processors.plan_cache_info()["builds"] == builds and I.same_bits(q2.view(torch.uint8), q.view(torch.uint8))
+    assert q2.data_ptr() != q.data_ptr()                              # fresh outputs on every call
+
+
+def test_quantize_grouped_weights_argument_errors(cuda):
+    w = I.weights(128, 256).to(cuda)
+    with pytest.raises(RuntimeError, match="must be BF16"):
+        slime_amd.quantize_grouped_weights([w, w.float()])
+    with pytest.raises(RuntimeError, match="expected"):
+        slime_amd.quantize_grouped_weights([w, w[:64]])
+    with pytest.raises(RuntimeError, match="must be on"):
+        slime_amd.quantize_grouped_weights([w, w.cpu()])
+    with pytest.raises(ValueError):
+        slime_amd.quantize_grouped_weights([])
+    q, s = slime_amd.quantize_grouped_weights([w[:0], w[:0]])
+    assert q.shape == (2, 0, 256) and s.shape == (2, 0, 2)
