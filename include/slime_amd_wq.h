@@ -399,19 +399,18 @@ int wq_delta_xor_items(const wq_delta_chunk_item *items, int64_t n_items, const 
                        int write_diff, int update_old, void *stream);
 
 /* ---------------------------------------------------------------------------------------------
- * XXH3-128 (seed 0) of n > 240 bytes in device memory: the digest checksum("xxh3-128", new) attaches to every
+ * XXH3-128 (seed 0) of n >= 0 bytes in device memory: the digest checksum("xxh3-128", new) attaches to every
  * changed tensor of a published delta (slime/utils/disk_delta.py:40-58; the default of
  * --update-weight-delta-checksum, slime/utils/arguments.py:186-188), computed where the tensor lives instead of
  * after a copy to the host.  digest: DEVICE uint64[2] = {low64, high64}; the reference's hexdigest() is
  * high64 then low64, most significant byte first.  workspace: DEVICE, wq_xxh3_workspace_bytes(n) bytes
  * (64 per KiB of input), 16-byte aligned, overwritten.  Any alignment of `data` (16-byte aligned inputs take
- * the fast path).  n <= 240 (XXH3's short-input forms) returns WQ_ERR_UNSUPPORTED: hash those on the host. */
+ * the fast path; NULL allowed for n = 0).  Inputs up to 240 bytes take XXH3's short forms on one lane. */
 int64_t wq_xxh3_workspace_bytes(int64_t n);
 int wq_xxh3_128(const void *data, int64_t n, uint64_t *workspace, uint64_t *digest, void *stream);
 
 /* Many tensors, two launches.  `descs` DEVICE array; item_start DEVICE int64[n_desc+1], exclusive prefix sum of
- * ceil(((n - 1) / 1024) / 16) per tensor (work items of 16 KiB).  Tensors of 240 bytes or less are skipped
- * (their digest slot is left untouched). */
+ * ceil(((n - 1) / 1024) / 16) per tensor (work items of 16 KiB; 0 for n <= 1024). */
 typedef struct wq_xxh3_desc {
     const void *data;
     int64_t n;

@@ -1,4 +1,5 @@
-"""TEST INFRASTRUCTURE: XXH3-128 (seed 0, default secret) of inputs longer than 240 bytes, restated in numpy.
+"""TEST INFRASTRUCTURE: XXH3-128 (seed 0, default secret), restated in numpy (long inputs) and plain integers (the
+forms for 0..240 bytes).
 
 The reference's delta publisher digests every changed tensor with ``checksum("xxh3-128", new)``
 (slime/utils/disk_delta.py:40-58, default of --update-weight-delta-checksum, slime/utils/arguments.py:186-188), i.e.
@@ -91,12 +92,99 @@ def _merge(acc, offset: int, start: int) -> int:
     return _avalanche(r)
 
 
+PRIME_MX2 = 0x9FB21C651E98DF25
+
+
+def _s64(off: int) -> int:
+    return int.from_bytes(SECRET[off:off + 8], "little")
+
+
+def _s32(off: int) -> int:
+    return int.from_bytes(SECRET[off:off + 4], "little")
+
+
+def _le(b: bytes, off: int, size: int) -> int:
+    return int.from_bytes(b[off:off + size], "little")
+
+
+def _xxh64_avalanche(h: int) -> int:
+    h ^= h >> 33
+    h = (h * P64_2) & M64
+    h ^= h >> 29
+    h = (h * P64_3) & M64
+    return h ^ (h >> 32)
+
+
+def _mix16(b: bytes, off: int, soff: int) -> int:
+    return _mul128_fold64(_le(b, off, 8) ^ _s64(soff), _le(b, off + 8, 8) ^ _s64(soff + 8))
+
+
+def _mix32(acc, b: bytes, o1: int, o2: int, soff: int):
+    low, high = acc
+    low = (low + _mix16(b, o1, soff)) & M64
+    low ^= (_le(b, o2, 8) + _le(b, o2 + 8, 8)) & M64
+    high = (high + _mix16(b, o2, soff + 16)) & M64
+    high ^= (_le(b, o1, 8) + _le(b, o1 + 8, 8)) & M64
+    return low, high
+
+
+def _finish_mid(acc, n: int) -> tuple[int, int]:
+    low, high = acc
+    h_low = (low + high) & M64
+    h_high = (low * P64_1 + high * P64_4 + n * P64_2) & M64
+    return _avalanche(h_low), (-_avalanche(h_high)) & M64
+
+
+def xxh3_128_short(b: bytes) -> tuple[int, int]:
+    """The forms for inputs of 0..240 bytes (XXH3_len_0to16_128b, _17to128_128b, _129to240_128b; seed 0)."""
+    n = len(b)
+    if n == 0:
+        return _xxh64_avalanche(_s64(64) ^ _s64(72)), _xxh64_avalanche(_s64(80) ^ _s64(88))
+    if n <= 3:
+        lo = (b[0] << 16) | (b[n >> 1] << 24) | b[n - 1] | (n << 8)
+        swapped = int.from_bytes(lo.to_bytes(4, "little"), "big")
+        hi = ((swapped << 13) | (swapped >> 19)) & 0xFFFFFFFF
+        return _xxh64_avalanche(lo ^ (_s32(0) ^ _s32(4))), _xxh64_avalanche(hi ^ (_s32(8) ^ _s32(12)))
+    if n <= 8:
+        keyed = (_le(b, 0, 4) + (_le(b, n - 4, 4) << 32)) ^ (_s64(16) ^ _s64(24))
+        p = keyed * (P64_1 + (n << 2))
+        low, high = p & M64, p >> 64
+        high = (high + (low << 1)) & M64
+        low ^= high >> 3
+        low ^= low >> 35
+        low = (low * PRIME_MX2) & M64
+        low ^= low >> 28
+        return low, _avalanche(high)
+    if n <= 16:
+        in_lo, in_hi = _le(b, 0, 8), _le(b, n - 8, 8)
+        p = (in_lo ^ in_hi ^ (_s64(32) ^ _s64(40))) * P64_1
+        low, high = p & M64, p >> 64
+        low = (low + ((n - 1) << 54)) & M64
+        in_hi ^= _s64(48) ^ _s64(56)
+        high = (high + in_hi + (in_hi & 0xFFFFFFFF) * (P32_2 - 1)) & M64
+        low ^= int.from_bytes(high.to_bytes(8, "little"), "big")
+        q = low * P64_2
+        return _avalanche(q & M64), _avalanche(((q >> 64) + high * P64_2) & M64)
+    acc = ((n * P64_1) & M64, 0)
+    if n <= 128:
+        for i in range((n - 1) // 32, -1, -1):
+            acc = _mix32(acc, b, 16 * i, n - 16 * (i + 1), 32 * i)
+        return _finish_mid(acc, n)
+    for i in range(32, 160, 32):
+        acc = _mix32(acc, b, i - 32, i - 16, i - 32)
+    acc = (_avalanche(acc[0]), _avalanche(acc[1]))
+    for i in range(160, n + 1, 32):
+        acc = _mix32(acc, b, i - 32, i - 16, 3 + i - 160)
+    acc = _mix32(acc, b, n - 16, n - 32, 136 - 17 - 16)
+    return _finish_mid(acc, n)
+
+
 def xxh3_128(data) -> tuple[int, int]:
-    """-> (low64, high64) of XXH3_128bits(data) for len(data) > 240."""
+    """-> (low64, high64) of XXH3_128bits(data)."""
     data = np.frombuffer(bytes(data), dtype=np.uint8)
     n = data.size
     if n <= 240:
-        raise ValueError("the short-input forms of XXH3 are not restated here")
+        return xxh3_128_short(data.tobytes())
     n_blocks = (n - 1) // BLOCK
     acc = chain(block_sums(data, n_blocks))
     with np.errstate(over="ignore"):

@@ -13,7 +13,7 @@
 //   xxh3_chain_kernel        per tensor, eight lanes walk acc <- scramble(acc + sums[k]) (about 60 clocks a block), add
 //                            the tail - the stripes of the last partial block and the last 64 bytes, read straight from
 //                            the tensor - and one lane folds the accumulators into the two 64-bit halves.
-// Inputs of 240 bytes or less use XXH3's short forms, which are not provided (the caller hashes those on the host).
+// Inputs of 240 bytes or less use XXH3's short forms: one lane of the second kernel computes those.
 
 #include "wq_common.h"
 
@@ -154,6 +154,96 @@ __device__ __forceinline__ uint64_t avalanche(uint64_t h)
     return h ^ (h >> 32);
 }
 
+// ---- inputs of 0..240 bytes: XXH3's short forms, one lane (a few hundred dependent operations at most) --------------
+
+constexpr uint64_t kMx2 = 0x9FB21C651E98DF25ull;
+
+__device__ __forceinline__ uint32_t secret32(int off)
+{
+    return (uint32_t)kXxh3Secret[off] | ((uint32_t)kXxh3Secret[off + 1] << 8) | ((uint32_t)kXxh3Secret[off + 2] << 16) |
+           ((uint32_t)kXxh3Secret[off + 3] << 24);
+}
+
+__device__ __forceinline__ uint64_t xxh64_avalanche(uint64_t h)
+{
+    h ^= h >> 33;
+    h *= kP64_2;
+    h ^= h >> 29;
+    h *= kP64_3;
+    return h ^ (h >> 32);
+}
+
+__device__ __forceinline__ uint64_t bswap64(uint64_t v)
+{
+    return ((uint64_t)__builtin_bswap32((uint32_t)v) << 32) | __builtin_bswap32((uint32_t)(v >> 32));
+}
+
+__device__ __forceinline__ uint64_t mix16(const uint8_t* p, int soff)
+{
+    return mul128_fold64(load64_bytes(p) ^ secret64(soff), load64_bytes(p + 8) ^ secret64(soff + 8));
+}
+
+__device__ __forceinline__ void mix32(uint64_t& low, uint64_t& high, const uint8_t* p1, const uint8_t* p2, int soff)
+{
+    low += mix16(p1, soff);
+    low ^= load64_bytes(p2) + load64_bytes(p2 + 8);
+    high += mix16(p2, soff + 16);
+    high ^= load64_bytes(p1) + load64_bytes(p1 + 8);
+}
+
+__device__ void xxh3_short(const uint8_t* p, int n, uint64_t& out_low, uint64_t& out_high)
+{
+    if (n == 0) {
+        out_low = xxh64_avalanche(secret64(64) ^ secret64(72));
+        out_high = xxh64_avalanche(secret64(80) ^ secret64(88));
+    } else if (n <= 3) {
+        const uint32_t lo = ((uint32_t)p[0] << 16) | ((uint32_t)p[n >> 1] << 24) | (uint32_t)p[n - 1] | ((uint32_t)n << 8);
+        const uint32_t sw = __builtin_bswap32(lo), hi = (sw << 13) | (sw >> 19);
+        out_low = xxh64_avalanche((uint64_t)lo ^ (uint64_t)(secret32(0) ^ secret32(4)));
+        out_high = xxh64_avalanche((uint64_t)hi ^ (uint64_t)(secret32(8) ^ secret32(12)));
+    } else if (n <= 8) {
+        uint32_t a = 0, b = 0;
+        for (int k = 0; k < 4; ++k) {
+            a |= (uint32_t)p[k] << (8 * k);
+            b |= (uint32_t)p[n - 4 + k] << (8 * k);
+        }
+        const uint64_t keyed = ((uint64_t)a + ((uint64_t)b << 32)) ^ (secret64(16) ^ secret64(24));
+        const uint64_t mult = kP64_1 + ((uint64_t)n << 2);
+        uint64_t low = keyed * mult, high = __umul64hi(keyed, mult);
+        high += low << 1;
+        low ^= high >> 3;
+        low ^= low >> 35;
+        low *= kMx2;
+        low ^= low >> 28;
+        out_low = low;
+        out_high = avalanche(high);
+    } else if (n <= 16) {
+        const uint64_t in_lo = load64_bytes(p);
+        uint64_t in_hi = load64_bytes(p + n - 8);
+        const uint64_t x = in_lo ^ in_hi ^ (secret64(32) ^ secret64(40));
+        uint64_t low = x * kP64_1, high = __umul64hi(x, kP64_1);
+        low += (uint64_t)(n - 1) << 54;
+        in_hi ^= secret64(48) ^ secret64(56);
+        high += in_hi + (in_hi & 0xFFFFFFFFull) * (kP32_2 - 1);
+        low ^= bswap64(high);
+        out_low = avalanche(low * kP64_2);
+        out_high = avalanche(__umul64hi(low, kP64_2) + high * kP64_2);
+    } else {
+        uint64_t low = (uint64_t)n * kP64_1, high = 0;
+        if (n <= 128) {
+            for (int i = (n - 1) / 32; i >= 0; --i) mix32(low, high, p + 16 * i, p + n - 16 * (i + 1), 32 * i);
+        } else {
+            for (int i = 32; i < 160; i += 32) mix32(low, high, p + i - 32, p + i - 16, i - 32);
+            low = avalanche(low);
+            high = avalanche(high);
+            for (int i = 160; i <= n; i += 32) mix32(low, high, p + i - 32, p + i - 16, 3 + i - 160);
+            mix32(low, high, p + n - 16, p + n - 32, 136 - 17 - 16);
+        }
+        out_low = avalanche(low + high);
+        out_high = 0 - avalanche(low * kP64_1 + high * kP64_4 + (uint64_t)n * kP64_2);
+    }
+}
+
 // one wavefront per tensor; lanes 0..7 own one accumulator each
 __global__ __launch_bounds__(64) void xxh3_chain_kernel(const wq_xxh3_desc single, const wq_xxh3_desc* __restrict__ descs,
                                                         int n_desc)
@@ -161,8 +251,16 @@ __global__ __launch_bounds__(64) void xxh3_chain_kernel(const wq_xxh3_desc singl
     const int t = blockIdx.x;
     if (t >= n_desc) return;
     const wq_xxh3_desc d = descs ? descs[t] : single;
-    if (d.n <= 240) return;                   // short forms: not provided (rejected on the host for the single form)
     const int lane = threadIdx.x, i = lane & 7;
+    if (d.n <= 240) {                         // uniform per wavefront
+        if (lane == 0) {
+            uint64_t low, high;
+            xxh3_short((const uint8_t*)d.data, (int)d.n, low, high);
+            d.digest[0] = low;
+            d.digest[1] = high;
+        }
+        return;
+    }
     const uint64_t init[8] = {kP32_3, kP64_1, kP64_2, kP64_3, kP64_4, kP32_2, kP64_5, kP32_1};
     uint64_t acc = init[0];
 #pragma unroll
@@ -251,8 +349,7 @@ WQ_EXPORT int64_t wq_xxh3_workspace_bytes(int64_t n) { return n > 0 ? ((n - 1) /
 WQ_EXPORT int wq_xxh3_128(const void* data, int64_t n, uint64_t* workspace, uint64_t* digest, void* stream)
 {
     if (n < 0) return WQ_ERR_SHAPE;
-    if (n <= 240) return WQ_ERR_UNSUPPORTED;
-    if (!data || !workspace || !digest) return WQ_ERR_NULL;
+    if ((n > 0 && !data) || !workspace || !digest) return WQ_ERR_NULL;
     if (((uintptr_t)workspace & 15) || ((uintptr_t)digest & 7)) return WQ_ERR_ALIGN;
     hipStream_t st = (hipStream_t)stream;
     Xxh3Args a{};

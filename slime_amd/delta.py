@@ -11,7 +11,8 @@ only the diff of a tensor that did change has to cross PCIe for compression.
 snapshot-keeping loop body (``diff_and_compress`` + ``collect`` without the zstd step, which stays on the
 host).  ``adler32`` comes out of the diff pass itself; ``xxh3-128`` - the reference's default - is computed on the GPU
 too (its per-block sums at memory speed, the sequential scramble chain by eight lanes per tensor: ``xxh3_128`` /
-``xxh3_128_many``), so a changed tensor's bytes never cross PCIe for their digest.  ``blake3`` is a host digest.
+``xxh3_128_many``), so a changed tensor's bytes never cross PCIe for their digest.  ``blake3`` is a host digest, as in
+the reference.
 """
 
 from __future__ import annotations
@@ -174,46 +175,35 @@ def overwrite_encode(new: torch.Tensor, old: torch.Tensor) -> torch.Tensor:
     return out
 
 
-XXH3_SHORT = 240     # inputs up to this size use XXH3's short forms: hashed on the host (a few hundred bytes to copy)
-
-
 def _hex128(low: int, high: int) -> str:
     return f"{high & 0xFFFFFFFFFFFFFFFF:016x}{low & 0xFFFFFFFFFFFFFFFF:016x}"
 
 
 def xxh3_128_many(tensors) -> list:
     """``xxhash.xxh3_128(bytes of t).hexdigest()`` for every tensor, computed on the GPU with two launches and one
-    synchronisation (tensors of 240 bytes or less: on the host).  -> list of 32-digit hex strings."""
+    synchronisation.  -> list of 32-digit hex strings."""
     flats = [_as_bytes(t, "xxh3_128") for t in tensors]
-    out = [None] * len(flats)
-    big = [i for i, f in enumerate(flats) if f.numel() > XXH3_SHORT]
-    if big:
-        device = flats[big[0]].device
-        lib = _lib.load()
-        ws_off, total_ws, items, n_items = [], 0, [0], 0
-        for i in big:
-            n = flats[i].numel()
-            ws_off.append(total_ws)
-            total_ws += (lib.wq_xxh3_workspace_bytes(n) + 255) // 256 * 256
-            n_items += -(-((n - 1) // 1024) // 16)
-            items.append(n_items)
-        ws = torch.empty(total_ws // 8, dtype=torch.int64, device=device)
-        digests = torch.empty((len(big), 2), dtype=torch.int64, device=device)
-        rows = [[flats[i].data_ptr(), flats[i].numel(), ws.data_ptr() + o, digests.data_ptr() + 16 * k]
-                for k, (i, o) in enumerate(zip(big, ws_off))]
-        descs = torch.tensor(rows, dtype=torch.int64).to(device)
-        starts = torch.tensor(items, dtype=torch.int64).to(device)
-        with torch.cuda.device(device):
-            rc = lib.wq_xxh3_128_grouped(descs.data_ptr(), starts.data_ptr(), len(big), n_items, _lib.stream_ptr(device))
-        _lib.check(rc, "xxh3_128")
-        for i, (low, high) in zip(big, digests.tolist()):
-            out[i] = _hex128(low, high)
-    for i, f in enumerate(flats):
-        if out[i] is None:
-            from .delta_host import host_checksum
-
-            out[i] = host_checksum("xxh3-128", f)
-    return out
+    if not flats:
+        return []
+    device = flats[0].device
+    lib = _lib.load()
+    ws_off, total_ws, items, n_items = [], 0, [0], 0
+    for f in flats:
+        n = f.numel()
+        ws_off.append(total_ws)
+        total_ws += (lib.wq_xxh3_workspace_bytes(n) + 255) // 256 * 256
+        n_items += -(-((n - 1) // 1024) // 16) if n > 0 else 0
+        items.append(n_items)
+    ws = torch.empty(total_ws // 8, dtype=torch.int64, device=device)
+    digests = torch.empty((len(flats), 2), dtype=torch.int64, device=device)
+    rows = [[f.data_ptr(), f.numel(), ws.data_ptr() + o, digests.data_ptr() + 16 * k]
+            for k, (f, o) in enumerate(zip(flats, ws_off))]
+    descs = torch.tensor(rows, dtype=torch.int64).to(device)
+    starts = torch.tensor(items, dtype=torch.int64).to(device)
+    with torch.cuda.device(device):
+        rc = lib.wq_xxh3_128_grouped(descs.data_ptr(), starts.data_ptr(), len(flats), n_items, _lib.stream_ptr(device))
+    _lib.check(rc, "xxh3_128")
+    return [_hex128(low, high) for low, high in digests.tolist()]
 
 
 def xxh3_128(buf: torch.Tensor) -> str:

@@ -1,5 +1,6 @@
-"""Host-side digests for the delta publisher: the sequential hash functions the GPU does not compute
-(slime/utils/disk_delta.py:40-58: xxh3-128 via ``xxhash``, blake3 via ``blake3``)."""
+"""The one digest of the delta publisher that stays a host computation: blake3, a tree hash with its own package
+(slime/utils/disk_delta.py:46-49 imports ``blake3`` the same way).  adler32 and xxh3-128 are computed on the GPU
+(``slime_amd.delta.checksum``)."""
 
 from __future__ import annotations
 
@@ -7,16 +8,10 @@ import torch
 
 
 def host_checksum(algorithm: str, buf: torch.Tensor) -> str:
-    data = buf.detach().contiguous().view(torch.uint8).reshape(-1).cpu().numpy()
-    if algorithm == "xxh3-128":
-        import xxhash
-
-        h = xxhash.xxh3_128()
-    elif algorithm == "blake3":
-        import blake3
-
-        h = blake3.blake3()
-    else:
+    if algorithm != "blake3":
         raise KeyError(f"unknown checksum algorithm {algorithm!r}")
-    h.update(data)
+    import blake3
+
+    h = blake3.blake3()
+    h.update(buf.detach().contiguous().view(torch.uint8).reshape(-1).cpu().numpy())
     return h.hexdigest()

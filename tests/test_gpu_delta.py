@@ -100,7 +100,7 @@ def test_delta_encoder_follows_the_reference_loop(cuda, encoding):
     assert enc.total_bytes == 3 * sum(v.size for v in snapshot.values()) and enc.changed_bytes > 0
 
 
-def test_host_digest_for_sequential_hashes(cuda):
+def test_encoder_with_the_xxh3_digest(cuda):
     import xxhash
 
     x = torch.arange(100000, dtype=torch.int32).view(torch.uint8)
@@ -158,3 +158,10 @@ def test_delta_encoder_bucket(cuda):
         else:
             assert diff is None and name not in ("l2.weight", "l5.weight")
         assert np.array_equal(enc.snapshot[name].cpu().numpy(), new)
+
+
+def test_unknown_digest_names(cuda):
+    x = torch.zeros(64, dtype=torch.uint8, device=cuda)
+    with pytest.raises(KeyError):
+        delta.checksum("md5", x)
+    assert delta.checksum("xxh3-128", x[:0]) == "99aa06d3014798d86001c324468d497f"      # XXH3_128bits of the empty input

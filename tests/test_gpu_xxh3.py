@@ -19,6 +19,13 @@ def _bytes(n, seed):
     return torch.from_numpy(np.random.default_rng(seed).integers(0, 256, n, dtype=np.uint8))
 
 
+def test_short_forms_every_length(cuda):
+    xs = [_bytes(n, 300 + n) for n in range(0, 241)] + [torch.full((n,), 255, dtype=torch.uint8) for n in (1, 3, 8, 16, 17, 128, 129, 240)]
+    got = delta.xxh3_128_many([x.to(cuda) for x in xs])
+    for x, g in zip(xs, got):
+        assert g == _lib_hex(x) and g == X.hexdigest(x.numpy()), x.numel()
+
+
 @pytest.mark.parametrize("n", [241, 256, 305, 1023, 1024, 1025, 1088, 1089, 2047, 2048, 2049, 16383, 16384, 16385, 16384 * 3 + 1,
                                65536 + 64, (1 << 20) - 2, 1 << 20, (1 << 20) + 2, 5 * (1 << 20) + 777])
 def test_every_boundary_against_the_library(cuda, n):
@@ -56,7 +63,10 @@ def test_special_contents_and_unaligned_base(cuda):
         assert delta._hex128(low, high) == _lib_hex(x[off:off + n]), off
     out = torch.zeros(2, dtype=torch.int64, device=cuda)
     ws = torch.empty(64, dtype=torch.int64, device=cuda)
-    assert lib.wq_xxh3_128(xg.data_ptr(), 240, ws.data_ptr(), out.data_ptr(), _lib.stream_ptr(cuda)) == -4     # short forms
+    assert lib.wq_xxh3_128(xg.data_ptr() + 3, 240, ws.data_ptr(), out.data_ptr(), _lib.stream_ptr(cuda)) == 0    # short form
+    assert delta._hex128(*out.tolist()) == _lib_hex(x[3:243])
+    assert lib.wq_xxh3_128(None, 0, ws.data_ptr(), out.data_ptr(), _lib.stream_ptr(cuda)) == 0
+    assert delta._hex128(*out.tolist()) == xxhash.xxh3_128(b"").hexdigest()
     assert lib.wq_xxh3_128(xg.data_ptr(), -1, ws.data_ptr(), out.data_ptr(), _lib.stream_ptr(cuda)) == -2
     assert lib.wq_xxh3_128(None, 1000, ws.data_ptr(), out.data_ptr(), _lib.stream_ptr(cuda)) == -1
 
@@ -72,7 +82,7 @@ def test_delta_encoder_uses_the_gpu_digest_by_default(cuda, monkeypatch):
     from slime_amd import delta_host
 
     def no_host(*a, **k):
-        raise AssertionError("the digest of a long tensor must not be computed on the host")
+        raise AssertionError("an xxh3-128 digest must not be computed on the host")
 
     monkeypatch.setattr(delta_host, "host_checksum", no_host)
     g = torch.Generator().manual_seed(9)

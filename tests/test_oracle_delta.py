@@ -50,19 +50,14 @@ def test_overwrite_encoding_layout_and_round_trip():
 
 
 def test_host_digests():
-    # the sequential digests stay on the host (slime/utils/disk_delta.py:40-58): xxh3-128 through `xxhash`, blake3
-    # through `blake3` when that package is installed (ImportError otherwise, as in the reference), KeyError for
-    # unknown names
+    # blake3 is the one digest left to the host (slime/utils/disk_delta.py:46-49): through the `blake3` package when it
+    # is installed (ImportError otherwise, as in the reference); unknown names raise KeyError, as the reference's do
     import torch
-    import xxhash
 
     from slime_amd.delta_host import host_checksum
 
-    assert host_checksum("xxh3-128", torch.empty(0, dtype=torch.uint8)) == "99aa06d3014798d86001c324468d497f"   # empty input
     w = torch.arange(1000, dtype=torch.float32).to(torch.bfloat16).view(20, 50)
     raw = w.view(torch.uint8).numpy().tobytes()
-    assert host_checksum("xxh3-128", w) == xxhash.xxh3_128(raw).hexdigest()
-    assert host_checksum("xxh3-128", w.t()) == xxhash.xxh3_128(w.t().contiguous().view(torch.uint8).numpy().tobytes()).hexdigest()
     try:
         import blake3
     except ImportError:
@@ -70,5 +65,6 @@ def test_host_digests():
             host_checksum("blake3", w)
     else:
         assert host_checksum("blake3", w) == blake3.blake3(raw).hexdigest()
-    with pytest.raises(KeyError):
-        host_checksum("md5", w)
+    for name in ("md5", "xxh3-128", "adler32"):
+        with pytest.raises(KeyError):
+            host_checksum(name, w)

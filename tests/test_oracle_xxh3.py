@@ -42,5 +42,14 @@ def test_block_sums_are_order_free_and_the_chain_is_not():
         shuffled = X.stripe_terms(words, keys)[np.random.default_rng(0).permutation(16)].sum(axis=0, dtype=np.uint64)
     assert np.array_equal(shuffled, s[0])
     assert not np.array_equal(X.chain(s), X.chain(s[::-1]))
-    with pytest.raises(ValueError):
-        X.xxh3_128(d[:240])
+
+
+def test_short_forms_every_length():
+    for n in range(0, 241):
+        for seed in (n, n + 1000):
+            d = _data(n, seed)
+            assert X.hexdigest(d) == xxhash.xxh3_128(d.tobytes()).hexdigest(), n
+    for n in (1, 3, 8, 16, 17, 128, 129, 240):
+        for fill in (0, 255):
+            d = np.full(n, fill, np.uint8)
+            assert X.hexdigest(d) == xxhash.xxh3_128(d.tobytes()).hexdigest(), (n, fill)
