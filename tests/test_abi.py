@@ -219,3 +219,25 @@ def test_no_mixed_precision_fma_in_the_dequantiser(tmp_path):
                            os.path.join(csrc, "wq_fp8_dequant.hip")], stderr=subprocess.DEVNULL)
     asm = out.read_text()
     assert "v_cvt_f16_f32" in asm and "fma_mix" not in asm and "mad_mix" not in asm
+
+
+def test_product_never_touches_the_oracle_or_falls_back_to_the_host():
+    """The package must not import, load or run anything under oracle/ (test infrastructure), and its entry points must
+    refuse to work without the HIP library rather than compute on the host."""
+    import glob
+
+    pkg = os.path.join(ROOT, "slime_amd")
+    for path in glob.glob(os.path.join(pkg, "**", "*.py"), recursive=True) + [os.path.join(ROOT, "fake_int4_quant_cuda.py")]:
+        text = open(path).read()
+        assert not re.search(r"^\s*(from|import)\s+oracle\b|libwq_oracle|oracle[/.]", text, re.M), path
+    import torch
+
+    import slime_amd
+
+    if not torch.cuda.is_available():
+        w = torch.zeros(128, 128, dtype=torch.bfloat16)
+        for call in (lambda: slime_amd.block_fp8(w, (128, 128)), lambda: slime_amd.pack_layer(w, 128, True),
+                     lambda: slime_amd.weight_dequant(w.view(torch.uint8)[:, :128].view(torch.float8_e4m3fn), torch.ones(1, 1)),
+                     lambda: slime_amd.fp8_aligned_weight(w), lambda: slime_amd.delta.checksum("xxh3-128", w)):
+            with pytest.raises(RuntimeError):
+                call()
