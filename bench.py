@@ -359,6 +359,17 @@ def bench_bucket(dev, steps, warmup, layers):
     torch.cuda.synchronize()
     evL = conv.kernel_ms() / steps
     launchesL = sum(b.launches for b in state["out"])
+    state["out"] = None
+    # the loop this replaces, on this build's own per-tensor kernels (so the difference is launches and copies, not
+    # arithmetic): quantize_params per Megatron parameter, then the flatten copy; two layers, scaled to all of them
+    sample = per_layer[:2]
+
+    def loop_and_flatten():
+        state["out"] = None
+        state["out"] = [B.flatten_named_tensors(B.per_param_loop(None, params, cfg)) for params in sample]
+
+    wallP, _, _ = _time_launches(loop_and_flatten, 3, 1)
+    state["out"] = None
     out = {"workload": f"Qwen3-30B-A3B-shaped state dict after name conversion, {layers} layers, {n_tensors} tensors "
                        f"({len(quantised)} quantised to block-FP8 with the weight-sync arithmetic, the rest copied), written "
                        "into the one uint8 buffer + metadata a FlattenedTensorBucket consumer reads; fresh output buffer per sync",
@@ -368,6 +379,11 @@ def bench_bucket(dev, steps, warmup, layers):
                           "bf16_GBps": 2 * elements / ev1 / 1e6},
            "bucket_per_layer": {"launches_per_sync": launchesL, "ms_per_sync_kernels": evL, "ms_per_sync_wall": wallL,
                                 "hbm_frac": algo_bytes / evL / 1e6 / HBM_PEAK_GBS, "bf16_GBps": 2 * elements / evL / 1e6},
+           "per_parameter_loop_then_flatten": {
+               "what": "quantize_params once per Megatron parameter (one cached-table launch each) followed by the flatten "
+                       "copy into one buffer, per layer bucket - the shape of the reference's loop, on this build's kernels",
+               "ms_per_sync_wall": wallP * layers / len(sample), "measured_on_layers": len(sample),
+               "quantiser_launches_per_sync": 258 * layers},
            "table_builds": conv.plan_builds, "parity_tensors_checked": 3}
     del state, conv, whole, per_layer, quantised
     torch.cuda.empty_cache()
