@@ -360,6 +360,36 @@ def bench_bucket(dev, steps, warmup, layers):
     evL = conv.kernel_ms() / steps
     launchesL = sum(b.launches for b in state["out"])
     state["out"] = None
+    # the INT4 weight sync of the same state dict: experts to compressed-tensors INT4 (symmetric, group 128, the
+    # converter's default ignore rules), everything else copied through; one bucket per layer
+    cfg4 = {"quant_method": "compressed-tensors",
+            "config_groups": {"group_0": {"weights": {"group_size": 128, "symmetric": True, "num_bits": 4}}},
+            "ignore": ["re:.*lm_head.*", "re:.*norm.*", "re:.*embed.*", "re:.*self_attn.*", "re:.*shared_experts.*",
+                       "re:.*mlp\\.(gate|up|gate_up|down)_proj.*", "re:.*mlp\\.gate\\.*"]}
+    conv4 = B.BucketConverter(None, cfg4)
+
+    def int4_per_layer():
+        state["out"] = None
+        state["out"] = [conv4.convert(params, bucket_id=i) for i, params in enumerate(per_layer)]
+
+    wall4, _, _ = _time_launches(int4_per_layer, steps, warmup)
+    conv4.time_kernels = True
+    for _ in range(steps):
+        int4_per_layer()
+    torch.cuda.synchronize()
+    ev4 = conv4.kernel_ms() / steps
+    launches4 = sum(b.launches for b in state["out"])
+    named4 = dict(state["out"][0].reconstruct_tensors())
+    n0, t0_ = quantised[4]                                   # an expert projection of layer 0
+    assert ".experts." in n0
+    po, so, _ = c_oracle.int4_pack_layer(t0_.cpu().contiguous(), 128, True)
+    assert torch.equal(named4[n0.replace(".weight", ".weight_packed")].cpu(), po)
+    assert torch.equal(named4[n0.replace(".weight", ".weight_scale")].cpu().view(torch.int16), so.view(torch.int16))
+    expert_el = sum(t.numel() for n, t in quantised if ".experts." in n)
+    passed = sum(t.numel() * t.element_size() for _, cv in whole for n, t in cv if ".experts." not in n)
+    algo4 = int(expert_el * 2.515625) + 2 * passed
+    del named4, conv4
+    state["out"] = None
     # the loop this replaces, on this build's own per-tensor kernels (so the difference is launches and copies, not
     # arithmetic): quantize_params per Megatron parameter, then the flatten copy; two layers, scaled to all of them
     sample = per_layer[:2]
@@ -379,6 +409,10 @@ def bench_bucket(dev, steps, warmup, layers):
                           "bf16_GBps": 2 * elements / ev1 / 1e6},
            "bucket_per_layer": {"launches_per_sync": launchesL, "ms_per_sync_kernels": evL, "ms_per_sync_wall": wallL,
                                 "hbm_frac": algo_bytes / evL / 1e6 / HBM_PEAK_GBS, "bf16_GBps": 2 * elements / evL / 1e6},
+           "int4_bucket_per_layer": {"what": "the same state dict through the compressed-tensors INT4 branch: 18 432 expert "
+                                             "weights packed (sym, group 128), attention / norms / router copied through",
+                                     "launches_per_sync": launches4, "ms_per_sync_kernels": ev4, "ms_per_sync_wall": wall4,
+                                     "hbm_frac": algo4 / ev4 / 1e6 / HBM_PEAK_GBS, "bf16_GBps": 2 * expert_el / ev4 / 1e6},
            "per_parameter_loop_then_flatten": {
                "what": "quantize_params once per Megatron parameter (one cached-table launch each) followed by the flatten "
                        "copy into one buffer, per layer bucket - the shape of the reference's loop, on this build's kernels",
