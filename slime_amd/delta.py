@@ -179,31 +179,53 @@ def _hex128(low: int, high: int) -> str:
     return f"{high & 0xFFFFFFFFFFFFFFFF:016x}{low & 0xFFFFFFFFFFFFFFFF:016x}"
 
 
+class Xxh3Plan:
+    """xxh3-128 of a fixed list of tensors: the descriptor table, the workspace (64 bytes per KiB) and the digest buffer
+    are set up once; ``run()`` is two launches and no host work, ``hexdigests()`` synchronises and formats.  The tensors
+    are hashed where they are, so they must stay contiguous at 16-byte aligned addresses (what ``run()`` hashes is their
+    content at that moment)."""
+
+    def __init__(self, tensors):
+        self.tensors = [_as_bytes(t, "Xxh3Plan") for t in tensors]
+        self.n = len(self.tensors)
+        if not self.n:
+            return
+        self.device = self.tensors[0].device
+        lib = _lib.load()
+        ws_off, total_ws, items, n_items = [], 0, [0], 0
+        for f in self.tensors:
+            n = f.numel()
+            ws_off.append(total_ws)
+            total_ws += (lib.wq_xxh3_workspace_bytes(n) + 255) // 256 * 256
+            n_items += -(-((n - 1) // 1024) // 16) if n > 0 else 0
+            items.append(n_items)
+        self._ws = torch.empty(total_ws // 8, dtype=torch.int64, device=self.device)
+        self.digests = torch.empty((self.n, 2), dtype=torch.int64, device=self.device)       # [low64, high64] per tensor
+        rows = [[f.data_ptr(), f.numel(), self._ws.data_ptr() + o, self.digests.data_ptr() + 16 * k]
+                for k, (f, o) in enumerate(zip(self.tensors, ws_off))]
+        self._descs = torch.tensor(rows, dtype=torch.int64).to(self.device)
+        self._starts = torch.tensor(items, dtype=torch.int64).to(self.device)
+        self._n_items = n_items
+
+    def run(self) -> torch.Tensor:
+        if self.n:
+            with torch.cuda.device(self.device):
+                rc = _lib.load().wq_xxh3_128_grouped(self._descs.data_ptr(), self._starts.data_ptr(), self.n, self._n_items,
+                                                     _lib.stream_ptr(self.device))
+            _lib.check(rc, "xxh3_128")
+            return self.digests
+        return torch.empty((0, 2), dtype=torch.int64)
+
+    def hexdigests(self) -> list:
+        return [_hex128(low, high) for low, high in self.digests.tolist()] if self.n else []
+
+
 def xxh3_128_many(tensors) -> list:
     """``xxhash.xxh3_128(bytes of t).hexdigest()`` for every tensor, computed on the GPU with two launches and one
     synchronisation.  -> list of 32-digit hex strings."""
-    flats = [_as_bytes(t, "xxh3_128") for t in tensors]
-    if not flats:
-        return []
-    device = flats[0].device
-    lib = _lib.load()
-    ws_off, total_ws, items, n_items = [], 0, [0], 0
-    for f in flats:
-        n = f.numel()
-        ws_off.append(total_ws)
-        total_ws += (lib.wq_xxh3_workspace_bytes(n) + 255) // 256 * 256
-        n_items += -(-((n - 1) // 1024) // 16) if n > 0 else 0
-        items.append(n_items)
-    ws = torch.empty(total_ws // 8, dtype=torch.int64, device=device)
-    digests = torch.empty((len(flats), 2), dtype=torch.int64, device=device)
-    rows = [[f.data_ptr(), f.numel(), ws.data_ptr() + o, digests.data_ptr() + 16 * k]
-            for k, (f, o) in enumerate(zip(flats, ws_off))]
-    descs = torch.tensor(rows, dtype=torch.int64).to(device)
-    starts = torch.tensor(items, dtype=torch.int64).to(device)
-    with torch.cuda.device(device):
-        rc = lib.wq_xxh3_128_grouped(descs.data_ptr(), starts.data_ptr(), len(flats), n_items, _lib.stream_ptr(device))
-    _lib.check(rc, "xxh3_128")
-    return [_hex128(low, high) for low, high in digests.tolist()]
+    plan = Xxh3Plan(tensors)
+    plan.run()
+    return plan.hexdigests()
 
 
 def xxh3_128(buf: torch.Tensor) -> str:

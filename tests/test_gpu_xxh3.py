@@ -39,6 +39,15 @@ def test_many_tensors_two_launches(cuda):
     xs = [_bytes(n, 50 + i) for i, n in enumerate(sizes)]
     got = delta.xxh3_128_many([x.to(cuda) for x in xs])
     assert got == [_lib_hex(x) for x in xs]
+    plan = delta.Xxh3Plan([x.to(cuda) for x in xs])
+    for _ in range(2):                       # a plan is reusable: it hashes what the tensors hold when run() is called
+        plan.run()
+        assert plan.hexdigests() == got
+    plan.tensors[6][:100] ^= 0xFF
+    plan.run()
+    again = plan.hexdigests()
+    assert again[6] != got[6] and again[:6] == got[:6] and again[7:] == got[7:]
+    assert delta.Xxh3Plan([]).hexdigests() == [] and delta.xxh3_128_many([]) == []
     # bf16 weights and views: the digest is over the bytes of the contiguous tensor, as tensor.contiguous().view(uint8) gives
     g = torch.Generator().manual_seed(1)
     w = (torch.randn(300, 520, generator=g) * 0.02).to(torch.bfloat16)
