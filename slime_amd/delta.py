@@ -32,6 +32,15 @@ def _as_bytes(t: torch.Tensor, what: str) -> torch.Tensor:
     return flat
 
 
+def _as_bytes_in_place(t: torch.Tensor, what: str) -> torch.Tensor:
+    """For plans, which read the tensor again on every run: a byte view of the tensor itself, never a copy."""
+    _lib.require_gpu(t, what)
+    if not t.is_contiguous() or t.data_ptr() % 16:
+        raise ValueError(f"{what}: tensors of a plan must be contiguous at 16-byte aligned addresses (a copy would be "
+                         f"hashed / diffed instead of the live weight); got strides {t.stride()}, address % 16 = {t.data_ptr() % 16}")
+    return t.detach().view(torch.uint8).reshape(-1)
+
+
 def _workspace(n: int, device) -> torch.Tensor:
     return torch.empty(_lib.load().wq_delta_workspace_bytes(n) // 8, dtype=torch.int64, device=device)
 
@@ -110,7 +119,7 @@ class XorDiffPlan:
     def __init__(self, news, olds, want_diff: bool = True):
         if not news or len(news) != len(olds):
             raise ValueError("XorDiffPlan: need one snapshot per tensor and at least one tensor")
-        self.news = [_as_bytes(t, "XorDiffPlan") for t in news]
+        self.news = [_as_bytes_in_place(t, "XorDiffPlan") for t in news]
         self.olds = list(olds)
         self.want_diff = bool(want_diff)
         device = self.news[0].device
@@ -185,8 +194,8 @@ class Xxh3Plan:
     are hashed where they are, so they must stay contiguous at 16-byte aligned addresses (what ``run()`` hashes is their
     content at that moment)."""
 
-    def __init__(self, tensors):
-        self.tensors = [_as_bytes(t, "Xxh3Plan") for t in tensors]
+    def __init__(self, tensors, in_place: bool = True):
+        self.tensors = [(_as_bytes_in_place if in_place else _as_bytes)(t, "Xxh3Plan") for t in tensors]
         self.n = len(self.tensors)
         if not self.n:
             return
@@ -223,7 +232,7 @@ class Xxh3Plan:
 def xxh3_128_many(tensors) -> list:
     """``xxhash.xxh3_128(bytes of t).hexdigest()`` for every tensor, computed on the GPU with two launches and one
     synchronisation.  -> list of 32-digit hex strings."""
-    plan = Xxh3Plan(tensors)
+    plan = Xxh3Plan(tensors, in_place=False)       # one-shot: unaligned or strided inputs may be hashed from a copy
     plan.run()
     return plan.hexdigests()
 

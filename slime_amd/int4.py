@@ -366,8 +366,11 @@ class Int4DequantPlan:
                     or sc.numel() != M * (N // self.group) or p.device != self.device or sc.device != self.device:
                 raise ValueError(f"Int4DequantPlan: packed {tuple(p.shape)} {p.dtype} / scale {tuple(sc.shape)} {sc.dtype} "
                                  f"do not describe a [{M}, {N}] weight with groups of {self.group}")
-            self.packeds.append(p.contiguous())
-            self.scales.append(sc.contiguous())
+            if not p.is_contiguous() or not sc.is_contiguous():
+                # a plan reads its inputs again on every run: a silent copy would freeze them at construction time
+                raise ValueError("Int4DequantPlan: packed weights and scales must be contiguous")
+            self.packeds.append(p)
+            self.scales.append(sc)
             y_off.append(total)
             total += (M * N + 127) // 128 * 128
         self.flat_y = torch.empty(max(total, 1), dtype=torch.bfloat16, device=self.device)

@@ -165,3 +165,24 @@ def test_unknown_digest_names(cuda):
     with pytest.raises(KeyError):
         delta.checksum("md5", x)
     assert delta.checksum("xxh3-128", x[:0]) == "99aa06d3014798d86001c324468d497f"      # XXH3_128bits of the empty input
+
+
+def test_plans_refuse_inputs_they_would_have_to_copy(cuda):
+    """A plan reads its tensors again on every run; an unaligned or strided tensor would be frozen into a copy at
+    construction time, so it is refused (the one-shot functions copy and are fine)."""
+    base = torch.zeros(4096 + 16, dtype=torch.uint8, device=cuda)
+    odd = base[1:4097]                                   # 1 byte off a 16-byte boundary
+    strided = torch.zeros(64, 128, dtype=torch.bfloat16, device=cuda)[:, ::2]
+    for bad in (odd, strided):
+        with pytest.raises(ValueError, match="contiguous at 16-byte aligned"):
+            delta.Xxh3Plan([bad])
+        with pytest.raises(ValueError, match="contiguous at 16-byte aligned"):
+            delta.XorDiffPlan([bad], [torch.zeros(bad.numel() * bad.element_size(), dtype=torch.uint8, device=cuda)])
+        assert len(delta.xxh3_128(bad)) == 32            # one-shot form: hashed from a copy
+    good = base[:4096]
+    plan = delta.Xxh3Plan([good])
+    plan.run()
+    before = plan.hexdigests()
+    good[7] = 9                                          # the live tensor changes ...
+    plan.run()
+    assert plan.hexdigests() != before                   # ... and the plan sees it
