@@ -23,7 +23,15 @@ namespace wq {
 constexpr int kDeltaSteps = 4;
 constexpr int kDeltaChunk = WQ_DELTA_CHUNK;          // bytes of each input per workgroup
 constexpr int kDeltaItemsPerXcdRun = 32;
-constexpr int kDeltaOccupancyPadBytes = 0;           // unused dynamic LDS that caps workgroups per CU
+// Residency and bytes in flight, measured on the Qwen3-4B-shaped state dict (xor diff + snapshot update, % of the 8 TB/s
+// HBM peak at 4 bytes of traffic per byte; the plain copy kernel reached 72.5 % on that box).  Workgroups per CU x steps
+// in flight per lane (a step = one 16-byte piece of each input):
+//   8 x 4 (everything at once, full occupancy)   70.6        4 x 4   74.3        3 x 4   76.0        2 x 4   77.2
+//   8 x 2   70.2      4 x 2   74.9      3 x 2   77.4      2 x 2   75.4
+//   8 x 1   70.0      7 x 1   71.3      4 x 1   74.8      3 x 1   78.1 - 78.7  <- used      2 x 1   69.2      1 x 1   40.5
+// The fewer bytes a CU has in flight, the better this memory system streams - down to about 24 KiB per CU.
+constexpr int kDeltaOccupancyPadBytes = 50 * 1024;   // unused dynamic LDS that caps workgroups per CU: 3
+constexpr int kDeltaWindow = 1;                      // steps (a 16-byte piece of each input per lane) in flight
 constexpr uint32_t kAdlerMod = 65521u;
 static_assert(kDeltaChunk == 256 * 16 * kDeltaSteps, "chunk = 256 lanes x 16 bytes x steps");
 
@@ -78,21 +86,29 @@ __device__ __forceinline__ void delta_xor_chunk(const uint8_t* __restrict__ nw, 
 {
     const int64_t base = item * kDeltaChunk;
     u32x4 a[kDeltaSteps], b[kDeltaSteps];
-    if (n >= 16) {
+    const bool whole = n >= 16;
+    auto issue = [&](int i) {
+        // lanes past the end re-read the last whole piece instead of branching around the load
+        const int64_t off = base + (int64_t)(i * 256 + threadIdx.x) * 16;
+        const int64_t safe = min(off, (n / 16 - 1) * 16);
+        a[i] = ldg_nt<u32x4>(nw + safe);
+        b[i] = ldg_nt<u32x4>(old + safe);
+    };
+    if (whole) {
 #pragma unroll
-        for (int i = 0; i < kDeltaSteps; ++i) {
-            // lanes past the end re-read the last whole piece instead of branching around the load
-            const int64_t off = base + (int64_t)(i * 256 + threadIdx.x) * 16;
-            const int64_t safe = min(off, (n / 16 - 1) * 16);
-            a[i] = ldg_nt<u32x4>(nw + safe);
-            b[i] = ldg_nt<u32x4>(old + safe);
-        }
+        for (int i = 0; i < kDeltaWindow && i < kDeltaSteps; ++i) issue(i);
     }
     // W of the chunk = P + 4096 * Q with P = sum over pieces of (16 * lane) * s + r and Q = sum of step * s:
     // both stay far below 2^32 per row, so the reduction runs on dwords
     uint32_t changed = 0, s_lane = 0, p_lane = 0, q_lane = 0;
 #pragma unroll
     for (int i = 0; i < kDeltaSteps; ++i) {
+        if (kDeltaWindow < kDeltaSteps) {
+            // a rolling window: the pieces of step i + window are requested once those of step i are about to be used
+            asm volatile("" :: "v"(a[i].x), "v"(b[i].x));
+            if (whole && i + kDeltaWindow < kDeltaSteps) issue(i + kDeltaWindow);
+            __builtin_amdgcn_sched_barrier(0);
+        }
         const uint32_t local = (uint32_t)(i * 256 + threadIdx.x) * 16;
         const int64_t off = base + local;
         int valid = 16;

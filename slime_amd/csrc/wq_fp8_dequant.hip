@@ -24,6 +24,7 @@ constexpr int kSteps = kSegsPerWg / 4;           // loads in flight per lane
 // segments per workgroup x resident workgroups per CU: 32x8 74.0, 32x4 79.3, 16x8 76.5, 16x5 79.4 (used),
 // 16x4 78.2, 8x8 79.7, 8x5 73.1.  A compute-free kernel with the same 1:2 read:write mix tops out at 83 %.
 constexpr int kDeqItemsPerXcdRun = 32;
+constexpr int kDeqWindow = 4;                          // steps whose loads are in flight (kSteps = all)
 constexpr unsigned kDeqOccupancyPadBytes = 27 * 1024;  // unused dynamic LDS: at most 5 workgroups per CU
 static_assert(kSeg == 512 && kSegsPerWg % 4 == 0, "a segment is 64 lanes x 8 codes; four waves per workgroup");
 
@@ -133,11 +134,10 @@ __global__ __launch_bounds__(256) void fp8_block_dequant_kernel(const DeqArgs a,
         float sc[kSteps];
         uint32_t row[kSteps], col[kSteps];
         bool ok[kSteps];
-        // Phase 1: issue every load of the workgroup's strip - codes and their block scales - before any
+        // The loads of the workgroup's strip - codes and their block scales - run kDeqWindow steps ahead of their
         // use.  Lanes with nothing to do read the tensor's first codes / scale instead of branching
         // around the load: a predicated load makes the compiler wait for earlier loads first.
-#pragma unroll
-        for (int i = 0; i < kSteps; ++i) {
+        auto issue = [&](int i) {
             row[i] = r;
             col[i] = c * kSeg + lane * 8;
             ok[i] = seg0 + 4 * i < n_segs && col[i] < N;
@@ -147,9 +147,16 @@ __global__ __launch_bounds__(256) void fp8_block_dequant_kernel(const DeqArgs a,
             sc[i] = ldg<float>(d.s + (ok[i] ? sr * kt + sc_col : 0));
             c += 4;
             while (c >= spr) { c -= spr; ++r; }
-        }
+        };
+#pragma unroll
+        for (int i = 0; i < kDeqWindow && i < kSteps; ++i) issue(i);
 #pragma unroll
         for (int i = 0; i < kSteps; ++i) {
+            if (kDeqWindow < kSteps) {
+                asm volatile("" :: "v"(v[i].x), "v"(sc[i]));
+                if (i + kDeqWindow < kSteps) issue(i + kDeqWindow);
+                __builtin_amdgcn_sched_barrier(0);
+            }
             if (!ok[i]) continue;
             if (MODE == WQ_DEQ_MODE_BF16SCALE) sc[i] = u2f(f32_to_bf16_bits(sc[i]) << 16);
             const uint64_t off = (uint64_t)row[i] * N + col[i];

@@ -25,6 +25,7 @@ constexpr int kFakeLoads = 128 / kFakeRowSlots;
 // 8 / 16 / 32 / 64 tiles per XCD: 73.5 / 74.2 / 74.4 / 74.1.  The quantiser followed by the dequantiser: 78.8 % of their
 // 6 bytes per element, i.e. 1.42x the time.
 constexpr int kFakeTilesPerXcdRun = 32;
+constexpr int kFakeWindow = 8;                          // 16-byte loads in flight per lane (8 = the whole tile)
 constexpr unsigned kFakeOccupancyPadBytes = 50 * 1024;  // unused dynamic LDS: at most 3 workgroups per CU
 
 struct FakeArgs {
@@ -66,26 +67,40 @@ __device__ __forceinline__ void fake_tile_vec128(const FakeArgs& a, int64_t tm, 
     const bool full = rows == 128 && pieces == 16;
     const uint32_t coff = (uint32_t)min(cc, pieces - 1) * 16u;
 
-    // every lane loads from a valid address (row and piece clamped into the tile); lanes outside the tensor are zeroed
+    // every lane loads from a valid address (row and piece clamped into the tile); lanes outside the tensor are zeroed.
+    // Full tiles keep kFakeWindow loads in flight per lane while the block maximum is folded (see the quantiser).
     u32x4 v[kFakeLoads];
+    uint32_t m = 0;
+    if (full) {
 #pragma unroll
-    for (int i = 0; i < kFakeLoads; ++i) {
-        const uint32_t r = full ? (uint32_t)(rb + kFakeRowSlots * i) : (uint32_t)min(rb + kFakeRowSlots * i, rows - 1);
-        v[i] = ldg_nt<u32x4>(xt + (r * xrow + coff));
-    }
-    if (!full) {
+        for (int i = 0; i < kFakeWindow && i < kFakeLoads; ++i)
+            v[i] = ldg_nt<u32x4>(xt + ((uint32_t)(rb + kFakeRowSlots * i) * xrow + coff));
+#pragma unroll
+        for (int i = 0; i < kFakeLoads; ++i) {
+            m = pk_absmax(m, v[i].x);
+            m = pk_absmax(m, v[i].y);
+            m = pk_absmax(m, v[i].z);
+            m = pk_absmax(m, v[i].w);
+            __builtin_amdgcn_sched_barrier(0);
+            if (i + kFakeWindow < kFakeLoads)
+                v[i + kFakeWindow] = ldg_nt<u32x4>(xt + ((uint32_t)(rb + kFakeRowSlots * (i + kFakeWindow)) * xrow + coff));
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < kFakeLoads; ++i) {
+            const uint32_t r = (uint32_t)min(rb + kFakeRowSlots * i, rows - 1);
+            v[i] = ldg_nt<u32x4>(xt + (r * xrow + coff));
+        }
 #pragma unroll
         for (int i = 0; i < kFakeLoads; ++i)
             if (!(col_ok && rb + kFakeRowSlots * i < rows)) v[i] = (u32x4){0u, 0u, 0u, 0u};
-    }
-
-    uint32_t m = 0;
 #pragma unroll
-    for (int i = 0; i < kFakeLoads; ++i) {
-        m = pk_absmax(m, v[i].x);
-        m = pk_absmax(m, v[i].y);
-        m = pk_absmax(m, v[i].z);
-        m = pk_absmax(m, v[i].w);
+        for (int i = 0; i < kFakeLoads; ++i) {
+            m = pk_absmax(m, v[i].x);
+            m = pk_absmax(m, v[i].y);
+            m = pk_absmax(m, v[i].z);
+            m = pk_absmax(m, v[i].w);
+        }
     }
     m = row16_max_u32(pk_fold(m));
     if (cc == 0) lds[rb] = m;

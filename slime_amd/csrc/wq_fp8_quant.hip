@@ -1,9 +1,9 @@
 // bf16 -> block-FP8 (e4m3fn) quantisation for gfx950.
 //
 // Vector kernel (128x128 blocks, unit column stride, 16-byte aligned rows): one 256-thread
-// workgroup owns one block.  Each lane issues eight 16-byte loads (8 bf16 each, rows rb+16*i), so a
-// wavefront load covers four 256-byte row segments and the whole 32 KiB block is in flight before
-// the first use.  The block lives in registers from then on: amax is an integer max over the bf16
+// workgroup owns one block.  Each lane issues eight 16-byte loads (8 bf16 each, rows rb+16*i; a
+// wavefront load covers four 256-byte row segments), a few at a time (kTileWindow), and the 32 KiB block lives in
+// registers from then on: amax is an integer max over the bf16
 // magnitude bits (packed 16-bit max), reduced over 16 lanes with DPP and across the workgroup
 // through 64 bytes of LDS; the scale is computed once; every element is divided with a
 // reciprocal + two FMA refinement that equals the IEEE quotient, converted with v_cvt_pk_fp8_f32
@@ -29,6 +29,13 @@ namespace wq {
 constexpr int kTileThreads = 256;
 constexpr int kTilesPerXcdRun = 32;               // consecutive tiles handed to one XCD (xcd_chunked_item)
 constexpr unsigned kOccupancyPadBytes = 36 * 1024;  // unused dynamic LDS: caps residency at 4 workgroups per CU
+// 16-byte loads a lane keeps in flight while it folds the block maximum: the load of step i + window is issued when step
+// i has been folded in.  On the full Qwen3-30B-A3B-shaped state dict (4 workgroups per CU): all 8 at once 79.1 %, 6: 79.5,
+// 4: 79.1, 3: 79.5, 2: 80.6-80.8 (used), 1: 72.1; with 5 or more workgroups per CU a window lowers the rate.  The
+// Qwen3-4B-shaped pass does not move (76.3-76.6 either way).  A compute-free 2:1 stream of the same shape is fastest at 2
+// workgroups per CU (84 %): fewer bytes in flight per CU suit the memory system, and the window gets part of that while
+// four workgroups keep the arithmetic overlapped.
+constexpr int kTileWindow = 2;
 constexpr int kRowSlots = kTileThreads / 16;   // rows covered by one load step of the workgroup
 constexpr int kTileLoads = 128 / kRowSlots;    // 16-byte loads per lane
 constexpr int kTileWaves = kTileThreads / 64;
@@ -68,9 +75,19 @@ __device__ __forceinline__ void quant_tile_vec128(const wq_fp8_quant_desc& d, in
     const bool full = (tm * 128 + 128 <= d.M) && (tn * 128 + 128 <= d.N);
 
     u32x4 v[kTileLoads];
+    uint32_t m = 0;
     if (full) {
 #pragma unroll
-        for (int i = 0; i < kTileLoads; ++i) v[i] = ldg_nt<u32x4>(xt + (xoff + i * xstep));
+        for (int i = 0; i < kTileWindow && i < kTileLoads; ++i) v[i] = ldg_nt<u32x4>(xt + (xoff + i * xstep));
+#pragma unroll
+        for (int i = 0; i < kTileLoads; ++i) {
+            m = pk_absmax(m, v[i].x);
+            m = pk_absmax(m, v[i].y);
+            m = pk_absmax(m, v[i].z);
+            m = pk_absmax(m, v[i].w);
+            __builtin_amdgcn_sched_barrier(0);      // keep the next load behind this step's use of its data
+            if (i + kTileWindow < kTileLoads) v[i + kTileWindow] = ldg_nt<u32x4>(xt + (xoff + (i + kTileWindow) * xstep));
+        }
     } else {
         // Edge tile: every lane loads from a valid address - its row and piece clamped into the tile - and the lanes
         // outside the tensor are zeroed afterwards.  (Loads predicated per lane make the compiler wait for the earlier
@@ -88,13 +105,14 @@ __device__ __forceinline__ void quant_tile_vec128(const wq_fp8_quant_desc& d, in
             if (!(col_ok && kRowSlots * i < rows_left)) v[i] = (u32x4){0u, 0u, 0u, 0u};
     }
 
-    uint32_t m = 0;
+    if (!full) {
 #pragma unroll
-    for (int i = 0; i < kTileLoads; ++i) {
-        m = pk_absmax(m, v[i].x);
-        m = pk_absmax(m, v[i].y);
-        m = pk_absmax(m, v[i].z);
-        m = pk_absmax(m, v[i].w);
+        for (int i = 0; i < kTileLoads; ++i) {
+            m = pk_absmax(m, v[i].x);
+            m = pk_absmax(m, v[i].y);
+            m = pk_absmax(m, v[i].z);
+            m = pk_absmax(m, v[i].w);
+        }
     }
     m = row16_max_u32(pk_fold(m));
     if (cc == 0) lds[rb] = m;

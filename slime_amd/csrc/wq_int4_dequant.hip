@@ -106,6 +106,7 @@ __global__ __launch_bounds__(256) void int4_dequant_any_kernel(const uint32_t* _
 constexpr int kSteGroupsPerWg = 64;
 constexpr int kSteItemsPerXcdRun = 32;
 constexpr int kSteOccupancyPadBytes = 36 * 1024;
+constexpr int kSteWindow = 4;                     // 16-byte loads in flight per lane (4 = all of a work item with 128-element groups)
 
 // ITEMS: one pre-resolved descriptor per work item (many tensors in one launch), pointing at the item's first group.
 template <int L, bool ITEMS>
@@ -128,13 +129,19 @@ __global__ __launch_bounds__(256) void int4_fake_ste_kernel(const uint16_t* __re
         g0 = cl;
     }
     u32x4 v[STEPS];
-#pragma unroll
-    for (int i = 0; i < STEPS; ++i) {
+    auto issue = [&](int i) {
         const int64_t g = min(g0 + i * CL, n_groups - 1);
         v[i] = ldg_nt<u32x4>(x + g * (8 * L) + ll * 8);
-    }
+    };
+#pragma unroll
+    for (int i = 0; i < kSteWindow && i < STEPS; ++i) issue(i);
 #pragma unroll
     for (int i = 0; i < STEPS; ++i) {
+        if (kSteWindow < STEPS) {
+            asm volatile("" :: "v"(v[i].x));
+            if (i + kSteWindow < STEPS) issue(i + kSteWindow);
+            __builtin_amdgcn_sched_barrier(0);
+        }
         const int64_t g = g0 + i * CL;
         const uint32_t wd[4] = {v[i].x, v[i].y, v[i].z, v[i].w};
         float xs[8];

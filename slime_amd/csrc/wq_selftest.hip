@@ -123,16 +123,21 @@ __global__ void selftest_decode_fp8_kernel(uint64_t* out)
     if (bad) report(out, c);
 }
 
-__global__ __launch_bounds__(256) void copy_kernel(const u32x4* __restrict__ src, u32x4* __restrict__ dst, int64_t n16)
+// A plain copy, launched the way that streams fastest on this part (measured with a compute-free sweep over work order,
+// residency and loads per lane): runs of 64 consecutive 16 KiB items per XCD, two workgroups per CU, four 16-byte loads
+// per lane in flight.  In dispatch order at full occupancy the same copy is 10 points slower.
+constexpr int kCopyItemsPerXcdRun = 64;
+constexpr unsigned kCopyOccupancyPadBytes = 77 * 1024;
+
+__global__ __launch_bounds__(256) void copy_kernel(const u32x4* __restrict__ src, u32x4* __restrict__ dst, int64_t n16,
+                                                   int64_t items)
 {
-    const int64_t base = ((int64_t)blockIdx.x + (int64_t)blockIdx.y * gridDim.x) * 1024 + threadIdx.x;
+    const int64_t slot = (int64_t)blockIdx.x + (int64_t)blockIdx.y * gridDim.x;
+    if (slot >= items) return;
+    const int64_t base = xcd_chunked_item(slot, items, kCopyItemsPerXcdRun) * 1024 + threadIdx.x;
     u32x4 v[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int64_t k = base + i * 256;
-        v[i] = (u32x4){0u, 0u, 0u, 0u};
-        if (k < n16) v[i] = __builtin_nontemporal_load(src + k);
-    }
+    for (int i = 0; i < 4; ++i) v[i] = __builtin_nontemporal_load(src + min(base + i * 256, n16 - 1));
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int64_t k = base + i * 256;
@@ -236,7 +241,10 @@ WQ_EXPORT int wq_copy_bytes(const void* src, void* dst, int64_t n_bytes, void* s
     if (!src || !dst) return WQ_ERR_NULL;
     if (((uintptr_t)src & 15) || ((uintptr_t)dst & 15)) return WQ_ERR_ALIGN;
     const int64_t n16 = n_bytes / 16;
-    copy_kernel<<<grid_for_items(cdiv64(n16, 1024)), 256, 0, (hipStream_t)stream>>>((const u32x4*)src, (u32x4*)dst, n16);
+    if (n16 == 0) return WQ_OK;
+    const int64_t items = cdiv64(n16, 1024);
+    copy_kernel<<<grid_for_items(items), 256, kCopyOccupancyPadBytes, (hipStream_t)stream>>>((const u32x4*)src, (u32x4*)dst,
+                                                                                           n16, items);
     WQ_LAUNCH_CHECK();
     return WQ_OK;
 }
