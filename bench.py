@@ -86,7 +86,7 @@ KERNEL_SOURCES = {
     "int4_pack": ("wq_int4.hip", "wq_common.h"),
     "fp8_block_dequant": ("wq_fp8_dequant.hip", "wq_common.h"),
     "int4_dequant": ("wq_int4_dequant.hip", "wq_common.h"),
-    "delta_xor": ("wq_delta.hip", "wq_common.h"),
+    "delta_xor": ("wq_delta.hip", "wq_common.h", "wq_xxh3_common.h"),
     "fp8_fake_quant": ("wq_fp8_fake.hip", "wq_common.h"),
 }
 
@@ -592,7 +592,8 @@ def bench_delta(dev, steps, warmup):
     assert results[5].tolist() == [changed, int(delta_ref.adler32_ref(check_new), 16)] and changed == 4096
     nbytes = sum(nw.numel() for nw in news)
     xxh3 = _bench_xxh3(news, steps, warmup)
-    out = {"xxh3_128": xxh3,
+    fused = _bench_delta_with_digest(news, olds, steps, warmup)
+    out = {"xxh3_128": xxh3, "with_xxh3_digest": fused,
            "workload": "Qwen3-4B-shaped state dict (252 bf16 tensors, 7.27 GB) against its snapshot in HBM: xor diff, "
                        "changed-byte count, adler32, snapshot update; two launches for the whole bucket",
            "tensors": len(news), "weight_GB": nbytes / 1e9, "kernel_ms": ev_ms, "wall_ms": wall_ms,
@@ -601,6 +602,41 @@ def bench_delta(dev, steps, warmup):
     del news, olds, plan
     torch.cuda.empty_cache()
     return out
+
+
+def _bench_delta_with_digest(news, olds, steps, warmup):
+    """The delta pass with the default digest riding on it: the bytes the diff reads also feed XXH3's block sums, one more
+    launch walks them - three launches for diff, counts, adler32, snapshot update and xxh3-128 of the whole bucket."""
+    import torch
+
+    from slime_amd import delta
+
+    plan = delta.XorDiffPlan(news, olds, xxh3=True)
+    wall_ms, ev_ms, _ = _time_launches(lambda: plan.run(update_snapshot=True), steps, warmup)
+    news[2][100:200] ^= 5
+    plan.run(update_snapshot=True)
+    got = plan.hexdigests()
+    assert got[2] == delta.xxh3_128(news[2]) and all(g is None for i, g in enumerate(got) if i != 2)
+    # timed runs above ran on an unchanged bucket (no digest walk); time the walk with every tensor changed
+    torch.cuda.synchronize()
+    t = []
+    for _ in range(max(steps // 2, 3)):
+        for old in olds:
+            old[0] ^= 1                                     # one byte per tensor differs again: every digest is walked
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        plan.run(update_snapshot=True)
+        e1.record()
+        torch.cuda.synchronize()
+        t.append(e0.elapsed_time(e1))
+    assert plan.results[:, 0].tolist() == [1] * len(news) and plan.hexdigests()[4] == delta.xxh3_128(news[4])
+    nbytes = sum(nw.numel() for nw in news)
+    ms = sum(t) / len(t)
+    return {"workload": "the same pass with the xxh3-128 digest of every tensor computed from the bytes the diff reads "
+                        "(64 bytes of block sums per KiB written by the diff kernel, then the per-tensor walk): three launches",
+            "ms_all_tensors_changed": ms, "ms_no_tensor_changed": ev_ms, "weight_GBps": nbytes / ms / 1e6,
+            "hbm_frac_of_diff_kernel_when_unchanged": (4 + 1 / 16) * nbytes / ev_ms / 1e6 / HBM_PEAK_GBS}
 
 
 def _bench_xxh3(news, steps, warmup):

@@ -32,7 +32,7 @@
 extern "C" {
 #endif
 
-#define WQ_ABI_VERSION 15
+#define WQ_ABI_VERSION 16
 
 enum {
     WQ_OK = 0,
@@ -372,21 +372,31 @@ int wq_delta_xor_noalloc(const void *new_bytes, void *old_bytes, void *diff, int
  * whose fields mean what the arguments of wq_delta_xor mean (a tensor with n == 0 is allowed); `chunk_start`
  * is a DEVICE int64[n_desc+1] exclusive prefix sum of ceil(n / WQ_DELTA_CHUNK); total_chunks = chunk_start[n_desc].
  * With write_diff == 0 the `diff` fields are ignored.  The entry point cannot check alignment of the pointers
- * inside `descs`: the caller guarantees what wq_delta_xor checks. */
+ * inside `descs`: the caller guarantees what wq_delta_xor checks.
+ *
+ * with_xxh3 != 0 adds the XXH3-128 digest of the new bytes of every tensor that changed - checksum("xxh3-128", new),
+ * the digest diff_and_compress attaches by default (slime/utils/disk_delta.py:40-58) - to the same pass: the bytes
+ * the diff reads anyway also feed the per-block sums (written to `xxh3_sums`: wq_xxh3_workspace_bytes(n) bytes,
+ * 16-byte aligned), and one more small launch walks them into `xxh3_digest` ({low64, high64}, as wq_xxh3_128).  A
+ * tensor with result[0] == 0 gets the digest {0, 0}: nothing is published for it.  With with_xxh3 == 0 the two
+ * fields are ignored. */
 typedef struct wq_delta_desc {
     const void *new_bytes;
     void *old_bytes;
     void *diff;
     int64_t n;
-    void *workspace;     /* wq_delta_workspace_bytes(n) bytes */
-    uint64_t *result;    /* 2 x uint64 */
+    void *workspace;        /* wq_delta_workspace_bytes(n) bytes */
+    uint64_t *result;       /* 2 x uint64 */
+    uint64_t *xxh3_sums;    /* with_xxh3: wq_xxh3_workspace_bytes(n) bytes */
+    uint64_t *xxh3_digest;  /* with_xxh3: 2 x uint64 */
 } wq_delta_desc;
 int wq_delta_xor_grouped(const wq_delta_desc *descs, const int64_t *chunk_start, int n_desc,
-                         int64_t total_chunks, int write_diff, int update_old, void *stream);
+                         int64_t total_chunks, int write_diff, int update_old, int with_xxh3, void *stream);
 
 /* wq_delta_xor_grouped with the owner of every chunk resolved beforehand: `items` holds one descriptor per
- * WQ_DELTA_CHUNK of every tensor (the tensor's buffers and the chunk's index inside it); `descs` is still needed,
- * per tensor, by the pass that folds the per-chunk sums into `result`. */
+ * WQ_DELTA_CHUNK of every tensor (the tensor's buffers and the chunk's index inside it; 64 bytes, so that an item is
+ * one aligned scalar load); `descs` is still needed, per tensor, by the passes that fold the per-chunk sums into
+ * `result` and walk the digest. */
 typedef struct wq_delta_chunk_item {
     const void *new_bytes;
     void *old_bytes;
@@ -394,9 +404,15 @@ typedef struct wq_delta_chunk_item {
     int64_t n;
     void *workspace;
     int64_t chunk;
+    uint64_t *xxh3_sums;    /* the tensor's, as in its wq_delta_desc */
+    int64_t reserved;
 } wq_delta_chunk_item;
 int wq_delta_xor_items(const wq_delta_chunk_item *items, int64_t n_items, const wq_delta_desc *descs, int n_desc,
-                       int write_diff, int update_old, void *stream);
+                       int write_diff, int update_old, int with_xxh3, void *stream);
+
+/* wq_delta_xor plus the digest, for one tensor: xxh3_workspace and digest as in wq_xxh3_128. */
+int wq_delta_xor_xxh3(const void *new_bytes, void *old_bytes, void *diff, int64_t n, int update_old,
+                      void *workspace, uint64_t *result, uint64_t *xxh3_workspace, uint64_t *digest, void *stream);
 
 /* ---------------------------------------------------------------------------------------------
  * XXH3-128 (seed 0) of n >= 0 bytes in device memory: the digest checksum("xxh3-128", new) attaches to every

@@ -15,7 +15,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libslime_amd_wq.so")
 
-ABI_VERSION = 15
+ABI_VERSION = 16
 
 # selectors (mirrors of the header's enums)
 DTYPE_BF16, DTYPE_F32, DTYPE_F16, DTYPE_F64 = 0, 1, 2, 3
@@ -52,7 +52,7 @@ SIGNATURES = {
     "wq_int4_group_quant_pack_asym_items": [_vp, _i64, _vp, _vp, _int, _vp],
     "wq_int4_zero_point_pack_grouped": [_vp, _vp, _int, _i64, _vp, _vp, _vp],
     "wq_int4_fake_quant_ste_items": [_vp, _i64, _vp, _int, _int, _vp],
-    "wq_delta_xor_items": [_vp, _i64, _vp, _int, _int, _int, _vp],
+    "wq_delta_xor_items": [_vp, _i64, _vp, _int, _int, _int, _int, _vp],
     "wq_int4_fake_quant": [_vp, _int, _i64, _i64, _i64, _i64, _int, _int, _int, _vp, _vp, _vp, _vp],
     "wq_int4_group_quant_pack": [_vp, _i64, _i64, _i64, _int, _vp, _vp, _vp],
     "wq_int4_group_quant_pack_grouped": [_vp, _vp, _int, _i64, _int, _vp],
@@ -66,7 +66,8 @@ SIGNATURES = {
     "wq_delta_xor": [_vp, _vp, _vp, _i64, _int, _vp, _vp, _vp],
     "wq_delta_overwrite_encode": [_vp, _vp, _i64, _vp, ctypes.c_uint32, _vp, _vp],
     "wq_delta_xor_noalloc": [_vp, _vp, _vp, _i64, _int, _vp, _vp],
-    "wq_delta_xor_grouped": [_vp, _vp, _int, _i64, _int, _int, _vp],
+    "wq_delta_xor_grouped": [_vp, _vp, _int, _i64, _int, _int, _int, _vp],
+    "wq_delta_xor_xxh3": [_vp, _vp, _vp, _i64, _int, _vp, _vp, _vp, _vp, _vp],
     "wq_selftest_fp8_elem": [_u32, _u32, _int, _vp, _vp],
     "wq_selftest_int4_elem": [_u32, _u32, _vp, _vp],
     "wq_selftest_cvt_fp8": [_u64, _u64, _vp, _vp],

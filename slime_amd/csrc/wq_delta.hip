@@ -4,7 +4,9 @@
 // publisher needs from them: diff = new ^ old, the number of changed bytes, the two adler32 sums of the
 // new bytes, and (optionally) the snapshot brought up to date.  A workgroup owns a 16 KiB chunk; every
 // lane has four 16-byte pieces of both inputs in flight before first use.  Per-chunk partial results go
-// to a workspace row (no atomics, nothing to clear), and a one-workgroup kernel folds the rows.
+// to a workspace row (no atomics, nothing to clear), and a one-workgroup kernel folds the rows.  On request the pass
+// also leaves XXH3's per-block sums of the new bytes (a wavefront's 64 x 16 bytes of one step are exactly one 1 KiB
+// block, lane for lane in the layout those sums want), so the digest costs no second read of the tensor.
 //
 // adler32 over n bytes d_0..d_{n-1}:  A = 1 + sum d_i,  B = n + sum (n - i) d_i,  both mod 65521, digest
 // (B << 16) | A.  Both sums are linear in the bytes, so a chunk at byte offset `base` contributes
@@ -17,6 +19,7 @@
 #include <atomic>
 
 #include "wq_common.h"
+#include "wq_xxh3_common.h"
 
 namespace wq {
 
@@ -79,13 +82,15 @@ __device__ __forceinline__ void store_tail(uint8_t* p, u32x4 v, int valid)
 }
 
 // One 16 KiB chunk of one tensor.  partials: [chunks of the tensor][3] uint64 = {changed bytes, S, W}.
-template <bool DIFF, bool UPDATE>
+template <bool DIFF, bool UPDATE, bool XXH3>
 __device__ __forceinline__ void delta_xor_chunk(const uint8_t* __restrict__ nw, uint8_t* __restrict__ old,
                                                 uint8_t* __restrict__ diff, int64_t n, uint64_t* __restrict__ partials,
-                                                int64_t item, uint32_t (*red)[4])
+                                                uint64_t* __restrict__ xsums, int64_t item, uint32_t (*red)[4])
 {
     const int64_t base = item * kDeltaChunk;
     u32x4 a[kDeltaSteps], b[kDeltaSteps];
+    uint64_t k0 = 0, k1 = 0, xs0[kDeltaSteps], xs1[kDeltaSteps];
+    if (XXH3) xxh3_lane_keys(threadIdx.x & 63, k0, k1);
     const bool whole = n >= 16;
     auto issue = [&](int i) {
         // lanes past the end re-read the last whole piece instead of branching around the load
@@ -131,12 +136,30 @@ __device__ __forceinline__ void delta_xor_chunk(const uint8_t* __restrict__ nw, 
         s_lane += s;
         p_lane += (uint32_t)threadIdx.x * 16u * s + r;
         q_lane += (uint32_t)i * s;
+        if (XXH3)
+            xxh3_lane_terms(((uint64_t)a[i].y << 32) | a[i].x, ((uint64_t)a[i].w << 32) | a[i].z, k0, k1, xs0[i], xs1[i]);
         if (valid == 16) {
             if (DIFF) stg_nt<u32x4>(diff + off, d);
             if (UPDATE) stg_nt<u32x4>(old + off, a[i]);
         } else if (valid > 0) {
             if (DIFF) store_tail(diff + off, d, valid);
             if (UPDATE) store_tail(old + off, a[i], valid);
+        }
+    }
+    if (XXH3) {
+        // the wavefront's piece of step i is block 16 * item + 4 * i + wave of the tensor; only blocks that end before
+        // the last byte are summed here (the rest is the digest walk's tail, read from the tensor)
+        const int64_t nb = scrambled_blocks(n);
+        const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+#pragma unroll
+        for (int i = 0; i < kDeltaSteps; ++i) {
+            const int64_t blk = item * (kDeltaChunk / kXxhBlock) + i * 4 + wave;
+            xxh3_block_reduce(xs0[i], xs1[i]);
+            if (lane < 4 && blk < nb) {
+                uint64_t* out = xsums + blk * 8 + 2 * lane;
+                out[0] = xs0[i];
+                out[1] = xs1[i];
+            }
         }
     }
     changed = row16_sum_u32(changed);
@@ -169,7 +192,7 @@ struct DeltaArgs {
 
 // GROUPED: 0 = one tensor in the kernel arguments, 1 = descriptor array + prefix sums (the owner of a chunk is
 // searched), 2 = one pre-resolved descriptor per chunk
-template <bool DIFF, bool UPDATE, int GROUPED>
+template <bool DIFF, bool UPDATE, int GROUPED, bool XXH3>
 __global__ __launch_bounds__(256) void delta_xor_kernel(const DeltaArgs a, int64_t items)
 {
     __shared__ uint32_t red[16][4];      // per 16-lane row: changed, S, P, Q
@@ -183,13 +206,13 @@ __global__ __launch_bounds__(256) void delta_xor_kernel(const DeltaArgs a, int64
         item -= a.chunk_start[di];
     } else if (GROUPED == 2) {
         const wq_delta_chunk_item it = a.items[item];
-        d = wq_delta_desc{it.new_bytes, it.old_bytes, it.diff, it.n, it.workspace, nullptr};
+        d = wq_delta_desc{it.new_bytes, it.old_bytes, it.diff, it.n, it.workspace, nullptr, it.xxh3_sums, nullptr};
         item = it.chunk;
     } else {
         d = a.d;
     }
-    delta_xor_chunk<DIFF, UPDATE>((const uint8_t*)d.new_bytes, (uint8_t*)d.old_bytes, (uint8_t*)d.diff, d.n,
-                                  (uint64_t*)d.workspace, item, red);
+    delta_xor_chunk<DIFF, UPDATE, XXH3>((const uint8_t*)d.new_bytes, (uint8_t*)d.old_bytes, (uint8_t*)d.diff, d.n,
+                                        (uint64_t*)d.workspace, d.xxh3_sums, item, red);
 }
 
 // result[0] = changed bytes, result[1] = adler32 of the new bytes.  One workgroup of 1024 lanes per tensor; every lane keeps
@@ -375,36 +398,57 @@ WQ_EXPORT int64_t wq_delta_workspace_bytes(int64_t n)
     return cdiv64(n > 0 ? n : 1, kDeltaChunk) * 32;      // 24 bytes of partials + a 4-byte scan slot, rounded up
 }
 
-template <int GROUPED>
-static void launch_delta_xor(const DeltaArgs& a, int64_t items, bool diff, bool update, hipStream_t st)
+template <int GROUPED, bool XXH3>
+static void launch_delta_xor_x(const DeltaArgs& a, int64_t items, bool diff, bool update, hipStream_t st)
 {
     const dim3 g = grid_for_items(items);
-    if (diff && update) delta_xor_kernel<true, true, GROUPED><<<g, 256, kDeltaOccupancyPadBytes, st>>>(a, items);
-    else if (diff) delta_xor_kernel<true, false, GROUPED><<<g, 256, kDeltaOccupancyPadBytes, st>>>(a, items);
-    else if (update) delta_xor_kernel<false, true, GROUPED><<<g, 256, kDeltaOccupancyPadBytes, st>>>(a, items);
-    else delta_xor_kernel<false, false, GROUPED><<<g, 256, kDeltaOccupancyPadBytes, st>>>(a, items);
+    if (diff && update) delta_xor_kernel<true, true, GROUPED, XXH3><<<g, 256, kDeltaOccupancyPadBytes, st>>>(a, items);
+    else if (diff) delta_xor_kernel<true, false, GROUPED, XXH3><<<g, 256, kDeltaOccupancyPadBytes, st>>>(a, items);
+    else if (update) delta_xor_kernel<false, true, GROUPED, XXH3><<<g, 256, kDeltaOccupancyPadBytes, st>>>(a, items);
+    else delta_xor_kernel<false, false, GROUPED, XXH3><<<g, 256, kDeltaOccupancyPadBytes, st>>>(a, items);
+}
+
+template <int GROUPED>
+static void launch_delta_xor(const DeltaArgs& a, int64_t items, bool diff, bool update, bool xxh3, hipStream_t st)
+{
+    if (xxh3) launch_delta_xor_x<GROUPED, true>(a, items, diff, update, st);
+    else launch_delta_xor_x<GROUPED, false>(a, items, diff, update, st);
+}
+
+static int delta_xor_one(const void* new_bytes, void* old_bytes, void* diff, int64_t n, int update_old, void* workspace,
+                         uint64_t* result, uint64_t* xxh3_workspace, uint64_t* digest, bool xxh3, hipStream_t st)
+{
+    if (n < 0) return WQ_ERR_SHAPE;
+    if (!result || !workspace || (xxh3 && (!xxh3_workspace || !digest))) return WQ_ERR_NULL;
+    if (n > 0 && (!new_bytes || !old_bytes)) return WQ_ERR_NULL;
+    if (((uintptr_t)new_bytes & 15) || ((uintptr_t)old_bytes & 15) || ((uintptr_t)diff & 15) ||
+        ((uintptr_t)workspace & 7) || ((uintptr_t)result & 7))
+        return WQ_ERR_ALIGN;
+    if (xxh3 && (((uintptr_t)xxh3_workspace & 15) || ((uintptr_t)digest & 7))) return WQ_ERR_ALIGN;
+    const int64_t items = n > 0 ? cdiv64(n, kDeltaChunk) : 0;
+    DeltaArgs a{};
+    a.d = wq_delta_desc{new_bytes, old_bytes, diff, n, workspace, result, xxh3_workspace, digest};
+    if (items > 0) {
+        launch_delta_xor<0>(a, items, diff != nullptr, update_old != 0, xxh3, st);
+        WQ_LAUNCH_CHECK();
+    }
+    delta_fold_kernel<false><<<1, kFoldThreads, 0, st>>>(a);
+    WQ_LAUNCH_CHECK();
+    return xxh3 ? xxh3_chain_for_delta(&a.d, nullptr, 1, st) : WQ_OK;
 }
 
 WQ_EXPORT int wq_delta_xor(const void* new_bytes, void* old_bytes, void* diff, int64_t n, int update_old,
                            void* workspace, uint64_t* result, void* stream)
 {
-    if (n < 0) return WQ_ERR_SHAPE;
-    if (!result || !workspace) return WQ_ERR_NULL;
-    if (n > 0 && (!new_bytes || !old_bytes)) return WQ_ERR_NULL;
-    if (((uintptr_t)new_bytes & 15) || ((uintptr_t)old_bytes & 15) || ((uintptr_t)diff & 15) ||
-        ((uintptr_t)workspace & 7) || ((uintptr_t)result & 7))
-        return WQ_ERR_ALIGN;
-    hipStream_t st = (hipStream_t)stream;
-    const int64_t items = n > 0 ? cdiv64(n, kDeltaChunk) : 0;
-    DeltaArgs a{};
-    a.d = wq_delta_desc{new_bytes, old_bytes, diff, n, workspace, result};
-    if (items > 0) {
-        launch_delta_xor<0>(a, items, diff != nullptr, update_old != 0, st);
-        WQ_LAUNCH_CHECK();
-    }
-    delta_fold_kernel<false><<<1, kFoldThreads, 0, st>>>(a);
-    WQ_LAUNCH_CHECK();
-    return WQ_OK;
+    return delta_xor_one(new_bytes, old_bytes, diff, n, update_old, workspace, result, nullptr, nullptr, false,
+                         (hipStream_t)stream);
+}
+
+WQ_EXPORT int wq_delta_xor_xxh3(const void* new_bytes, void* old_bytes, void* diff, int64_t n, int update_old,
+                                void* workspace, uint64_t* result, uint64_t* xxh3_workspace, uint64_t* digest, void* stream)
+{
+    return delta_xor_one(new_bytes, old_bytes, diff, n, update_old, workspace, result, xxh3_workspace, digest, true,
+                         (hipStream_t)stream);
 }
 
 // ---- the same pass for callers that cannot allocate ------------------------------------------------------
@@ -451,7 +495,7 @@ WQ_EXPORT int wq_delta_xor_noalloc(const void* new_bytes, void* old_bytes, void*
 }
 
 WQ_EXPORT int wq_delta_xor_grouped(const wq_delta_desc* descs, const int64_t* chunk_start, int n_desc,
-                                   int64_t total_chunks, int write_diff, int update_old, void* stream)
+                                   int64_t total_chunks, int write_diff, int update_old, int with_xxh3, void* stream)
 {
     if (n_desc < 0 || total_chunks < 0) return WQ_ERR_SHAPE;
     if (n_desc == 0) return WQ_OK;
@@ -462,16 +506,16 @@ WQ_EXPORT int wq_delta_xor_grouped(const wq_delta_desc* descs, const int64_t* ch
     a.chunk_start = chunk_start;
     a.n_desc = n_desc;
     if (total_chunks > 0) {
-        launch_delta_xor<1>(a, total_chunks, write_diff != 0, update_old != 0, st);
+        launch_delta_xor<1>(a, total_chunks, write_diff != 0, update_old != 0, with_xxh3 != 0, st);
         WQ_LAUNCH_CHECK();
     }
     delta_fold_kernel<true><<<n_desc, kFoldThreads, 0, st>>>(a);
     WQ_LAUNCH_CHECK();
-    return WQ_OK;
+    return with_xxh3 ? xxh3_chain_for_delta(nullptr, descs, n_desc, st) : WQ_OK;
 }
 
 WQ_EXPORT int wq_delta_xor_items(const wq_delta_chunk_item* items, int64_t n_items, const wq_delta_desc* descs, int n_desc,
-                                 int write_diff, int update_old, void* stream)
+                                 int write_diff, int update_old, int with_xxh3, void* stream)
 {
     if (n_desc < 0 || n_items < 0) return WQ_ERR_SHAPE;
     if (n_desc == 0) return WQ_OK;
@@ -482,12 +526,12 @@ WQ_EXPORT int wq_delta_xor_items(const wq_delta_chunk_item* items, int64_t n_ite
     a.n_desc = n_desc;
     a.items = items;
     if (n_items > 0) {
-        launch_delta_xor<2>(a, n_items, write_diff != 0, update_old != 0, st);
+        launch_delta_xor<2>(a, n_items, write_diff != 0, update_old != 0, with_xxh3 != 0, st);
         WQ_LAUNCH_CHECK();
     }
     delta_fold_kernel<true><<<n_desc, kFoldThreads, 0, st>>>(a);
     WQ_LAUNCH_CHECK();
-    return WQ_OK;
+    return with_xxh3 ? xxh3_chain_for_delta(nullptr, descs, n_desc, st) : WQ_OK;
 }
 
 WQ_EXPORT int wq_delta_overwrite_encode(const void* new_bytes, const void* old_bytes, int64_t n, void* workspace,

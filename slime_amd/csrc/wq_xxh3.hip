@@ -10,34 +10,17 @@
 //   xxh3_block_sums_kernel   the eight sums of every block, at memory speed: a wavefront takes a block with one
 //                            16-byte load per lane (lane l holds words 2j, 2j+1 of stripe l / 4, j = l % 4), multiplies
 //                            in place and adds across the sixteen lanes that share j; 64 bytes of sums per KiB.
-//   xxh3_chain_kernel        per tensor, eight lanes walk acc <- scramble(acc + sums[k]) (about 60 clocks a block), add
+//   xxh3_chain_kernel        per tensor, eight lanes walk acc <- scramble(acc + sums[k]) (about 50 clocks a block), add
 //                            the tail - the stripes of the last partial block and the last 64 bytes, read straight from
 //                            the tensor - and one lane folds the accumulators into the two 64-bit halves.
 // Inputs of 240 bytes or less use XXH3's short forms: one lane of the second kernel computes those.
+// The delta pass can leave the block sums itself (it reads the same bytes); then only the walk runs, over its descriptors.
 
 #include "wq_common.h"
+#include "wq_xxh3_common.h"
 
 namespace wq {
 
-__constant__ uint8_t kXxh3Secret[192] = {
-    0xb8, 0xfe, 0x6c, 0x39, 0x23, 0xa4, 0x4b, 0xbe, 0x7c, 0x01, 0x81, 0x2c, 0xf7, 0x21, 0xad, 0x1c,
-    0xde, 0xd4, 0x6d, 0xe9, 0x83, 0x90, 0x97, 0xdb, 0x72, 0x40, 0xa4, 0xa4, 0xb7, 0xb3, 0x67, 0x1f,
-    0xcb, 0x79, 0xe6, 0x4e, 0xcc, 0xc0, 0xe5, 0x78, 0x82, 0x5a, 0xd0, 0x7d, 0xcc, 0xff, 0x72, 0x21,
-    0xb8, 0x08, 0x46, 0x74, 0xf7, 0x43, 0x24, 0x8e, 0xe0, 0x35, 0x90, 0xe6, 0x81, 0x3a, 0x26, 0x4c,
-    0x3c, 0x28, 0x52, 0xbb, 0x91, 0xc3, 0x00, 0xcb, 0x88, 0xd0, 0x65, 0x8b, 0x1b, 0x53, 0x2e, 0xa3,
-    0x71, 0x64, 0x48, 0x97, 0xa2, 0x0d, 0xf9, 0x4e, 0x38, 0x19, 0xef, 0x46, 0xa9, 0xde, 0xac, 0xd8,
-    0xa8, 0xfa, 0x76, 0x3f, 0xe3, 0x9c, 0x34, 0x3f, 0xf9, 0xdc, 0xbb, 0xc7, 0xc7, 0x0b, 0x4f, 0x1d,
-    0x8a, 0x51, 0xe0, 0x4b, 0xcd, 0xb4, 0x59, 0x31, 0xc8, 0x9f, 0x7e, 0xc9, 0xd9, 0x78, 0x73, 0x64,
-    0xea, 0xc5, 0xac, 0x83, 0x34, 0xd3, 0xeb, 0xc3, 0xc5, 0x81, 0xa0, 0xff, 0xfa, 0x13, 0x63, 0xeb,
-    0x17, 0x0d, 0xdd, 0x51, 0xb7, 0xf0, 0xda, 0x49, 0xd3, 0x16, 0x55, 0x26, 0x29, 0xd4, 0x68, 0x9e,
-    0x2b, 0x16, 0xbe, 0x58, 0x7d, 0x47, 0xa1, 0xfc, 0x8f, 0xf8, 0xb8, 0xd1, 0x7a, 0xd0, 0x31, 0xce,
-    0x45, 0xcb, 0x3a, 0x8f, 0x95, 0x16, 0x04, 0x28, 0xaf, 0xd7, 0xfb, 0xca, 0xbb, 0x4b, 0x40, 0x7e,
-};
-
-constexpr uint64_t kP32_1 = 0x9E3779B1ull, kP32_2 = 0x85EBCA77ull, kP32_3 = 0xC2B2AE3Dull;
-constexpr uint64_t kP64_1 = 0x9E3779B185EBCA87ull, kP64_2 = 0xC2B2AE3D27D4EB4Full, kP64_3 = 0x165667B19E3779F9ull;
-constexpr uint64_t kP64_4 = 0x85EBCA77C2B2AE63ull, kP64_5 = 0x27D4EB2F165667C5ull, kMx1 = 0x165667919E3779F9ull;
-constexpr int kXxhBlock = 1024, kXxhStripe = 64;
 constexpr int kXxhBlocksPerItem = 16;      // a work item of the sums kernel: 16 KiB, four blocks per wavefront
 constexpr int kXxhItemsPerXcdRun = 32;
 
@@ -48,43 +31,11 @@ struct Xxh3Args {
     int32_t n_desc;
 };
 
-// little-endian u64 of the secret at any byte offset
-__device__ __forceinline__ uint64_t secret64(int off)
-{
-    uint64_t v = 0;
-#pragma unroll
-    for (int b = 0; b < 8; ++b) v |= (uint64_t)kXxh3Secret[off + b] << (8 * b);
-    return v;
-}
-
-__device__ __forceinline__ uint64_t load64_bytes(const uint8_t* p)
-{
-    uint64_t v = 0;
-#pragma unroll
-    for (int b = 0; b < 8; ++b) v |= (uint64_t)p[b] << (8 * b);
-    return v;
-}
-
-__device__ __forceinline__ uint64_t mul_halves(uint64_t x) { return (x & 0xFFFFFFFFull) * (x >> 32); }
-
 __device__ __forceinline__ uint64_t shfl_xor_u64(uint64_t v, int mask)
 {
     const uint32_t lo = (uint32_t)__shfl_xor((int)(uint32_t)v, mask), hi = (uint32_t)__shfl_xor((int)(uint32_t)(v >> 32), mask);
     return ((uint64_t)hi << 32) | lo;
 }
-
-// v + (v of the lane 4 further on in the 16-lane row) + ... : the sum over the four lanes of a row that share lane % 4,
-// by two rotations of the row (DPP row_ror:4, row_ror:8)
-__device__ __forceinline__ uint64_t row_sum_stride4_u64(uint64_t v)
-{
-    uint32_t lo = (uint32_t)v, hi = (uint32_t)(v >> 32);
-    v += ((uint64_t)dpp_u32<0x124>(hi) << 32) | dpp_u32<0x124>(lo);
-    lo = (uint32_t)v, hi = (uint32_t)(v >> 32);
-    v += ((uint64_t)dpp_u32<0x128>(hi) << 32) | dpp_u32<0x128>(lo);
-    return v;
-}
-
-__device__ __forceinline__ int64_t scrambled_blocks(int64_t n) { return (n - 1) / kXxhBlock; }
 
 template <int GROUPED>
 __global__ __launch_bounds__(256) void xxh3_block_sums_kernel(const Xxh3Args a, const int64_t total_items)
@@ -103,9 +54,8 @@ __global__ __launch_bounds__(256) void xxh3_block_sums_kernel(const Xxh3Args a, 
     }
     const int64_t nb = scrambled_blocks(d.n);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
-    const int stripe = lane >> 2, pair = lane & 3;
-    // stripe s reads the secret at 8 s: word i of the stripe meets the secret's u64 number s + i
-    const uint64_t k0 = secret64(8 * (stripe + 2 * pair)), k1 = secret64(8 * (stripe + 2 * pair + 1));
+    uint64_t k0, k1;
+    xxh3_lane_keys(lane, k0, k1);
     const uint8_t* base = (const uint8_t*)d.data;
     const bool aligned = ((uintptr_t)base & 15) == 0;
     constexpr int PER_WAVE = kXxhBlocksPerItem / 4;
@@ -128,15 +78,9 @@ __global__ __launch_bounds__(256) void xxh3_block_sums_kernel(const Xxh3Args a, 
 #pragma unroll
     for (int i = 0; i < PER_WAVE; ++i) {
         const int64_t b = local * kXxhBlocksPerItem + wave + 4 * i;
-        uint64_t s0 = d1[i] + mul_halves(d0[i] ^ k0);      // into accumulator 2 * pair
-        uint64_t s1 = d0[i] + mul_halves(d1[i] ^ k1);      // into accumulator 2 * pair + 1
-        s0 = row_sum_stride4_u64(s0);                       // stripes 4r .. 4r+3 of row r
-        s1 = row_sum_stride4_u64(s1);
-#pragma unroll
-        for (int m = 16; m < 64; m <<= 1) {                 // the four rows
-            s0 += shfl_xor_u64(s0, m);
-            s1 += shfl_xor_u64(s1, m);
-        }
+        uint64_t s0, s1;
+        xxh3_lane_terms(d0[i], d1[i], k0, k1, s0, s1);
+        xxh3_block_reduce(s0, s1);
         if (lane < 4 && b < nb) {
             uint64_t* out = d.sums + b * 8 + 2 * lane;
             out[0] = s0;
@@ -244,14 +188,46 @@ __device__ void xxh3_short(const uint8_t* p, int n, uint64_t& out_low, uint64_t&
     }
 }
 
+// XXH3's scramble of one accumulator, ((a ^ a >> 47) ^ key) * PRIME32_1 mod 2^64, plus `add`.  The two halves of the
+// product are kept independent: the low word's 32 x 32 -> 64 multiply-add (which takes `add` along) and the high word's
+// 32 x 32 -> 32 multiply can be in flight together, and one 32-bit add joins them.  Written as a 64-bit multiply the
+// compiler chains two v_mad_u64_u32, the second waiting for the first - and the walk is nothing but that dependency.
+__device__ __forceinline__ uint64_t scramble_then_add(uint64_t a, uint64_t key, uint64_t add)
+{
+    const uint32_t lo = (uint32_t)a, hi = (uint32_t)(a >> 32);
+    const uint32_t xh = hi ^ (uint32_t)(key >> 32);
+    const uint32_t xl = lo ^ (hi >> 15) ^ (uint32_t)key;
+    uint32_t top = xh * (uint32_t)kP32_1;
+    asm volatile("" : "+v"(top));                       // keep it a product of its own
+    const uint64_t low = (uint64_t)xl * (uint32_t)kP32_1 + add;
+    return (((uint64_t)((uint32_t)(low >> 32) + top)) << 32) | (uint32_t)low;
+}
+
 // one wavefront per tensor; lanes 0..7 own one accumulator each
-__global__ __launch_bounds__(64) void xxh3_chain_kernel(const wq_xxh3_desc single, const wq_xxh3_desc* __restrict__ descs,
-                                                        int n_desc)
+__device__ __forceinline__ wq_xxh3_desc chain_view(const wq_xxh3_desc& d, bool& skip)
+{
+    skip = false;
+    return d;
+}
+// after a delta pass: the digest of a tensor that did not change is not wanted (nothing is published for it)
+__device__ __forceinline__ wq_xxh3_desc chain_view(const wq_delta_desc& d, bool& skip)
+{
+    skip = d.result[0] == 0;
+    return wq_xxh3_desc{d.new_bytes, d.n, d.xxh3_sums, d.xxh3_digest};
+}
+
+template <typename Desc>
+__global__ __launch_bounds__(64) void xxh3_chain_kernel(const Desc single, const Desc* __restrict__ descs, int n_desc)
 {
     const int t = blockIdx.x;
     if (t >= n_desc) return;
-    const wq_xxh3_desc d = descs ? descs[t] : single;
+    bool skip;
+    const wq_xxh3_desc d = chain_view(descs ? descs[t] : single, skip);
     const int lane = threadIdx.x, i = lane & 7;
+    if (skip) {                               // uniform per wavefront
+        if (lane < 2) d.digest[lane] = 0;
+        return;
+    }
     if (d.n <= 240) {                         // uniform per wavefront
         if (lane == 0) {
             uint64_t low, high;
@@ -269,41 +245,41 @@ __global__ __launch_bounds__(64) void xxh3_chain_kernel(const wq_xxh3_desc singl
     const int64_t nb = scrambled_blocks(d.n);
     const uint64_t* s = d.sums + i;
 
-    // The walk.  A block costs about 55 clocks of dependent arithmetic and a load from HBM takes well over a thousand,
-    // so the sums are fetched 32 blocks ahead: four batches of eight are in flight, and the batch just consumed is
-    // refilled at once with the blocks 32 further on.
-    constexpr int U = 8, DEPTH = 4;
-    uint64_t ring[DEPTH][U];
-    int64_t k = 0;
-    if (nb >= DEPTH * U) {
+    // The walk, acc <- scramble(acc + sums[k]) for every block, carried as b_k = acc_k + sums[k]:
+    // b_k = scramble(b_{k-1}) + sums[k], so that the addition rides on the multiply-add of the scramble.  A block costs
+    // about 50 clocks of dependent arithmetic (20 ns) and a load from HBM takes well over a microsecond, so the sums are
+    // fetched 64 blocks ahead: eight batches of eight are in flight, and the batch just consumed is refilled at once with
+    // the blocks 64 further on.  Measured per block on a 256 MiB tensor: 32 ahead 23.9 ns, 48: 21.2, 64: 20.2, 80: 21.9,
+    // 96: 22.7, 128: 27.2 (the ring no longer fits the registers).
+    if (nb > 0) {
+        constexpr int U = 8, DEPTH = 8;
+        uint64_t ring[DEPTH][U];
+        acc += s[0];
+        const uint64_t* rest = s + 8;          // sums[1 ..]
+        const int64_t m = nb - 1;
+        int64_t k = 0;
+        if (m >= DEPTH * U) {
 #pragma unroll
-        for (int b = 0; b < DEPTH; ++b)
+            for (int b = 0; b < DEPTH; ++b)
 #pragma unroll
-            for (int u = 0; u < U; ++u) ring[b][u] = s[(b * U + u) * 8];
-        for (; k + 2 * DEPTH * U <= nb; k += DEPTH * U) {
+                for (int u = 0; u < U; ++u) ring[b][u] = rest[(b * U + u) * 8];
+            for (; k + 2 * DEPTH * U <= m; k += DEPTH * U) {
 #pragma unroll
-            for (int b = 0; b < DEPTH; ++b) {
+                for (int b = 0; b < DEPTH; ++b) {
 #pragma unroll
-                for (int u = 0; u < U; ++u) {
-                    acc += ring[b][u];
-                    acc = ((acc ^ (acc >> 47)) ^ scramble_key) * kP32_1;
+                    for (int u = 0; u < U; ++u) acc = scramble_then_add(acc, scramble_key, ring[b][u]);
+#pragma unroll
+                    for (int u = 0; u < U; ++u) ring[b][u] = rest[(k + (DEPTH + b) * U + u) * 8];
                 }
-#pragma unroll
-                for (int u = 0; u < U; ++u) ring[b][u] = s[(k + (DEPTH + b) * U + u) * 8];
             }
+#pragma unroll
+            for (int b = 0; b < DEPTH; ++b)
+#pragma unroll
+                for (int u = 0; u < U; ++u) acc = scramble_then_add(acc, scramble_key, ring[b][u]);
+            k += DEPTH * U;
         }
-#pragma unroll
-        for (int b = 0; b < DEPTH; ++b)
-#pragma unroll
-            for (int u = 0; u < U; ++u) {
-                acc += ring[b][u];
-                acc = ((acc ^ (acc >> 47)) ^ scramble_key) * kP32_1;
-            }
-        k += DEPTH * U;
-    }
-    for (; k < nb; ++k) {
-        acc += s[k * 8];
-        acc = ((acc ^ (acc >> 47)) ^ scramble_key) * kP32_1;
+        for (; k < m; ++k) acc = scramble_then_add(acc, scramble_key, rest[k * 8]);
+        acc = scramble_then_add(acc, scramble_key, 0);
     }
 
     // the last partial block: its whole stripes, then the last 64 bytes of the input under their own key
@@ -338,6 +314,13 @@ __global__ __launch_bounds__(64) void xxh3_chain_kernel(const wq_xxh3_desc singl
     }
 }
 
+int xxh3_chain_for_delta(const wq_delta_desc* single, const wq_delta_desc* descs, int n_desc, hipStream_t st)
+{
+    xxh3_chain_kernel<wq_delta_desc><<<n_desc, 64, 0, st>>>(single ? *single : wq_delta_desc{}, descs, n_desc);
+    WQ_LAUNCH_CHECK();
+    return WQ_OK;
+}
+
 static inline int64_t xxh3_items(int64_t n) { return cdiv64(n > 0 ? (n - 1) / kXxhBlock : 0, kXxhBlocksPerItem); }
 
 }  // namespace wq
@@ -359,7 +342,7 @@ WQ_EXPORT int wq_xxh3_128(const void* data, int64_t n, uint64_t* workspace, uint
         xxh3_block_sums_kernel<0><<<grid_for_items(items), 256, 0, st>>>(a, items);
         WQ_LAUNCH_CHECK();
     }
-    xxh3_chain_kernel<<<1, 64, 0, st>>>(a.d, nullptr, 1);
+    xxh3_chain_kernel<wq_xxh3_desc><<<1, 64, 0, st>>>(a.d, nullptr, 1);
     WQ_LAUNCH_CHECK();
     return WQ_OK;
 }
@@ -379,7 +362,7 @@ WQ_EXPORT int wq_xxh3_128_grouped(const wq_xxh3_desc* descs, const int64_t* item
         xxh3_block_sums_kernel<1><<<grid_for_items(total_items), 256, 0, st>>>(a, total_items);
         WQ_LAUNCH_CHECK();
     }
-    xxh3_chain_kernel<<<n_desc, 64, 0, st>>>(wq_xxh3_desc{}, descs, n_desc);
+    xxh3_chain_kernel<wq_xxh3_desc><<<n_desc, 64, 0, st>>>(wq_xxh3_desc{}, descs, n_desc);
     WQ_LAUNCH_CHECK();
     return WQ_OK;
 }

@@ -70,90 +70,104 @@ def _align(n: int, a: int = 256) -> int:
     return (n + a - 1) // a * a
 
 
-def xor_diff_many(news, olds, update_snapshot: bool = False, want_diff: bool = True):
-    """``xor_diff`` over a bucket of tensors with two kernel launches in total.
-
-    -> (diffs: list of uint8 views into one flat buffer, or None without ``want_diff``;
-        results: int64 [len(news), 2] on the device = [changed bytes, adler32(new)] per tensor)."""
-    if len(news) != len(olds):
-        raise ValueError("xor_diff_many: need one snapshot per tensor")
-    if not news:
-        return ([] if want_diff else None), torch.empty((0, 2), dtype=torch.int64)
-    flat = [_as_bytes(t, "xor_diff_many") for t in news]
-    device = flat[0].device
+def _bucket_tables(flat, olds, want_diff: bool, xxh3: bool, device):
+    """Buffers and the per-tensor descriptor rows (wq_delta_desc: new, old, diff, n, workspace, result, xxh3_sums,
+    xxh3_digest) of a bucket: one flat diff buffer, one flat workspace (delta rows, then the digest's block sums)."""
     lib = _lib.load()
-    d_off, w_off, d_total, w_total = [], [], 0, 0
+    d_off, w_off, x_off, d_total, w_total = [], [], [], 0, 0
     for nw, old in zip(flat, olds):
         _check_old(nw, old)
         d_off.append(d_total)
         w_off.append(w_total)
         d_total += _align(nw.numel())
         w_total += _align(lib.wq_delta_workspace_bytes(nw.numel()))
+    for nw in flat:
+        x_off.append(w_total)
+        if xxh3:
+            w_total += _align(lib.wq_xxh3_workspace_bytes(nw.numel()))
     flat_diff = torch.empty(max(d_total, 1), dtype=torch.uint8, device=device) if want_diff else None
     flat_ws = torch.empty(w_total // 8, dtype=torch.int64, device=device)
     results = torch.empty((len(flat), 2), dtype=torch.int64, device=device)
-    rows, starts, chunks = [], [0], 0
+    digests = torch.empty((len(flat), 2), dtype=torch.int64, device=device) if xxh3 else None     # [low64, high64]
+    rows = []
     for i, (nw, old) in enumerate(zip(flat, olds)):
-        n = nw.numel()
-        rows.append([nw.data_ptr(), old.data_ptr(), flat_diff.data_ptr() + d_off[i] if want_diff else 0, n,
-                     flat_ws.data_ptr() + w_off[i], results.data_ptr() + 16 * i])
-        chunks += -(-n // CHUNK)
+        rows.append([nw.data_ptr(), old.data_ptr(), flat_diff.data_ptr() + d_off[i] if want_diff else 0, nw.numel(),
+                     flat_ws.data_ptr() + w_off[i], results.data_ptr() + 16 * i,
+                     flat_ws.data_ptr() + x_off[i] if xxh3 else 0, digests.data_ptr() + 16 * i if xxh3 else 0])
+    diffs = [flat_diff[o:o + nw.numel()] for o, nw in zip(d_off, flat)] if want_diff else None
+    return rows, flat_diff, flat_ws, results, digests, diffs
+
+
+def xor_diff_many(news, olds, update_snapshot: bool = False, want_diff: bool = True, xxh3: bool = False):
+    """``xor_diff`` over a bucket of tensors with two kernel launches in total (three with ``xxh3``).
+
+    -> (diffs: list of uint8 views into one flat buffer, or None without ``want_diff``;
+        results: int64 [len(news), 2] on the device = [changed bytes, adler32(new)] per tensor)
+       and, with ``xxh3``, a third value: int64 [len(news), 2] on the device = [low64, high64] of xxh3-128 of the new
+       bytes of every tensor that changed ([0, 0] for the others), computed by the same pass over the tensors."""
+    if len(news) != len(olds):
+        raise ValueError("xor_diff_many: need one snapshot per tensor")
+    if not news:
+        empty = torch.empty((0, 2), dtype=torch.int64)
+        return (([] if want_diff else None), empty) + ((empty,) if xxh3 else ())
+    flat = [_as_bytes(t, "xor_diff_many") for t in news]
+    device = flat[0].device
+    rows, flat_diff, flat_ws, results, digests, diffs = _bucket_tables(flat, olds, want_diff, xxh3, device)
+    starts, chunks = [0], 0
+    for nw in flat:
+        chunks += -(-nw.numel() // CHUNK)
         starts.append(chunks)
     descs = torch.tensor(rows, dtype=torch.int64).to(device)
     start_t = torch.tensor(starts, dtype=torch.int64).to(device)
     with torch.cuda.device(device):
-        rc = lib.wq_delta_xor_grouped(descs.data_ptr(), start_t.data_ptr(), len(flat), chunks, int(want_diff),
-                                      int(update_snapshot), _lib.stream_ptr(device))
+        rc = _lib.load().wq_delta_xor_grouped(descs.data_ptr(), start_t.data_ptr(), len(flat), chunks, int(want_diff),
+                                              int(update_snapshot), int(xxh3), _lib.stream_ptr(device))
     _lib.check(rc, "xor_diff_many")
-    diffs = [flat_diff[o:o + nw.numel()] for o, nw in zip(d_off, flat)] if want_diff else None
-    return diffs, results
+    return (diffs, results) + ((digests,) if xxh3 else ())
 
 
 class XorDiffPlan:
     """``xor_diff_many`` for a FIXED bucket - the same weight tensors against the same snapshots every weight sync - with
-    the per-chunk work table built once: every 16 KiB chunk has its own pre-resolved descriptor (48 bytes per 64 KiB of
+    the per-chunk work table built once: every 16 KiB chunk has its own pre-resolved descriptor (64 bytes per 64 KiB of
     traffic), so the kernel does one scalar load instead of searching the per-tensor prefix sums, and ``run()`` does no
-    host-side table work.  ``diffs`` (uint8 views into one flat buffer) and ``results`` (int64 [n, 2] = [changed bytes,
-    adler32(new)]) are owned by the plan and overwritten by every run."""
+    host-side table work.  ``diffs`` (uint8 views into one flat buffer), ``results`` (int64 [n, 2] = [changed bytes,
+    adler32(new)]) and, with ``xxh3``, ``digests`` (int64 [n, 2] = [low64, high64] of xxh3-128 of the new bytes, [0, 0]
+    for a tensor that did not change) are owned by the plan and overwritten by every run."""
 
-    def __init__(self, news, olds, want_diff: bool = True):
+    def __init__(self, news, olds, want_diff: bool = True, xxh3: bool = False):
         if not news or len(news) != len(olds):
             raise ValueError("XorDiffPlan: need one snapshot per tensor and at least one tensor")
         self.news = [_as_bytes_in_place(t, "XorDiffPlan") for t in news]
         self.olds = list(olds)
-        self.want_diff = bool(want_diff)
+        self.want_diff, self.xxh3 = bool(want_diff), bool(xxh3)
         device = self.news[0].device
-        lib = _lib.load()
-        d_off, w_off, d_total, w_total = [], [], 0, 0
-        for nw, old in zip(self.news, self.olds):
-            _check_old(nw, old)
-            d_off.append(d_total)
-            w_off.append(w_total)
-            d_total += _align(nw.numel())
-            w_total += _align(lib.wq_delta_workspace_bytes(nw.numel()))
-        self._flat_diff = torch.empty(max(d_total, 1), dtype=torch.uint8, device=device) if want_diff else None
-        self._flat_ws = torch.empty(w_total // 8, dtype=torch.int64, device=device)
-        self.results = torch.empty((len(self.news), 2), dtype=torch.int64, device=device)
-        rows = []
-        for i, (nw, old) in enumerate(zip(self.news, self.olds)):
-            rows.append([nw.data_ptr(), old.data_ptr(), self._flat_diff.data_ptr() + d_off[i] if want_diff else 0, nw.numel(),
-                         self._flat_ws.data_ptr() + w_off[i], self.results.data_ptr() + 16 * i])
+        rows, self._flat_diff, self._flat_ws, self.results, self.digests, self.diffs = _bucket_tables(
+            self.news, self.olds, self.want_diff, self.xxh3, device)
         desc = torch.tensor(rows, dtype=torch.int64)
         counts = (desc[:, 3] + CHUNK - 1) // CHUNK
         owner = torch.repeat_interleave(torch.arange(len(rows)), counts)
         chunk = torch.arange(int(counts.sum()), dtype=torch.int64) - (torch.cumsum(counts, 0) - counts)[owner]
-        items = torch.cat([desc[owner][:, :5], chunk.unsqueeze(1)], dim=1)
+        picked = desc[owner]
+        # wq_delta_chunk_item: new, old, diff, n, workspace, chunk, xxh3_sums, reserved
+        items = torch.cat([picked[:, :5], chunk.unsqueeze(1), picked[:, 6:7], torch.zeros_like(chunk).unsqueeze(1)], dim=1)
         self._descs, self._items, self.n_items = desc.to(device), items.contiguous().to(device), items.shape[0]
         self.device = device
-        self.diffs = [self._flat_diff[o:o + nw.numel()] for o, nw in zip(d_off, self.news)] if want_diff else None
         self.nbytes = sum(nw.numel() for nw in self.news)
 
     def run(self, update_snapshot: bool = False):
         with torch.cuda.device(self.device):
             rc = _lib.load().wq_delta_xor_items(self._items.data_ptr(), self.n_items, self._descs.data_ptr(), len(self.news),
-                                                int(self.want_diff), int(update_snapshot), _lib.stream_ptr(self.device))
+                                                int(self.want_diff), int(update_snapshot), int(self.xxh3),
+                                                _lib.stream_ptr(self.device))
         _lib.check(rc, "XorDiffPlan.run")
         return self.diffs, self.results
+
+    def hexdigests(self) -> list:
+        """xxh3-128 hex digests after a run (synchronises); None for a tensor that did not change."""
+        if not self.xxh3:
+            raise ValueError("XorDiffPlan was built without xxh3")
+        changed = self.results[:, 0].tolist()
+        return [_hex128(low, high) if c else None for (low, high), c in zip(self.digests.tolist(), changed)]
 
 
 def _check_old(nw: torch.Tensor, old: torch.Tensor) -> None:
@@ -284,13 +298,11 @@ class DeltaEncoder:
         if self.delta_encoding != "xor":
             return [(name,) + self.encode(name, t) for name, t in named_tensors]
         named_tensors = list(named_tensors)
-        diffs, results = xor_diff_many([t for _, t in named_tensors], [self.snapshot[n] for n, _ in named_tensors],
-                                       update_snapshot=True)
-        results = results.tolist()
-        digests = {}
-        if self.checksum_algorithm == "xxh3-128":       # one grouped digest pass over the tensors that changed
-            moved = [i for i, (changed, _) in enumerate(results) if changed]
-            digests = dict(zip(moved, xxh3_128_many([named_tensors[i][1] for i in moved])))
+        fused = self.checksum_algorithm == "xxh3-128"       # the digest rides on the diff pass: no second read
+        got = xor_diff_many([t for _, t in named_tensors], [self.snapshot[n] for n, _ in named_tensors],
+                            update_snapshot=True, xxh3=fused)
+        diffs, results = got[0], got[1].tolist()
+        digests = {i: _hex128(low, high) for i, (low, high) in enumerate(got[2].tolist())} if fused else {}
         out = []
         for i, ((name, t), diff, (changed, adler)) in enumerate(zip(named_tensors, diffs, results)):
             self.total_bytes += diff.numel()
@@ -315,7 +327,19 @@ class DeltaEncoder:
         self.total_bytes += n
         ws = _workspace(n, nw.device)
         result = torch.empty(2, dtype=torch.int64, device=nw.device)
-        if self.delta_encoding == "xor":
+        digest = None
+        if self.delta_encoding == "xor" and self.checksum_algorithm == "xxh3-128":
+            diff = torch.empty_like(nw)
+            lib = _lib.load()
+            xws = torch.empty(lib.wq_xxh3_workspace_bytes(n) // 8, dtype=torch.int64, device=nw.device)
+            both = torch.empty(4, dtype=torch.int64, device=nw.device)      # result, then digest
+            with torch.cuda.device(nw.device):
+                rc = lib.wq_delta_xor_xxh3(nw.data_ptr(), old.data_ptr(), diff.data_ptr(), n, 1, ws.data_ptr(), both.data_ptr(),
+                                           xws.data_ptr(), both.data_ptr() + 16, _lib.stream_ptr(nw.device))
+            _lib.check(rc, "DeltaEncoder.encode")
+            changed, adler, low, high = (int(v) for v in both.tolist())
+            digest = _hex128(low, high)
+        elif self.delta_encoding == "xor":
             diff = torch.empty_like(nw)
             _xor_pass(nw, old, diff, True, ws, result)
             changed, adler = (int(v) for v in result.tolist())
@@ -333,5 +357,6 @@ class DeltaEncoder:
         if not changed:
             return None, None, 0
         self.changed_bytes += changed
-        digest = f"{adler:08x}" if self.checksum_algorithm == "adler32" else checksum(self.checksum_algorithm, nw)
+        if digest is None:
+            digest = f"{adler:08x}" if self.checksum_algorithm == "adler32" else checksum(self.checksum_algorithm, nw)
         return diff, digest, changed

@@ -111,3 +111,85 @@ def test_delta_encoder_uses_the_gpu_digest_by_default(cuda, monkeypatch):
     state["l0.weight"] = state["l0.weight"] - 1
     _, digest, changed = enc.encode("l0.weight", state["l0.weight"].to(cuda))
     assert changed and digest == _lib_hex(state["l0.weight"])
+
+
+# ---- the digest computed by the delta pass itself ----------------------------------------------------------------
+
+FUSED_SIZES = [0, 1, 15, 16, 17, 240, 241, 1023, 1024, 1025, 1088, 2049, 16383, 16384, 16385, 16384 + 1024, 16384 + 1025,
+               65521, 100000, (1 << 20) + 3, 16384 * 300, 16384 * 300 + 1, 2 * 2560 * 9728]
+
+
+def _fused_pairs():
+    rng = np.random.default_rng(77)
+    pairs = []
+    for i, n in enumerate(FUSED_SIZES):
+        new = rng.integers(0, 256, n, dtype=np.uint8)
+        old = new.copy()
+        if i % 5 != 3 and n:                      # every fifth tensor is left unchanged
+            flip = rng.random(n) < 0.05
+            flip[rng.integers(0, n)] = True
+            old[flip] ^= rng.integers(1, 256, int(flip.sum()), dtype=np.uint8)
+        pairs.append((new, old))
+    return pairs
+
+
+@pytest.mark.parametrize("form", ["searched", "per_chunk", "single"])
+@pytest.mark.parametrize("update", [False, True])
+def test_digest_from_the_delta_pass(cuda, form, update):
+    from oracle import delta_ref as D
+
+    pairs = _fused_pairs()
+    news = [torch.from_numpy(p[0]).to(cuda) for p in pairs]
+    olds = [torch.from_numpy(p[1]).to(cuda) for p in pairs]
+    if form == "searched":
+        diffs, results, digests = delta.xor_diff_many(news, olds, update_snapshot=update, xxh3=True)
+        hexes = [delta._hex128(lo, hi) if c else None for (lo, hi), (c, _) in zip(digests.tolist(), results.tolist())]
+    elif form == "per_chunk":
+        keep = [(a, b) for a, b in zip(news, olds) if a.numel()]          # a plan wants real addresses
+        plan = delta.XorDiffPlan([a for a, _ in keep], [b for _, b in keep], xxh3=True)
+        diffs, results = plan.run(update_snapshot=update)
+        hexes = plan.hexdigests()
+        pairs = [p for p in pairs if p[0].size]
+        olds = [b for _, b in keep]
+    else:
+        lib = _lib.load()
+        diffs, rows, hexes = [], [], []
+        for a, b in zip(news, olds):
+            n = a.numel()
+            diff = torch.empty_like(a)
+            ws = torch.empty(lib.wq_delta_workspace_bytes(n) // 8, dtype=torch.int64, device=cuda)
+            xws = torch.empty(lib.wq_xxh3_workspace_bytes(n) // 8, dtype=torch.int64, device=cuda)
+            out = torch.empty(4, dtype=torch.int64, device=cuda)
+            _lib.check(lib.wq_delta_xor_xxh3(a.data_ptr() if n else None, b.data_ptr() if n else None, diff.data_ptr() if n else None,
+                                             n, int(update), ws.data_ptr(), out.data_ptr(), xws.data_ptr(), out.data_ptr() + 16,
+                                             _lib.stream_ptr(cuda)), "wq_delta_xor_xxh3")
+            c, adler, lo, hi = out.tolist()
+            diffs.append(diff)
+            rows.append([c, adler])
+            hexes.append(delta._hex128(lo, hi) if c else None)
+            if not c:
+                assert (lo, hi) == (0, 0)
+        results = torch.tensor(rows)
+    for (new, old), diff, res, og, hx in zip(pairs, diffs, results.tolist(), olds, hexes):
+        want, changed = D.xor_delta_ref(new, old)
+        assert np.array_equal(diff.cpu().numpy(), want), new.size
+        assert res == [changed, int(D.adler32_ref(new), 16)], new.size
+        assert np.array_equal(og.cpu().numpy(), new if update else old), new.size
+        assert hx == (xxhash.xxh3_128(new.tobytes()).hexdigest() if changed else None), new.size
+
+
+def test_plan_with_digest_is_reusable_and_matches_the_two_pass_form(cuda):
+    g = torch.Generator(device=cuda).manual_seed(5)
+    news = [torch.randint(0, 256, (n,), dtype=torch.uint8, device=cuda, generator=g) for n in (300000, 16384 * 64, 5000, 2 * 1024 * 2560)]
+    olds = [t.clone() for t in news]
+    plan = delta.XorDiffPlan(news, olds, xxh3=True)
+    plan.run(update_snapshot=True)
+    assert plan.hexdigests() == [None] * 4 and plan.results[:, 0].tolist() == [0] * 4
+    news[1][12345] ^= 1
+    news[3][-1] ^= 0x80
+    plan.run(update_snapshot=True)
+    want = delta.xxh3_128_many(news)
+    assert plan.hexdigests() == [None, want[1], None, want[3]] and plan.results[:, 0].tolist() == [0, 1, 0, 1]
+    assert all(torch.equal(a, b) for a, b in zip(news, olds))
+    plan.run(update_snapshot=True)                     # snapshot caught up: nothing changed, no digests
+    assert plan.hexdigests() == [None] * 4
