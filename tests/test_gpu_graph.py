@@ -80,17 +80,22 @@ def test_bucket_convert_replays_in_a_graph(cuda, cfg):
             assert I.same_bits(a, b), (n, k)
 
 
-def test_delta_pass_replays_in_a_graph(cuda):
-    news = [I.weights(256, 384, seed=1).to(cuda), I.weights(1000, 130, seed=2).to(cuda)]
+@pytest.mark.parametrize("with_digest", [False, True])
+def test_delta_pass_replays_in_a_graph(cuda, with_digest):
+    news = [I.weights(256, 384, seed=1).to(cuda), I.weights(1000, 130, seed=2).to(cuda), I.weights(64, 128, seed=3).to(cuda)]
     olds = [t.clone().view(torch.uint8).flatten() for t in news]          # the snapshot in HBM
     _step(news, 7)
-    plan = delta.XorDiffPlan(news, olds, want_diff=True)
+    plan = delta.XorDiffPlan(news, olds, want_diff=True, xxh3=with_digest)
     graph = _capture(lambda: plan.run(update_snapshot=True))
     for k in range(3):
         before = [o.clone() for o in olds]
-        _step(news, k)
+        _step(news[:2], k)                                                  # the third tensor stays as it is
         graph.replay()
         torch.cuda.synchronize()
+        if with_digest:                                                     # the digest of what changed, nothing for the rest
+            moved = [not torch.equal(nw.view(torch.uint8).flatten(), ob) for nw, ob in zip(news, before)]
+            assert moved[1] and not moved[2], k
+            assert plan.hexdigests() == [h if m else None for h, m in zip(delta.xxh3_128_many(news), moved)], k
         for nw, old_before, old_now, diff, res in zip(news, before, olds, plan.diffs, plan.results.cpu()):
             nb = nw.view(torch.uint8).flatten()
             want = nb ^ old_before
