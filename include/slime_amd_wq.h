@@ -345,14 +345,16 @@ int wq_int4_fake_quant_ste_items(const wq_int4_ste_item *items, int64_t n_items,
  *
  * wq_delta_overwrite_encode replaces overwrite_encode(new, new != old), slime/utils/disk_delta.py:21-25:
  *   out = [count u32 LE][positions u32 LE x count, ascending][new[position] x count]
- * Call wq_delta_xor first on the same (new, old, n, workspace) with update_old == 0, read back
- * count = result[0], size `out` to 4 + 5 * count bytes (4-byte aligned), then call this.  n <= 2^32 - 1. */
+ * Call wq_delta_xor (or wq_delta_xor_xxh3) first on the same (new, old, n, workspace) with update_old == 0, read back
+ * count = result[0], size `out` to 4 + 5 * count bytes (4-byte aligned), then call this.  n <= 2^32 - 1.
+ * With update_old != 0 the same pass brings the snapshot up to date (old[i] = new[i]; `collect`:
+ * snapshot[name] = new, update_weight_from_disk_delta.py:246-251), so the encoding needs no third pass. */
 #define WQ_DELTA_CHUNK 16384
 int64_t wq_delta_workspace_bytes(int64_t n);
 int wq_delta_xor(const void *new_bytes, void *old_bytes, void *diff, int64_t n, int update_old,
                  void *workspace, uint64_t *result, void *stream);
-int wq_delta_overwrite_encode(const void *new_bytes, const void *old_bytes, int64_t n, void *workspace,
-                              uint32_t count, void *out, void *stream);
+int wq_delta_overwrite_encode(const void *new_bytes, void *old_bytes, int64_t n, void *workspace,
+                              uint32_t count, void *out, int update_old, void *stream);
 
 /* wq_delta_xor without the workspace argument, for callers that cannot allocate device memory (code under HIP
  * graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.

@@ -64,7 +64,7 @@ SIGNATURES = {
     "wq_int4_fake_quant_ste": [_vp, _vp, _i64, _i64, _int, _int, _vp],
     "wq_delta_workspace_bytes": [_i64],
     "wq_delta_xor": [_vp, _vp, _vp, _i64, _int, _vp, _vp, _vp],
-    "wq_delta_overwrite_encode": [_vp, _vp, _i64, _vp, ctypes.c_uint32, _vp, _vp],
+    "wq_delta_overwrite_encode": [_vp, _vp, _i64, _vp, ctypes.c_uint32, _vp, _int, _vp],
     "wq_delta_xor_noalloc": [_vp, _vp, _vp, _i64, _int, _vp, _vp],
     "wq_delta_xor_grouped": [_vp, _vp, _int, _i64, _int, _int, _int, _vp],
     "wq_delta_xor_xxh3": [_vp, _vp, _vp, _i64, _int, _vp, _vp, _vp, _vp, _vp],

@@ -333,7 +333,8 @@ __device__ __forceinline__ uint32_t wave_exclusive_sum(uint32_t v, uint32_t& tot
 // out = [count u32][positions u32 x count][values u8 x count].  A wave owns a contiguous quarter of the
 // chunk (four steps of 64 lanes x 16 bytes, all loaded before first use); lanes rank their changed bytes
 // with a wave prefix sum, waves are ordered through LDS, chunks through `offsets`.
-__global__ __launch_bounds__(256) void delta_overwrite_kernel(const uint8_t* __restrict__ nw, const uint8_t* __restrict__ old,
+template <bool UPDATE>
+__global__ __launch_bounds__(256) void delta_overwrite_kernel(const uint8_t* __restrict__ nw, uint8_t* __restrict__ old,
                                                              int64_t n, const uint32_t* __restrict__ offsets,
                                                              uint32_t count, uint8_t* __restrict__ out, int64_t items)
 {
@@ -384,6 +385,10 @@ __global__ __launch_bounds__(256) void delta_overwrite_kernel(const uint8_t* __r
             stg<uint32_t>(pos_out + r, (uint32_t)(off + k));
             stg<uint8_t>(val_out + r, (uint8_t)(w4[k >> 2] >> (8 * (k & 3))));
             ++r;
+        }
+        if (UPDATE && mask[i]) {                         // the snapshot catches up where it differs
+            if (off + 16 <= n) stg_nt<u32x4>(old + off, a[i]);
+            else store_tail(old + off, a[i], (int)(n - off));
         }
     }
 }
@@ -534,8 +539,8 @@ WQ_EXPORT int wq_delta_xor_items(const wq_delta_chunk_item* items, int64_t n_ite
     return with_xxh3 ? xxh3_chain_for_delta(nullptr, descs, n_desc, st) : WQ_OK;
 }
 
-WQ_EXPORT int wq_delta_overwrite_encode(const void* new_bytes, const void* old_bytes, int64_t n, void* workspace,
-                                        uint32_t count, void* out, void* stream)
+WQ_EXPORT int wq_delta_overwrite_encode(const void* new_bytes, void* old_bytes, int64_t n, void* workspace,
+                                        uint32_t count, void* out, int update_old, void* stream)
 {
     if (n < 0 || n > 0xFFFFFFFFll) return n < 0 ? WQ_ERR_SHAPE : WQ_ERR_TOO_LARGE;   // positions are uint32
     if (!out || !workspace) return WQ_ERR_NULL;
@@ -551,8 +556,12 @@ WQ_EXPORT int wq_delta_overwrite_encode(const void* new_bytes, const void* old_b
     }
     // an empty tensor still gets its header word (count = 0) from workgroup 0
     const int64_t launch_items = items > 0 ? items : 1;
-    delta_overwrite_kernel<<<grid_for_items(launch_items), 256, 0, st>>>(
-        (const uint8_t*)new_bytes, (const uint8_t*)old_bytes, n, offsets, count, (uint8_t*)out, launch_items);
+    if (update_old)
+        delta_overwrite_kernel<true><<<grid_for_items(launch_items), 256, 0, st>>>(
+            (const uint8_t*)new_bytes, (uint8_t*)old_bytes, n, offsets, count, (uint8_t*)out, launch_items);
+    else
+        delta_overwrite_kernel<false><<<grid_for_items(launch_items), 256, 0, st>>>(
+            (const uint8_t*)new_bytes, (uint8_t*)old_bytes, n, offsets, count, (uint8_t*)out, launch_items);
     WQ_LAUNCH_CHECK();
     return WQ_OK;
 }

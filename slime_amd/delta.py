@@ -178,10 +178,11 @@ def _check_old(nw: torch.Tensor, old: torch.Tensor) -> None:
         raise ValueError("snapshot must live on the tensor's device at a 16-byte aligned address")
 
 
-def overwrite_encode(new: torch.Tensor, old: torch.Tensor) -> torch.Tensor:
+def overwrite_encode(new: torch.Tensor, old: torch.Tensor, update_snapshot: bool = False) -> torch.Tensor:
     """The 'overwrite' delta of slime/utils/disk_delta.py:21-25 for ``changed_mask = new != old``:
     uint8 vector [count u32 LE][positions u32 LE x count][new values x count].  Synchronises once (the output
-    size depends on the count)."""
+    size depends on the count).  With ``update_snapshot`` the pass that writes the encoding also sets ``old`` to the
+    new bytes."""
     nw = _as_bytes(new, "overwrite_encode")
     _check_old(nw, old)
     if nw.numel() > 0xFFFFFFFF:
@@ -193,7 +194,7 @@ def overwrite_encode(new: torch.Tensor, old: torch.Tensor) -> torch.Tensor:
     out = torch.empty(4 + 5 * count, dtype=torch.uint8, device=nw.device)
     with torch.cuda.device(nw.device):
         rc = _lib.load().wq_delta_overwrite_encode(nw.data_ptr(), old.data_ptr(), nw.numel(), ws.data_ptr(), count,
-                                                   out.data_ptr(), _lib.stream_ptr(nw.device))
+                                                   out.data_ptr(), int(update_snapshot), _lib.stream_ptr(nw.device))
     _lib.check(rc, "overwrite_encode")
     return out
 
@@ -325,35 +326,30 @@ class DeltaEncoder:
         _check_old(nw, old)
         n = nw.numel()
         self.total_bytes += n
+        lib = _lib.load()
         ws = _workspace(n, nw.device)
-        result = torch.empty(2, dtype=torch.int64, device=nw.device)
-        digest = None
-        if self.delta_encoding == "xor" and self.checksum_algorithm == "xxh3-128":
-            diff = torch.empty_like(nw)
-            lib = _lib.load()
-            xws = torch.empty(lib.wq_xxh3_workspace_bytes(n) // 8, dtype=torch.int64, device=nw.device)
-            both = torch.empty(4, dtype=torch.int64, device=nw.device)      # result, then digest
+        both = torch.empty(4, dtype=torch.int64, device=nw.device)      # [changed bytes, adler32], then the digest
+        fused = self.checksum_algorithm == "xxh3-128"                   # the digest rides on the pass that counts / diffs
+        xor = self.delta_encoding == "xor"
+        diff = torch.empty_like(nw) if xor else None
+        with torch.cuda.device(nw.device):
+            if fused:
+                xws = torch.empty(lib.wq_xxh3_workspace_bytes(n) // 8, dtype=torch.int64, device=nw.device)
+                rc = lib.wq_delta_xor_xxh3(nw.data_ptr(), old.data_ptr(), diff.data_ptr() if xor else None, n, int(xor),
+                                           ws.data_ptr(), both.data_ptr(), xws.data_ptr(), both.data_ptr() + 16,
+                                           _lib.stream_ptr(nw.device))
+            else:
+                rc = lib.wq_delta_xor(nw.data_ptr(), old.data_ptr(), diff.data_ptr() if xor else None, n, int(xor),
+                                      ws.data_ptr(), both.data_ptr(), _lib.stream_ptr(nw.device))
+        _lib.check(rc, "DeltaEncoder.encode")
+        changed, adler, low, high = (int(v) for v in both.tolist())
+        digest = _hex128(low, high) if fused else None
+        if not xor and changed:                      # the second pass writes the encoding and brings the snapshot up to date
+            diff = torch.empty(4 + 5 * changed, dtype=torch.uint8, device=nw.device)
             with torch.cuda.device(nw.device):
-                rc = lib.wq_delta_xor_xxh3(nw.data_ptr(), old.data_ptr(), diff.data_ptr(), n, 1, ws.data_ptr(), both.data_ptr(),
-                                           xws.data_ptr(), both.data_ptr() + 16, _lib.stream_ptr(nw.device))
+                rc = lib.wq_delta_overwrite_encode(nw.data_ptr(), old.data_ptr(), n, ws.data_ptr(), changed, diff.data_ptr(), 1,
+                                                   _lib.stream_ptr(nw.device))
             _lib.check(rc, "DeltaEncoder.encode")
-            changed, adler, low, high = (int(v) for v in both.tolist())
-            digest = _hex128(low, high)
-        elif self.delta_encoding == "xor":
-            diff = torch.empty_like(nw)
-            _xor_pass(nw, old, diff, True, ws, result)
-            changed, adler = (int(v) for v in result.tolist())
-        else:
-            _xor_pass(nw, old, None, False, ws, result)
-            changed, adler = (int(v) for v in result.tolist())
-            diff = None
-            if changed:
-                diff = torch.empty(4 + 5 * changed, dtype=torch.uint8, device=nw.device)
-                with torch.cuda.device(nw.device):
-                    rc = _lib.load().wq_delta_overwrite_encode(nw.data_ptr(), old.data_ptr(), n, ws.data_ptr(), changed,
-                                                               diff.data_ptr(), _lib.stream_ptr(nw.device))
-                _lib.check(rc, "DeltaEncoder.encode")
-            old.copy_(nw)
         if not changed:
             return None, None, 0
         self.changed_bytes += changed

@@ -50,10 +50,14 @@ def test_adler32_extreme_bytes(cuda):
 @pytest.mark.parametrize("density", [0.0, 0.002, 0.3, 1.0])
 def test_overwrite_encode(cuda, n, density):
     new, old = _pair(n, density, 7 * n + 3)
-    enc = delta.overwrite_encode(torch.from_numpy(new).to(cuda), torch.from_numpy(old).to(cuda)).cpu().numpy()
+    old_dev = torch.from_numpy(old).to(cuda)
+    enc = delta.overwrite_encode(torch.from_numpy(new).to(cuda), old_dev).cpu().numpy()
     want, _ = D.overwrite_delta_ref(new, old)
     assert np.array_equal(enc, want)
     assert np.array_equal(D.overwrite_apply_ref(old, enc), new)
+    assert np.array_equal(old_dev.cpu().numpy(), old)                       # left alone unless asked
+    enc2 = delta.overwrite_encode(torch.from_numpy(new).to(cuda), old_dev, update_snapshot=True).cpu().numpy()
+    assert np.array_equal(enc2, want) and np.array_equal(old_dev.cpu().numpy(), new)
 
 
 def test_weights_of_any_dtype_and_views(cuda):
@@ -66,13 +70,19 @@ def test_weights_of_any_dtype_and_views(cuda):
     assert np.array_equal(diff.cpu().numpy(), want) and int(result[0]) == changed
 
 
+@pytest.mark.parametrize("digest_name", ["adler32", "xxh3-128"])
 @pytest.mark.parametrize("encoding", ["xor", "overwrite"])
-def test_delta_encoder_follows_the_reference_loop(cuda, encoding):
+def test_delta_encoder_follows_the_reference_loop(cuda, encoding, digest_name):
+    if digest_name == "adler32":
+        digest_ref = D.adler32_ref
+    else:
+        xxhash = pytest.importorskip("xxhash")
+        digest_ref = lambda b: xxhash.xxh3_128(b.tobytes()).hexdigest()   # noqa: E731
     names = ["a.weight", "b.weight", "c.bias"]
     shapes = [(512, 384), (129, 77), (1000,)]
     g = torch.Generator().manual_seed(5)
     state = {n: torch.randn(*s, generator=g).to(torch.bfloat16) for n, s in zip(names, shapes)}
-    enc = delta.DeltaEncoder(encoding, "adler32")
+    enc = delta.DeltaEncoder(encoding, digest_name)
     snapshot = {}
     for n, t in state.items():
         enc.capture(n, t.to(cuda))
@@ -91,7 +101,7 @@ def test_delta_encoder_follows_the_reference_loop(cuda, encoding):
                 want, want_changed = D.overwrite_delta_ref(new, snapshot[n])
             assert changed == want_changed
             if want_changed:
-                assert np.array_equal(diff.cpu().numpy(), want) and digest == D.adler32_ref(new)
+                assert np.array_equal(diff.cpu().numpy(), want) and digest == digest_ref(new)
             else:
                 assert diff is None and digest is None
             snapshot[n] = new.copy()
