@@ -110,7 +110,13 @@ def xor_diff_many(news, olds, update_snapshot: bool = False, want_diff: bool = T
     if not news:
         empty = torch.empty((0, 2), dtype=torch.int64)
         return (([] if want_diff else None), empty) + ((empty,) if xxh3 else ())
-    flat = [_as_bytes(t, "xor_diff_many") for t in news]
+    p = _grouped_pass([_as_bytes(t, "xor_diff_many") for t in news], olds, update_snapshot, want_diff, xxh3)
+    return (p["diffs"], p["results"]) + ((p["digests"],) if xxh3 else ())
+
+
+def _grouped_pass(flat, olds, update_snapshot: bool, want_diff: bool, xxh3: bool) -> dict:
+    """One wq_delta_xor_grouped over byte views ``flat``; keeps the workspace (its per-chunk counts are what the
+    overwrite encoding consumes) next to the results."""
     device = flat[0].device
     rows, flat_diff, flat_ws, results, digests, diffs = _bucket_tables(flat, olds, want_diff, xxh3, device)
     starts, chunks = [0], 0
@@ -123,7 +129,7 @@ def xor_diff_many(news, olds, update_snapshot: bool = False, want_diff: bool = T
         rc = _lib.load().wq_delta_xor_grouped(descs.data_ptr(), start_t.data_ptr(), len(flat), chunks, int(want_diff),
                                               int(update_snapshot), int(xxh3), _lib.stream_ptr(device))
     _lib.check(rc, "xor_diff_many")
-    return (diffs, results) + ((digests,) if xxh3 else ())
+    return {"rows": rows, "workspace": flat_ws, "results": results, "digests": digests, "diffs": diffs, "tables": (descs, start_t)}
 
 
 class XorDiffPlan:
@@ -294,27 +300,41 @@ class DeltaEncoder:
         self.snapshot[name] = _as_bytes(tensor, "DeltaEncoder.capture").clone()
 
     def encode_bucket(self, named_tensors):
-        """``encode`` for a list of (name, tensor) with two kernel launches and one synchronisation (xor encoding
-        only).  -> list of (name, diff_or_None, checksum_or_None, changed) in input order."""
-        if self.delta_encoding != "xor":
-            return [(name,) + self.encode(name, t) for name, t in named_tensors]
+        """``encode`` for a list of (name, tensor) with one synchronisation: one pass over the whole bucket for the xor
+        diff (or, for the overwrite encoding, the counts), adler32, the xxh3-128 digest and the snapshot update, then -
+        overwrite only - one scatter launch per tensor that changed.
+        -> list of (name, diff_or_None, checksum_or_None, changed) in input order."""
         named_tensors = list(named_tensors)
-        fused = self.checksum_algorithm == "xxh3-128"       # the digest rides on the diff pass: no second read
-        got = xor_diff_many([t for _, t in named_tensors], [self.snapshot[n] for n, _ in named_tensors],
-                            update_snapshot=True, xxh3=fused)
-        diffs, results = got[0], got[1].tolist()
-        digests = {i: _hex128(low, high) for i, (low, high) in enumerate(got[2].tolist())} if fused else {}
-        out = []
-        for i, ((name, t), diff, (changed, adler)) in enumerate(zip(named_tensors, diffs, results)):
-            self.total_bytes += diff.numel()
+        if not named_tensors:
+            return []
+        xor = self.delta_encoding == "xor"
+        fused = self.checksum_algorithm == "xxh3-128"       # the digest rides on the pass: no second read
+        flat = [_as_bytes(t, "DeltaEncoder.encode_bucket") for _, t in named_tensors]
+        olds = [self.snapshot[n] for n, _ in named_tensors]
+        if not xor and any(f.numel() > 0xFFFFFFFF for f in flat):
+            raise ValueError("overwrite encoding: positions are uint32; tensor too large")
+        p = _grouped_pass(flat, olds, update_snapshot=xor, want_diff=xor, xxh3=fused)
+        results = p["results"].tolist()                      # the one synchronisation
+        digests = p["digests"].tolist() if fused else None
+        lib, out = _lib.load(), []
+        for i, ((name, t), nw, old, (changed, adler)) in enumerate(zip(named_tensors, flat, olds, results)):
+            self.total_bytes += nw.numel()
             if not changed:
                 out.append((name, None, None, 0))
                 continue
             self.changed_bytes += changed
+            if xor:
+                diff = p["diffs"][i]
+            else:                                            # scatter + snapshot update, from the counts the pass left
+                diff = torch.empty(4 + 5 * changed, dtype=torch.uint8, device=nw.device)
+                with torch.cuda.device(nw.device):
+                    rc = lib.wq_delta_overwrite_encode(nw.data_ptr(), old.data_ptr(), nw.numel(), p["rows"][i][4], changed,
+                                                       diff.data_ptr(), 1, _lib.stream_ptr(nw.device))
+                _lib.check(rc, "DeltaEncoder.encode_bucket")
             if self.checksum_algorithm == "adler32":
                 digest = f"{adler:08x}"
-            elif i in digests:
-                digest = digests[i]
+            elif fused:
+                digest = _hex128(*digests[i])
             else:
                 digest = checksum(self.checksum_algorithm, t)
             out.append((name, diff, digest, changed))

@@ -148,26 +148,39 @@ def test_bucket_launch_equals_single_calls(cuda):
     assert none is None and torch.equal(results2, results)
 
 
-def test_delta_encoder_bucket(cuda):
+@pytest.mark.parametrize("digest_name", ["adler32", "xxh3-128"])
+@pytest.mark.parametrize("encoding", ["xor", "overwrite"])
+def test_delta_encoder_bucket(cuda, encoding, digest_name):
+    if digest_name == "adler32":
+        digest_ref = D.adler32_ref
+    else:
+        xxhash = pytest.importorskip("xxhash")
+        digest_ref = lambda b: xxhash.xxh3_128(b.tobytes()).hexdigest()   # noqa: E731
     g = torch.Generator().manual_seed(9)
-    state = {f"l{i}.weight": torch.randn(64 + i, 96, generator=g).to(torch.bfloat16) for i in range(6)}
-    enc = delta.DeltaEncoder("xor", "adler32")
+    state = {f"l{i}.weight": torch.randn(64 + i, 96 + 300 * i, generator=g).to(torch.bfloat16) for i in range(6)}
+    enc = delta.DeltaEncoder(encoding, digest_name)
     for n, t in state.items():
         enc.capture(n, t.to(cuda))
     old = {n: t.view(torch.uint8).reshape(-1).numpy().copy() for n, t in state.items()}
-    state["l2.weight"] = state["l2.weight"] * 2
-    state["l5.weight"] = state["l5.weight"] + 1
-    out = enc.encode_bucket([(n, t.to(cuda)) for n, t in state.items()])
-    assert [o[0] for o in out] == list(state)
-    for name, diff, digest, changed in out:
-        new = state[name].view(torch.uint8).reshape(-1).numpy()
-        want, want_changed = D.xor_delta_ref(new, old[name])
-        assert changed == want_changed
-        if changed:
-            assert np.array_equal(diff.cpu().numpy(), want) and digest == D.adler32_ref(new)
-        else:
-            assert diff is None and name not in ("l2.weight", "l5.weight")
-        assert np.array_equal(enc.snapshot[name].cpu().numpy(), new)
+    assert enc.encode_bucket([]) == []
+    for step in range(2):
+        state["l2.weight"] = state["l2.weight"] * 2
+        state["l5.weight"] = state["l5.weight"] + 1
+        if step:
+            state["l0.weight"] = -state["l0.weight"]
+        out = enc.encode_bucket([(n, t.to(cuda)) for n, t in state.items()])
+        assert [o[0] for o in out] == list(state)
+        for name, diff, digest, changed in out:
+            new = state[name].view(torch.uint8).reshape(-1).numpy()
+            want, want_changed = (D.xor_delta_ref if encoding == "xor" else D.overwrite_delta_ref)(new, old[name])
+            assert changed == want_changed
+            if changed:
+                assert np.array_equal(diff.cpu().numpy(), want) and digest == digest_ref(new)
+            else:
+                assert diff is None and digest is None and name not in ("l2.weight", "l5.weight")
+            assert np.array_equal(enc.snapshot[name].cpu().numpy(), new)
+            old[name] = new.copy()
+    assert enc.total_bytes == 2 * sum(v.size for v in old.values()) and enc.changed_bytes > 0
 
 
 def test_unknown_digest_names(cuda):
