@@ -760,9 +760,26 @@ def bench_copy(dev, steps, warmup, nbytes=4 << 30):
 
     wall_ms, ev_ms, ev_min = _time_launches(run, steps, warmup)
     assert torch.equal(src[:1 << 20], dst[:1 << 20]) and torch.equal(src[-(1 << 20):], dst[-(1 << 20):])
-    return {"workload": "copy_kernel 4 GiB", "bytes_read": nbytes, "bytes_written": nbytes, "kernel_ms": ev_ms,
-            "kernel_ms_min": ev_min, "GBps_read_plus_write": 2 * nbytes / ev_ms / 1e6,
-            "hbm_frac": 2 * nbytes / ev_ms / 1e6 / HBM_PEAK_GBS}
+    rec = {"workload": "copy_kernel 4 GiB", "bytes_read": nbytes, "bytes_written": nbytes, "kernel_ms": ev_ms,
+           "kernel_ms_min": ev_min, "GBps_read_plus_write": 2 * nbytes / ev_ms / 1e6,
+           "hbm_frac": 2 * nbytes / ev_ms / 1e6 / HBM_PEAK_GBS}
+    # the same for the quantisers' read:write mixes: compute-free 2:1 and 4:1 streams over the same 4 GiB of input
+    for ratio in (2, 4):
+        n_out = nbytes // ratio
+
+        def fold():
+            _lib.check(_lib.load().wq_stream_fold_bytes(src.data_ptr(), dst.data_ptr(), n_out, ratio, _lib.stream_ptr(dev)), "fold")
+
+        _, f_ms, f_min = _time_launches(fold, steps, warmup)
+        piece = {2: 16384, 4: 8192}[ratio]                   # bytes of output per work item
+        pieces = src[:ratio * piece].view(ratio, piece)
+        want = pieces[0].clone()
+        for r in range(1, ratio):
+            want ^= pieces[r]
+        assert torch.equal(dst[:piece], want)
+        rec[f"compute_free_{ratio}_to_1"] = {"bytes_read": nbytes, "bytes_written": n_out, "kernel_ms": f_ms, "kernel_ms_min": f_min,
+                                              "hbm_frac": (nbytes + n_out) / f_ms / 1e6 / HBM_PEAK_GBS}
+    return rec
 
 
 def bench_stream(dev, n_buckets=64, bucket_bytes=1 << 30, download=True):
@@ -1016,8 +1033,14 @@ def main():
         extras["delta_xor"] = bench_delta(dev, args.steps, args.warmup)
         extras["single_tensor_forms"] = bench_single_tensor_forms(dev, args.steps, args.warmup)
         extras["grouped_expert_weights"] = bench_grouped_experts(dev, args.steps, args.warmup)
-        # the practical ceiling of a 1:1 read:write stream on this very box, measured in this very run
-        extras["copy_kernel_calibration"] = bench_copy(dev, args.steps, args.warmup)
+        # the practical ceilings of 1:1, 2:1 and 4:1 read:write streams on this very box, measured in this very run
+        cal = bench_copy(dev, args.steps, args.warmup)
+        extras["copy_kernel_calibration"] = cal
+        line["roofline"]["same_run_compute_free_streams"] = {
+            "note": "fraction of the 8 TB/s peak that kernels with no arithmetic reach on this box in this run: plain copy, and the "
+                    "block-FP8 quantiser's (2:1) and the INT4 packer's (4:1) read:write mix over contiguous 16-32 KiB pieces",
+            "copy_1_to_1": cal["hbm_frac"], "fold_2_to_1": cal["compute_free_2_to_1"]["hbm_frac"],
+            "fold_4_to_1": cal["compute_free_4_to_1"]["hbm_frac"]}
         line["other_workloads"] = extras
     print(json.dumps(line))
 

@@ -461,6 +461,12 @@ int wq_selftest_decode_fp8(uint64_t *out, void *stream);
  * that hardware counters are scaled against. */
 int wq_copy_bytes(const void *src, void *dst, int64_t n_bytes, void *stream);
 
+/* A compute-free stream with `reads_per_write` (2 or 4) bytes read per byte written - the block-FP8 quantiser's and the
+ * INT4 packer's read:write mix: dst[16 KiB piece i] = xor of src[pieces reads_per_write * i ...].  n_out_bytes a multiple
+ * of 16384; src holds reads_per_write * n_out_bytes.  The benchmark runs it next to the quantisers to show what the
+ * memory system gives that mix on the box at hand. */
+int wq_stream_fold_bytes(const void *src, void *dst, int64_t n_out_bytes, int reads_per_write, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -74,6 +74,7 @@ SIGNATURES = {
     "wq_selftest_cvt_bf16": [_u64, _u64, _vp, _vp],
     "wq_selftest_decode_fp8": [_vp, _vp],
     "wq_copy_bytes": [_vp, _vp, _i64, _vp],
+    "wq_stream_fold_bytes": [_vp, _vp, _i64, _int, _vp],
 }
 
 _lib = None

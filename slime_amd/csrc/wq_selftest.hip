@@ -145,6 +145,37 @@ __global__ __launch_bounds__(256) void copy_kernel(const u32x4* __restrict__ src
     }
 }
 
+// A compute-free stream with R bytes read per byte written (R = 2: the block-FP8 quantiser's mix, R = 4: the INT4 packer's):
+// an item is STEPS x 4 KiB of output, the xor of R consecutive pieces of the input of that size.  It shows what the memory
+// system gives this read:write mix on the box at hand, the way the plain copy does for 1:1.
+constexpr int kFoldItemsPerXcdRun = 64;
+// Launch shape by measurement (% of the 8 TB/s HBM peak, 4 GiB read): both mixes stream best with eight 16-byte loads per lane
+// and two workgroups per CU - 2:1 83.3 (4 / 3 workgroups per CU: 78-80), 4:1 83.7 (four loads per lane 80.8, sixteen 78; at full
+// occupancy 74-77).
+constexpr unsigned kFoldPadBytes2 = 77 * 1024, kFoldPadBytes4 = 77 * 1024;      // two workgroups per CU
+constexpr int kFoldSteps2 = 4, kFoldSteps4 = 2;                                 // output pieces per lane
+
+template <int R, int STEPS>
+__global__ __launch_bounds__(256) void fold_kernel(const u32x4* __restrict__ src, u32x4* __restrict__ dst, int64_t items)
+{
+    const int64_t slot = (int64_t)blockIdx.x + (int64_t)blockIdx.y * gridDim.x;
+    if (slot >= items) return;
+    const int64_t item = xcd_chunked_item(slot, items, kFoldItemsPerXcdRun);
+    const u32x4* in = src + item * (R * STEPS * 256) + threadIdx.x;
+    u32x4 v[R][STEPS];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int i = 0; i < STEPS; ++i) v[r][i] = __builtin_nontemporal_load(in + (r * STEPS + i) * 256);
+#pragma unroll
+    for (int i = 0; i < STEPS; ++i) {
+        u32x4 acc = v[0][i];
+#pragma unroll
+        for (int r = 1; r < R; ++r) acc ^= v[r][i];
+        __builtin_nontemporal_store(acc, dst + item * (STEPS * 256) + i * 256 + threadIdx.x);
+    }
+}
+
 }  // namespace wq
 
 using namespace wq;
@@ -245,6 +276,25 @@ WQ_EXPORT int wq_copy_bytes(const void* src, void* dst, int64_t n_bytes, void* s
     const int64_t items = cdiv64(n16, 1024);
     copy_kernel<<<grid_for_items(items), 256, kCopyOccupancyPadBytes, (hipStream_t)stream>>>((const u32x4*)src, (u32x4*)dst,
                                                                                            n16, items);
+    WQ_LAUNCH_CHECK();
+    return WQ_OK;
+}
+
+WQ_EXPORT int wq_stream_fold_bytes(const void* src, void* dst, int64_t n_out_bytes, int reads_per_write, void* stream)
+{
+    if (n_out_bytes < 0 || (n_out_bytes % 16384)) return WQ_ERR_SHAPE;
+    if (reads_per_write != 2 && reads_per_write != 4) return WQ_ERR_MODE;
+    if (n_out_bytes == 0) return WQ_OK;
+    if (!src || !dst) return WQ_ERR_NULL;
+    if (((uintptr_t)src & 15) || ((uintptr_t)dst & 15)) return WQ_ERR_ALIGN;
+    hipStream_t st = (hipStream_t)stream;
+    if (reads_per_write == 2) {
+        const int64_t items = n_out_bytes / (kFoldSteps2 * 4096);
+        fold_kernel<2, kFoldSteps2><<<grid_for_items(items), 256, kFoldPadBytes2, st>>>((const u32x4*)src, (u32x4*)dst, items);
+    } else {
+        const int64_t items = n_out_bytes / (kFoldSteps4 * 4096);
+        fold_kernel<4, kFoldSteps4><<<grid_for_items(items), 256, kFoldPadBytes4, st>>>((const u32x4*)src, (u32x4*)dst, items);
+    }
     WQ_LAUNCH_CHECK();
     return WQ_OK;
 }

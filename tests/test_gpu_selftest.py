@@ -55,3 +55,23 @@ def test_copy_kernel(cuda):
     _lib.check(_lib.load().wq_copy_bytes(src.data_ptr(), dst.data_ptr(), src.numel(),
                                          torch.cuda.current_stream().cuda_stream), "copy")
     assert torch.equal(src, dst)
+
+
+@pytest.mark.parametrize("ratio, piece", [(2, 16384), (4, 8192)])
+def test_fold_stream_kernel(cuda, ratio, piece):
+    """The compute-free R:1 stream the benchmark uses as this box's ceiling for the quantisers' read:write mixes: every output
+    piece is the xor of R consecutive input pieces."""
+    g = torch.Generator().manual_seed(ratio)
+    n_out = 16384 * 37
+    src = torch.randint(0, 256, (ratio * n_out,), generator=g, dtype=torch.int32).to(torch.uint8).cuda()
+    dst = torch.zeros(n_out, dtype=torch.uint8, device="cuda")
+    lib = _lib.load()
+    _lib.check(lib.wq_stream_fold_bytes(src.data_ptr(), dst.data_ptr(), n_out, ratio, torch.cuda.current_stream().cuda_stream), "fold")
+    pieces = src.view(-1, ratio, piece)
+    want = pieces[:, 0].clone()
+    for r in range(1, ratio):
+        want ^= pieces[:, r]
+    assert torch.equal(dst, want.reshape(-1))
+    assert lib.wq_stream_fold_bytes(src.data_ptr(), dst.data_ptr(), n_out, 3, None) == -3          # mode
+    assert lib.wq_stream_fold_bytes(src.data_ptr(), dst.data_ptr(), n_out + 16, ratio, None) == -2  # shape
+    assert lib.wq_stream_fold_bytes(src.data_ptr() + 8, dst.data_ptr(), n_out, ratio, None) == -5   # alignment
