@@ -25,13 +25,15 @@ namespace wq {
 //   256 threads, runs of 32 tiles per XCD, 3 workgroups per CU                   73.6 %
 //   512 threads (4 loads per lane), runs of 16 / 32 / 64 tiles                   75.5 / 76.1 / 76.3 %
 //   512 threads, plain dispatch order                                            71.1 %
-// A compute-free kernel with the same 2:1 read:write mix tops out at 86 % on this part.
+// A compute-free kernel with the same tiles (128 rows x 256 bytes in, 128 x 128 out, same work order) reaches 81.5-82.9 %, one with
+// the same 2:1 mix over contiguous 32 KiB pieces 83-84 %.
 constexpr int kTileThreads = 256;
 constexpr int kTilesPerXcdRun = 32;               // consecutive tiles handed to one XCD (xcd_chunked_item)
 constexpr unsigned kOccupancyPadBytes = 36 * 1024;  // unused dynamic LDS: caps residency at 4 workgroups per CU
 // 16-byte loads a lane keeps in flight while it folds the block maximum: the load of step i + window is issued when step
 // i has been folded in.  On the full Qwen3-30B-A3B-shaped state dict (4 workgroups per CU): all 8 at once 79.1 %, 6: 79.5,
-// 4: 79.1, 3: 79.5, 2: 80.6-80.8 (used), 1: 72.1; with 5 or more workgroups per CU a window lowers the rate.  The
+// 4: 79.1, 3: 79.5, 2: 80.6-80.8 (used), 1: 72.1; with 5 or more workgroups per CU a window lowers the rate, and 3 per CU
+// is behind with every window (2: 77.7, 3: 80.1, 4: 80.0, 8: 78.7).  The
 // Qwen3-4B-shaped pass does not move (76.3-76.6 either way).  A compute-free 2:1 stream of the same shape is fastest at 2
 // workgroups per CU (84 %): fewer bytes in flight per CU suit the memory system, and the window gets part of that while
 // four workgroups keep the arithmetic overlapped.
