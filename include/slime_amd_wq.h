@@ -32,7 +32,7 @@
 extern "C" {
 #endif
 
-#define WQ_ABI_VERSION 16
+#define WQ_ABI_VERSION 17
 
 enum {
     WQ_OK = 0,
@@ -299,7 +299,7 @@ int wq_int4_dequant_any(const int32_t *packed, const void *scale, int scale_dtyp
  * packed word, to the scale of its first element and to its first output element, and its number of words.
  * `group` must be a power of two between 8 and 8 * WQ_INT4_DEQ_WORDS_PER_ITEM, so that an item starts on a group
  * boundary; y pointers 16-byte aligned. */
-#define WQ_INT4_DEQ_WORDS_PER_ITEM 2048
+#define WQ_INT4_DEQ_WORDS_PER_ITEM 512
 typedef struct wq_int4_dequant_item {
     const int32_t *packed;
     const void *scale;   /* bf16 */

@@ -15,7 +15,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libslime_amd_wq.so")
 
-ABI_VERSION = 16
+ABI_VERSION = 17
 
 # selectors (mirrors of the header's enums)
 DTYPE_BF16, DTYPE_F32, DTYPE_F16, DTYPE_F64 = 0, 1, 2, 3
@@ -24,7 +24,7 @@ DIV7_IEEE, DIV7_DEVICE = 0, 1
 DEQ_MODE_F32SCALE, DEQ_MODE_BF16SCALE = 0, 1
 DEQ_SEG, DEQ_SEGS_PER_WG = 512, 16
 INT4_GROUPS_PER_WG = 64
-INT4_DEQ_WORDS_PER_ITEM = 2048
+INT4_DEQ_WORDS_PER_ITEM = 512
 BUCKET_COPY_MARK, BUCKET_COPY_BYTES = -1, 32768
 
 _i64, _int, _vp, _u32, _u64 = ctypes.c_int64, ctypes.c_int, ctypes.c_void_p, ctypes.c_uint32, ctypes.c_uint64

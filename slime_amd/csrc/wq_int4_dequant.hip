@@ -2,8 +2,8 @@
 // estimator, for gfx950.
 //
 // int4_dequant_kernel: every lane turns one packed int32 (8 nibbles) into 8 bf16 and writes them with ONE
-// 16-byte store, so a wavefront reads 256 contiguous bytes and writes 1 KiB contiguous per step; eight steps
-// per lane are all in flight before first use.  f32(nibble - 8) * f32(scale) has at most 12 significant bits,
+// 16-byte store, so a wavefront reads 256 contiguous bytes and writes 1 KiB contiguous per step; the two steps
+// of a lane are both in flight before first use.  f32(nibble - 8) * f32(scale) has at most 12 significant bits,
 // so the fp32 product is exact and the only rounding is the final one to bf16, as in the reference's
 // (int8.to(f32) * scale.to(f32)).to(bf16).
 //
@@ -18,11 +18,15 @@ namespace wq {
 typedef float f32x2d __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2d __attribute__((ext_vector_type(2)));
 
-constexpr int kDqSteps = 8;                       // packed words per lane
-constexpr int kDqWordsPerWg = 256 * kDqSteps;     // 8 KiB of packed input, 64 KiB of bf16 output
+// Work item size and residency by measurement (Qwen3-30B-A3B experts, 8 layers, % of the HBM peak; a compute-free 1:4 stream of
+// the same shapes peaks at 82 % with two or four steps): 8 words per lane at 3 workgroups per CU 77.4-77.8; 4 words at 2 / 3 / 4 / 6
+// per CU 54.4 / 70.5 / 77.2 / 76.9; 3 words 73-76; 2 words at 6 per CU 72.8, at full occupancy 79.0-80.1 (used; runs of 16 / 64 / 128
+// items per XCD instead of 32: 77.4 / 79.5 / 79.4); 1 word 64-65.
+constexpr int kDqSteps = 2;                       // packed words per lane
+constexpr int kDqWordsPerWg = 256 * kDqSteps;     // 2 KiB of packed input, 16 KiB of bf16 output
 static_assert(kDqWordsPerWg == WQ_INT4_DEQ_WORDS_PER_ITEM, "work item size is part of the C ABI");
 constexpr int kDqItemsPerXcdRun = 32;
-constexpr int kDqOccupancyPadBytes = 45 * 1024;           // unused dynamic LDS that caps workgroups per CU
+constexpr int kDqOccupancyPadBytes = 0;           // unused dynamic LDS that would cap workgroups per CU: no cap
 
 __device__ __forceinline__ uint32_t pack2_bf16(float a, float b)
 {
