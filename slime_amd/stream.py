@@ -20,8 +20,6 @@ from typing import Callable, Iterable, Iterator
 
 import torch
 
-from . import _lib
-
 
 class BucketPipeline:
     """Runs ``kernel(dev_in_bucket) -> tuple of device tensors`` over host buckets with overlap.
