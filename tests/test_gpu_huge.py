@@ -100,3 +100,21 @@ def test_delta_pass_over_more_than_4_gib(cuda, big):
         want = zlib.adler32(host[i:i + (1 << 30)], want)
     assert adler == want
     assert delta.checksum("adler32", big) == f"{want:08x}"
+
+
+def test_digest_from_the_delta_pass_over_more_than_4_gib(cuda, big):
+    """4.27 GiB in one tensor: 4.5 M XXH3 blocks summed by the diff kernel and walked in one chain, against the stand-alone
+    digest kernels and the xxhash package on the host."""
+    xxhash = pytest.importorskip("xxhash")
+    nb = big.view(torch.uint8).view(-1)
+    old = nb.clone()
+    old[123456789] ^= 0x40                                                   # one byte differs: the tensor counts as changed
+    _, results, digests = delta.xor_diff_many([big], [old], update_snapshot=True, want_diff=False, xxh3=True)
+    assert results[0, 0].item() == 1 and torch.equal(old, nb)
+    got = delta._hex128(*digests[0].tolist())
+    assert got == delta.xxh3_128(big)
+    hasher = xxhash.xxh3_128()
+    host = nb.cpu().numpy()
+    for i in range(0, host.size, 1 << 30):
+        hasher.update(host[i:i + (1 << 30)])
+    assert got == hasher.hexdigest()
