@@ -23,6 +23,8 @@ import time
 ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
+if os.path.join(ROOT, "tests") not in sys.path:
+    sys.path.append(os.path.join(ROOT, "tests"))         # wq_testlib: the binding of the calibration kernels
 
 HBM_PEAK_GBS = 8000.0
 
@@ -57,6 +59,25 @@ def _time_launches(run, steps: int, warmup: int):
     """-> (wall ms per step over the whole timed region, mean per-launch ms from HIP events, min)."""
     wall_ms, mean, mn = _time_step([run], steps, warmup)
     return wall_ms, mean[0], mn[0]
+
+
+def _time_back_to_back(run, launches: int, rounds: int = 5):
+    """`launches` calls of `run` in a row between ONE pair of HIP events, `rounds` times -> median microseconds per
+    launch.  This is what a loop of per-tensor calls pays per call; an event pair around every single launch adds the
+    cost of the two event packets to each measurement."""
+    import torch
+
+    per = []
+    for _ in range(rounds):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(launches):
+            run()
+        b.record()
+        torch.cuda.synchronize()
+        per.append(a.elapsed_time(b) * 1e3 / launches)
+    per.sort()
+    return per[len(per) // 2]
 
 
 def _gen_bf16(shape, device, std=0.02, outliers=False):
@@ -208,6 +229,7 @@ def bench_cfg1(dev, steps, warmup, n_buffers=8):
     import torch
 
     import slime_amd
+    import wq_testlib
     from oracle import c_oracle
     from slime_amd import _lib
 
@@ -242,6 +264,22 @@ def bench_cfg1(dev, steps, warmup, n_buffers=8):
 
     wall_c, mean_c, _ = _time_step([cold_quant, cold_dequant], max(steps, 2 * n_buffers), max(warmup, n_buffers))
     wall_w, mean_w, _ = _time_step([lambda: quant(0), lambda: dequant(0)], max(steps, 2 * n_buffers), warmup)
+    # the same launches back to back (the shape of a per-tensor loop), and what an empty launch costs both ways
+    state["i"] = 0
+
+    def cold_dequant_next():
+        state["i"] = (state["i"] + 1) % n_buffers
+        dequant(state["i"])
+
+    q_b2b = _time_back_to_back(cold_quant, 8 * n_buffers)
+    d_b2b = _time_back_to_back(cold_dequant_next, 8 * n_buffers)
+    tl = wq_testlib.load()
+
+    def empty():
+        _lib.check(tl.wq_empty_launch(1024, 256, st), "empty launch")
+
+    _, empty_mean, _ = _time_step([empty], max(steps, 2 * n_buffers), warmup)
+    empty_b2b = _time_back_to_back(empty, 8 * n_buffers)
     qo, so = c_oracle.fp8_block_quant(w0, (128, 128), mode)
     assert torch.equal(qs[0].cpu(), qo) and torch.equal(ss[0].cpu().view(torch.int32), so.view(torch.int32))
     yo = c_oracle.fp8_block_dequant(qo, so, 128, 0)
@@ -253,10 +291,19 @@ def bench_cfg1(dev, steps, warmup, n_buffers=8):
            "quant_kernel_ms_warm": mean_w[0], "dequant_kernel_ms_warm": mean_w[1],
            "quant_hbm_frac_cold": algo / mean_c[0] / 1e6 / HBM_PEAK_GBS,
            "dequant_hbm_frac_cold": algo / mean_c[1] / 1e6 / HBM_PEAK_GBS,
+           "back_to_back": {"what": "64 launches in a row between one pair of events (a per-tensor loop), cold buffers; "
+                                    "microseconds per launch",
+                            "quant_us_cold": q_b2b, "dequant_us_cold": d_b2b,
+                            "quant_hbm_frac_cold": algo / q_b2b / 1e3 / HBM_PEAK_GBS,
+                            "dequant_hbm_frac_cold": algo / d_b2b / 1e3 / HBM_PEAK_GBS},
+           "empty_launch_us": {"what": "an empty kernel of 1024 workgroups x 256 lanes: the launch floor under both ways of timing",
+                               "event_pair_per_launch": empty_mean[0] * 1e3, "back_to_back": empty_b2b},
+           "mode": mode,
            "roundtrip_bf16_GBps_cold": 2 * M * N / (mean_c[0] + mean_c[1]) / 1e6,
            "roundtrip_bf16_GBps_warm": 2 * M * N / (mean_w[0] + mean_w[1]) / 1e6,
-           "note": "32 MiB tensors: launch latency and the tail of 1024 workgroups over 256 CUs are visible; warm runs "
-                   "are served from the last-level cache, so their rate is not an HBM figure"}
+           "note": "32 MiB tensors, one wave of workgroups: the *_kernel_ms_* figures bracket every launch with its own event "
+                   "pair and so contain the cost of the event packets (compare empty_launch_us); warm runs are served "
+                   "from the last-level cache, so their rate is not an HBM figure"}
     del ws, qs, ss, ys
     torch.cuda.empty_cache()
     return out
@@ -299,8 +346,7 @@ def bench_bucket(dev, steps, warmup, layers):
     from slime_amd import bucket as B
 
     cfg = {"quant_method": "fp8", "fmt": "e4m3", "activation_scheme": "dynamic", "weight_block_size": [128, 128]}
-    per_layer = []
-    for layer in range(layers):
+    def make_layer(layer):
         L, hf = f"module.module.decoder.layers.{layer}.", f"model.layers.{layer}."
         fc1 = _gen_bf16((128, 2 * 768, 2048), dev, outliers=True)
         fc2 = _gen_bf16((128, 2048, 768), dev, outliers=True)
@@ -316,7 +362,9 @@ def bench_bucket(dev, steps, warmup, layers):
             params.append((L + f"mlp.experts.linear_fc1.weight{e}",
                            [(hf + f"mlp.experts.{e}.gate_proj.weight", gate), (hf + f"mlp.experts.{e}.up_proj.weight", up)]))
             params.append((L + f"mlp.experts.linear_fc2.weight{e}", [(hf + f"mlp.experts.{e}.down_proj.weight", fc2[e])]))
-        per_layer.append(params)
+        return params
+
+    per_layer = [make_layer(layer) for layer in range(layers)]
     whole = [p for params in per_layer for p in params]
     n_tensors = sum(len(cv) for _, cv in whole)
     quantised = [(n, t) for _, cv in whole for n, t in cv if n.endswith("proj.weight")]
@@ -338,6 +386,31 @@ def bench_bucket(dev, steps, warmup, layers):
     torch.cuda.synchronize()
     first_ms = (time.perf_counter() - t0) * 1e3
     wall1, _, _ = _time_launches(one_bucket, steps, warmup)
+    # the call pattern of a sharded model: every sync presents the same names and shapes in freshly allocated tensors.
+    # A second copy of the state dict at other addresses, alternated with the first: every sync is a miss.
+    other = [p for layer in range(layers) for p in make_layer(layer)]
+    sets = [whole, other]
+    state["k"] = 0
+
+    def one_bucket_moved():
+        state["out"] = None
+        state["k"] ^= 1
+        state["out"] = conv.convert(sets[state["k"]], bucket_id="all")
+
+    resolves0 = conv.resolves
+    wall_moved, _, _ = _time_launches(one_bucket_moved, steps, warmup)
+    moved_resolves = conv.resolves - resolves0
+    named = dict(state["out"].reconstruct_tensors())
+    src = dict((n, t) for _, cv in sets[state["k"]] for n, t in cv)
+    for n in (quantised[0][0], quantised[-1][0]):
+        qo, so = c_oracle.fp8_block_quant(src[n].cpu().contiguous(), (128, 128), 1)
+        assert torch.equal(named[n].cpu().view(torch.uint8), qo), "moved bucket: FP8 parity failure"
+        assert torch.equal(named[n.replace(".weight", ".weight_scale_inv")].cpu().view(torch.int32), so.view(torch.int32))
+    assert moved_resolves == steps + warmup and conv.plan_builds == 1
+    del named, src, other, sets
+    state["out"] = None
+    torch.cuda.empty_cache()
+    one_bucket()                                  # back on the first set for the kernel timing below
     conv.time_kernels = True
     for _ in range(steps):
         one_bucket()
@@ -405,7 +478,11 @@ def bench_bucket(dev, steps, warmup, layers):
                        "into the one uint8 buffer + metadata a FlattenedTensorBucket consumer reads; fresh output buffer per sync",
            "tensors": n_tensors, "bf16_GB": 2 * elements / 1e9,
            "one_bucket": {"launches_per_sync": launches1, "ms_per_sync_kernels": ev1, "ms_per_sync_wall": wall1,
-                          "first_call_ms_table_build": first_ms, "hbm_frac": algo_bytes / ev1 / 1e6 / HBM_PEAK_GBS,
+                          "ms_per_sync_wall_inputs_reallocated_every_sync": wall_moved,
+                          "reallocated_note": "two copies of the state dict at different addresses alternate, so every sync "
+                                              "finds its inputs moved: one upload of 18 768 addresses and one resolve launch "
+                                              "over the per-item template, then the same conversion launch",
+                          "first_call_ms_layout_build": first_ms, "hbm_frac": algo_bytes / ev1 / 1e6 / HBM_PEAK_GBS,
                           "bf16_GBps": 2 * elements / ev1 / 1e6},
            "bucket_per_layer": {"launches_per_sync": launchesL, "ms_per_sync_kernels": evL, "ms_per_sync_wall": wallL,
                                 "hbm_frac": algo_bytes / evL / 1e6 / HBM_PEAK_GBS, "bf16_GBps": 2 * elements / evL / 1e6},
@@ -750,13 +827,14 @@ def bench_copy(dev, steps, warmup, nbytes=4 << 30):
     FETCH_SIZE / WRITE_SIZE counters, and the practical bandwidth ceiling of this box."""
     import torch
 
+    import wq_testlib
     from slime_amd import _lib
 
     src = torch.empty(nbytes, dtype=torch.uint8, device=dev).random_(0, 256)
     dst = torch.empty_like(src)
 
     def run():
-        _lib.check(_lib.load().wq_copy_bytes(src.data_ptr(), dst.data_ptr(), nbytes, _lib.stream_ptr(dev)), "copy")
+        _lib.check(wq_testlib.load().wq_copy_bytes(src.data_ptr(), dst.data_ptr(), nbytes, _lib.stream_ptr(dev)), "copy")
 
     wall_ms, ev_ms, ev_min = _time_launches(run, steps, warmup)
     assert torch.equal(src[:1 << 20], dst[:1 << 20]) and torch.equal(src[-(1 << 20):], dst[-(1 << 20):])
@@ -768,7 +846,7 @@ def bench_copy(dev, steps, warmup, nbytes=4 << 30):
         n_out = nbytes // ratio
 
         def fold():
-            _lib.check(_lib.load().wq_stream_fold_bytes(src.data_ptr(), dst.data_ptr(), n_out, ratio, _lib.stream_ptr(dev)), "fold")
+            _lib.check(wq_testlib.load().wq_stream_fold_bytes(src.data_ptr(), dst.data_ptr(), n_out, ratio, _lib.stream_ptr(dev)), "fold")
 
         _, f_ms, f_min = _time_launches(fold, steps, warmup)
         piece = {2: 16384, 4: 8192}[ratio]                   # bytes of output per work item

@@ -32,7 +32,7 @@
 extern "C" {
 #endif
 
-#define WQ_ABI_VERSION 17
+#define WQ_ABI_VERSION 18
 
 enum {
     WQ_OK = 0,
@@ -122,6 +122,19 @@ int wq_fp8_block_quant_tiles(const wq_fp8_quant_desc *tiles, int64_t n_tiles, in
 #define WQ_BUCKET_COPY_BYTES 32768
 int wq_fp8_bucket_convert(const wq_fp8_quant_desc *items, int64_t n_items, void *out_base, int bm, int bn, int mode,
                           void *stream);
+
+/* The bucket tables above hold the ADDRESS of every item's input, while the inputs of a weight-sync bucket are fresh
+ * tensors on every sync as soon as the model is sharded: all_gather_param fills torch.empty_like partitions and
+ * concatenates them (slime/backends/megatron_utils/update_weight/common.py:97,120) before
+ * HfWeightIteratorDirect._convert_to_hf_named_tensors (hf_weight_iterator_direct.py:50-67) sees them.  So that a moved
+ * bucket costs one small upload and one launch instead of a new table, the caller keeps the table as a TEMPLATE -
+ * `item_template`: DEVICE int64[n_items * words_per_item], the item descriptors of wq_fp8_bucket_convert (8 words),
+ * wq_int4_bucket_convert (4) or wq_int4_group_quant_pack_asym_items (5) with word 0 (x) holding the byte OFFSET of the
+ * item's input inside its tensor - plus `owner`: DEVICE int32[n_items], the index of that tensor, and passes the
+ * tensors' current addresses as `bases`: DEVICE int64[n_tensors].  Writes items[i] = item_template[i] with
+ * bases[owner[i]] added to word 0.  `items` must not alias `item_template`. */
+int wq_bucket_resolve_items(const int64_t *item_template, const int32_t *owner, const int64_t *bases,
+                            int64_t n_items, int words_per_item, int64_t *items, void *stream);
 
 /* wq_fp8_block_quant for bf16, fp16 or fp32 weights (`dtype` = WQ_DTYPE_*): the reference functions take any
  * floating dtype - block_fp8 computes amax and the 1e-12 floor in the weight dtype (the floor rounds to 0 in
@@ -437,35 +450,6 @@ typedef struct wq_xxh3_desc {
 } wq_xxh3_desc;
 int wq_xxh3_128_grouped(const wq_xxh3_desc *descs, const int64_t *item_start, int n_desc, int64_t total_items,
                         void *stream);
-
-/* ---------------------------------------------------------------------------------------------
- * Self-checks and calibration helpers (used by the test-suite and the benchmark, not by callers).
- *
- * wq_selftest_fp8_elem: for every bf16 amax a in [amax_lo, amax_hi) (bit patterns, finite) and every
- * bf16 x with |x| <= max(a, floor), compares the production element function (reciprocal + two FMA
- * refinement + hardware e4m3 conversion) with plain IEEE division + software RNE conversion.
- * Writes {mismatch count, first mismatching (a<<16|x)} to out[0..1] (DEVICE uint64[2], zeroed here).
- * wq_selftest_int4_elem: same for the INT4 element function q = rintf(x/scale).
- * wq_selftest_cvt_fp8: compares the hardware fp32->e4m3 conversion with the software one for the
- * fp32 bit patterns [lo, hi) whose magnitude is <= 464 or NaN. */
-int wq_selftest_fp8_elem(uint32_t amax_lo, uint32_t amax_hi, int mode, uint64_t *out, void *stream);
-int wq_selftest_int4_elem(uint32_t amax_lo, uint32_t amax_hi, uint64_t *out, void *stream);
-int wq_selftest_cvt_fp8(uint64_t lo, uint64_t hi, uint64_t *out, void *stream);
-/* wq_selftest_cvt_bf16: hardware fp32->bf16 conversion vs software RNE for the non-NaN fp32 bit
- * patterns in [lo, hi).  wq_selftest_decode_fp8: hardware e4m3fn->fp32 vs the format definition for all
- * 256 codes.  Same out[] convention. */
-int wq_selftest_cvt_bf16(uint64_t lo, uint64_t hi, uint64_t *out, void *stream);
-int wq_selftest_decode_fp8(uint64_t *out, void *stream);
-
-/* Plain 16-byte-per-lane copy of n_bytes (multiple of 16, 16-byte aligned): the known-traffic kernel
- * that hardware counters are scaled against. */
-int wq_copy_bytes(const void *src, void *dst, int64_t n_bytes, void *stream);
-
-/* A compute-free stream with `reads_per_write` (2 or 4) bytes read per byte written - the block-FP8 quantiser's and the
- * INT4 packer's read:write mix: dst[16 KiB piece i] = xor of src[pieces reads_per_write * i ...].  n_out_bytes a multiple
- * of 16384; src holds reads_per_write * n_out_bytes.  The benchmark runs it next to the quantisers to show what the
- * memory system gives that mix on the box at hand. */
-int wq_stream_fold_bytes(const void *src, void *dst, int64_t n_out_bytes, int reads_per_write, void *stream);
 
 #ifdef __cplusplus
 }

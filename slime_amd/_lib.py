@@ -15,7 +15,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libslime_amd_wq.so")
 
-ABI_VERSION = 17
+ABI_VERSION = 18
 
 # selectors (mirrors of the header's enums)
 DTYPE_BF16, DTYPE_F32, DTYPE_F16, DTYPE_F64 = 0, 1, 2, 3
@@ -38,6 +38,7 @@ SIGNATURES = {
     "wq_fp8_block_quant_tiles": [_vp, _i64, _int, _int, _int, _vp],
     "wq_fp8_bucket_convert": [_vp, _i64, _vp, _int, _int, _int, _vp],
     "wq_int4_bucket_convert": [_vp, _i64, _vp, _int, _vp],
+    "wq_bucket_resolve_items": [_vp, _vp, _vp, _i64, _int, _vp, _vp],
     "wq_fp8_block_quant_any": [_vp, _int, _i64, _i64, _i64, _i64, _vp, _i64, _vp, _int, _int, _int, _vp],
     "wq_fp8_row_quant": [_vp, _i64, _i64, _i64, _i64, _vp, _i64, _vp, _int, _vp],
     "wq_fp8_tensor_quant": [_vp, _i64, _i64, _i64, _i64, _vp, _i64, _vp, _vp, _int, _vp],
@@ -68,13 +69,6 @@ SIGNATURES = {
     "wq_delta_xor_noalloc": [_vp, _vp, _vp, _i64, _int, _vp, _vp],
     "wq_delta_xor_grouped": [_vp, _vp, _int, _i64, _int, _int, _int, _vp],
     "wq_delta_xor_xxh3": [_vp, _vp, _vp, _i64, _int, _vp, _vp, _vp, _vp, _vp],
-    "wq_selftest_fp8_elem": [_u32, _u32, _int, _vp, _vp],
-    "wq_selftest_int4_elem": [_u32, _u32, _vp, _vp],
-    "wq_selftest_cvt_fp8": [_u64, _u64, _vp, _vp],
-    "wq_selftest_cvt_bf16": [_u64, _u64, _vp, _vp],
-    "wq_selftest_decode_fp8": [_vp, _vp],
-    "wq_copy_bytes": [_vp, _vp, _i64, _vp],
-    "wq_stream_fold_bytes": [_vp, _vp, _i64, _int, _vp],
 }
 
 _lib = None

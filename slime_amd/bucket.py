@@ -11,10 +11,17 @@ a tile / a run of groups straight into its place in the flat buffer or copy a pi
 result has the layout the bucket consumer reads: one uint8 tensor plus ``(name, shape, dtype, start_idx, end_idx, numel)``
 per tensor, names in the order the per-parameter loop produces them, tensors packed back to back.
 
-The per-item table is built once per bucket *identity* (names, shapes, strides and addresses of the inputs) and cached:
-a weight sync that presents the same tensors again does no host-side table work.  Destinations in the table are offsets,
-so every call can write into a fresh buffer (the reference warns against reusing the IPC-facing one,
+The per-item table is built once per bucket *layout* (names, shapes, strides and dtypes) as a template that holds no
+address: inputs appear in it as (tensor index, byte offset).  On every sync the addresses of the bucket's tensors are
+compared with the ones the resolved table was made for; when any moved - which is every sync once the model is sharded,
+because gathered parameters are fresh allocations (update_weight/common.py:97,120) - the addresses are uploaded (8 bytes
+per tensor) and one small launch adds them to the template (``wq_bucket_resolve_items``).  Destinations in the table are
+offsets, so every call can write into a fresh buffer (the reference warns against reusing the IPC-facing one,
 update_weight_from_tensor.py:39-43) or into ``out=``.
+
+Tensors are packed back to back exactly as ``FlattenedTensorBucket`` packs them.  A bucket in which that puts a tensor at
+an offset that is not a multiple of its element size (an odd number of one-byte elements ahead of a wider tensor) is
+converted by the per-parameter loop and concatenated with ``torch.cat``, as the reference does.
 """
 
 from __future__ import annotations
@@ -24,6 +31,7 @@ import json
 from collections import OrderedDict
 from typing import Sequence
 
+import numpy as np
 import torch
 
 from . import _lib
@@ -83,9 +91,15 @@ def flatten_named_tensors(named_tensors) -> FlattenedBucket:
     return FlattenedBucket(torch.cat(parts, dim=0), meta, launches=len(parts) + 1)
 
 
-class _Plan:
-    __slots__ = ("kind", "items", "n_items", "total_bytes", "metadata", "keepalive", "late_copies", "group", "block", "device",
-                 "zero_bytes", "zp_rows", "zp_start", "zp_words", "n_zp")
+class _Layout:
+    """Everything about a bucket that does not depend on where its inputs live this sync."""
+    __slots__ = ("kind", "block", "group", "device", "metadata", "total_bytes", "n_tensors", "n_items", "width",
+                 "template", "owner", "items", "bases", "slot_src", "align", "const_base", "resolved_ptrs", "staging",
+                 "stage_events", "stage_next", "keepalive", "late_copies", "zero_bytes", "zp_rows", "zp_start",
+                 "zp_words", "n_zp", "fallback")
+
+
+_STAGING_DEPTH = 4
 
 
 class BucketConverter:
@@ -96,6 +110,9 @@ class BucketConverter:
     (FP8: not 2-D bf16 on the GPU; INT4: not contiguous 16-byte aligned bf16 with 32 / 64 / 128 groups; per-tensor FP8
     configurations) go through the per-tensor functions first and are copied in by the same launch, so
     the result is always what the per-parameter loop gives.
+
+    Calls of one converter must be ordered on one stream (or by the caller): the resolved work-item table and the
+    address upload buffer of a layout are reused from call to call.
     """
 
     def __init__(self, args=None, quantization_config=None, transform_ue8m0: bool = True, max_cached_plans: int = 256):
@@ -103,9 +120,10 @@ class BucketConverter:
         self.config = quantization_config
         self.transform_ue8m0 = transform_ue8m0
         self._config_key = json.dumps(quantization_config, sort_keys=True, default=str)
-        self._plans: OrderedDict = OrderedDict()
+        self._layouts: OrderedDict = OrderedDict()
         self._max = int(max_cached_plans)
-        self.plan_builds = 0
+        self.plan_builds = 0            # layouts built on the host (names, shapes, offsets, the per-item template)
+        self.resolves = 0               # syncs whose inputs had moved: one address upload + one resolve launch each
         self.time_kernels = False       # when set, convert() brackets its launch with events (kernel_ms())
         self.kernel_events = []
         method = None if quantization_config is None else quantization_config["quant_method"]
@@ -150,13 +168,14 @@ class BucketConverter:
             return ops
         return [("pass", n, t, ci) for ci, (n, t) in enumerate(converted)]
 
-    # ------------------------------------------------------------------ plan
+    # ------------------------------------------------------------------ layout
 
     @staticmethod
     def _key(params):
-        return tuple((mn, tuple((n, t.data_ptr(), tuple(t.shape), t.stride(), t.dtype) for n, t in conv)) for mn, conv in params)
+        """Identity of a bucket's layout: everything but the addresses."""
+        return tuple((mn, tuple((n, tuple(t.shape), t.stride(), t.dtype, t.device) for n, t in conv)) for mn, conv in params)
 
-    def _build(self, params) -> _Plan:
+    def _build(self, params) -> _Layout:
         self.plan_builds += 1
         device = None
         for _, conv in params:
@@ -169,21 +188,39 @@ class BucketConverter:
         if device is None:
             raise RuntimeError("BucketConverter: the bucket holds no GPU tensor; there is no CPU path")
         fp8 = self._method != "compressed-tensors"          # pass-through-only buckets use the FP8 launch's copy items
-        plan = _Plan()
+        plan = _Layout()
         asym = not fp8 and not self._sym
         plan.kind = "fp8" if fp8 else ("int4_asym" if asym else "int4")
         plan.block = tuple(int(b) for b in self._block) if (self._method == "fp8" and self._block is not None) else (128, 128)
         plan.group = int(self._group) if self._method == "compressed-tensors" else 128
+        plan.fallback = False
         bm, bn = plan.block
+
+        flat_index, k = {}, 0                           # (parameter, converted tensor) -> position among all tensors
+        for pi, (_, conv) in enumerate(params):
+            for ci in range(len(conv)):
+                flat_index[(pi, ci)] = k
+                k += 1
+        plan.n_tensors = k
+        slot_src, align = [], []                        # per input the launch reads: its position, its alignment mask
+
+        def slot(pi, ci, mask):
+            slot_src.append(flat_index[(pi, ci)])
+            align.append(mask)
+            return len(slot_src) - 1
 
         meta, off = [], 0
         quant_rows, copy_rows, late = [], [], []       # table rows per tensor; late = results only known at run time
         shape_rows, zp_entries, zero_off = [], [], 0
 
         def place(name, shape, dtype):
+            """The next tensor of the flat buffer, back to back as FlattenedTensorBucket packs them."""
             nonlocal off
             esz = torch.empty((), dtype=dtype).element_size()
-            off = -(-off // esz) * esz                  # natural alignment; real weight shapes never need padding
+            if off % esz:
+                # an odd-sized tensor ahead of a wider one: neither the kernels nor a consumer's .view(dtype) can
+                # address the wider tensor at this offset, and padding would not be the reference's layout
+                plan.fallback = True
             nbytes = esz
             for d in shape:
                 nbytes *= int(d)
@@ -197,7 +234,7 @@ class BucketConverter:
             if not nbytes:
                 return
             if t.is_cuda and t.device == device and t.is_contiguous():
-                copy_rows.append((len(meta) - 1, t.data_ptr(), start, nbytes))
+                copy_rows.append((len(meta) - 1, slot(pi, ci, 0), start, nbytes))
             else:
                 late.append((len(meta) - 1, pi, ci, None))
 
@@ -215,7 +252,7 @@ class BucketConverter:
                     M, N = t.shape
                     y0, _ = place(n, (M, N), FP8_DTYPE)
                     s0, _ = place(n.replace(".weight", ".weight_scale_inv"), (ceildiv(M, bm), ceildiv(N, bn)), torch.float32)
-                    quant_rows.append((len(meta) - 2, [t.data_ptr(), y0, s0, M, N, t.stride(0), t.stride(1), N]))
+                    quant_rows.append((len(meta) - 2, slot(pi, ci, 0), [0, y0, s0, M, N, t.stride(0), t.stride(1), N]))
                 else:
                     M, N = t.shape
                     if asym:        # zero points first, as the per-parameter loop emits them
@@ -226,25 +263,40 @@ class BucketConverter:
                     s0, _ = place(n.replace(".weight", ".weight_scale"), (M, N // plan.group), torch.bfloat16)
                     h0, _ = place(n.replace(".weight", ".weight_shape"), (2,), torch.int32)
                     if asym:
-                        quant_rows.append((len(meta) - 4, [t.data_ptr(), p0, s0, zero_off, M * N // plan.group]))
+                        quant_rows.append((len(meta) - 4, slot(pi, ci, 15), [0, p0, s0, zero_off, M * N // plan.group]))
                         zero_off += (2 * M * G + 15) // 16 * 16
                     else:
-                        quant_rows.append((len(meta) - 3, [t.data_ptr(), p0, s0, M * N // plan.group]))
+                        quant_rows.append((len(meta) - 3, slot(pi, ci, 15), [0, p0, s0, M * N // plan.group]))
                     shape_rows.append((len(meta) - 1, h0, (M, N)))
 
+        plan.total_bytes = off
+        plan.metadata = meta
+        plan.late_copies = late
+        plan.device = device
         plan.keepalive = []
+        plan.resolved_ptrs = None
+        plan.n_items, plan.template, plan.owner, plan.items = 0, None, None, None
+        plan.zero_bytes, plan.n_zp = zero_off, len(zp_entries)
+        if plan.fallback:
+            return plan
+
+        const_slot = len(slot_src)                      # one more base: the table of weight_shape values the layout owns
+        plan.const_base = 0
         if shape_rows:
             shapes = torch.tensor([sh for _, _, sh in shape_rows], dtype=torch.int32).to(device)
             plan.keepalive.append(shapes)
+            plan.const_base = shapes.data_ptr()
             for k, (mi, h0, _) in enumerate(shape_rows):
-                copy_rows.append((mi, shapes.data_ptr() + 8 * k, h0, 8))
+                copy_rows.append((mi, const_slot, h0, 8, 8 * k))
 
-        # ---- one table row per work item, in bucket order (ordered by the metadata index of the item's first output)
+        # ---- one template row per work item, in bucket order (ordered by the metadata index of the item's first
+        # output); word 0 is the item's byte offset inside its input tensor, `owner` says which tensor that is
         width = 8 if fp8 else (5 if asym else 4)
-        blocks, order = [], []
+        blocks, order, owners = [], [], []
         if quant_rows:
-            first = torch.tensor([mi for mi, _ in quant_rows], dtype=torch.int64)
-            rows = [r for _, r in quant_rows]
+            first = torch.tensor([mi for mi, _, _ in quant_rows], dtype=torch.int64)
+            row_slot = torch.tensor([s for _, s, _ in quant_rows], dtype=torch.int64)
+            rows = [r for _, _, r in quant_rows]
             if asym:
                 # x, packed, scale and the zero scratch advance with the item; n_groups is what is left of the tensor
                 full = torch.tensor(rows, dtype=torch.int64)
@@ -254,9 +306,10 @@ class BucketConverter:
             else:
                 table, owner, local = tile_table(rows, bm, bn) if fp8 else item_table(rows, plan.group)
             blocks.append(table)
+            owners.append(row_slot[owner])
             order.append(first[owner] * (1 << 32) + local)
         if copy_rows:
-            c = torch.tensor([(mi, src, dst, nb) for mi, src, dst, nb in copy_rows], dtype=torch.int64)
+            c = torch.tensor([(r + (0,))[:5] for r in copy_rows], dtype=torch.int64)     # mi, slot, dst, bytes, src offset
             counts = (c[:, 3] + _COPY - 1) // _COPY
             owner = torch.repeat_interleave(torch.arange(len(copy_rows)), counts)
             start = torch.cumsum(counts, 0) - counts
@@ -264,59 +317,98 @@ class BucketConverter:
             d = c[owner]
             nb = torch.clamp(d[:, 3] - local * _COPY, max=_COPY)
             zero = torch.zeros_like(nb)
+            src, dst = d[:, 4] + local * _COPY, d[:, 2] + local * _COPY
             if fp8:
-                blocks.append(torch.stack([d[:, 1] + local * _COPY, d[:, 2] + local * _COPY, zero, nb, zero,
-                                           torch.full_like(nb, _lib.BUCKET_COPY_MARK), zero, zero], dim=1))
+                blocks.append(torch.stack([src, dst, zero, nb, zero, torch.full_like(nb, _lib.BUCKET_COPY_MARK), zero, zero], dim=1))
             elif asym:
-                blocks.append(torch.stack([d[:, 1] + local * _COPY, d[:, 2] + local * _COPY, zero, zero, -nb], dim=1))
+                blocks.append(torch.stack([src, dst, zero, zero, -nb], dim=1))
             else:
-                blocks.append(torch.stack([d[:, 1] + local * _COPY, d[:, 2] + local * _COPY, zero, -nb], dim=1))
+                blocks.append(torch.stack([src, dst, zero, -nb], dim=1))
+            owners.append(d[:, 1])
             order.append(d[:, 0] * (1 << 32) + local)
         if blocks:
-            table = torch.cat(blocks, dim=0)
-            table = table[torch.argsort(torch.cat(order), stable=True)]
-            plan.items = table.contiguous().to(device)
-            plan.n_items = table.shape[0]
+            perm = torch.argsort(torch.cat(order), stable=True)
+            table = torch.cat(blocks, dim=0)[perm].contiguous()
             assert table.shape[1] == width
-        else:
-            plan.items, plan.n_items = None, 0
-        plan.zero_bytes, plan.n_zp = zero_off, len(zp_entries)
+            plan.n_items, plan.width = table.shape[0], width
+            plan.template = table.to(device)
+            plan.owner = torch.cat(owners)[perm].to(torch.int32).contiguous().to(device)
+            plan.items = torch.empty_like(plan.template)
+            plan.slot_src = np.asarray(slot_src, dtype=np.int64)
+            plan.align = np.asarray(align, dtype=np.int64)
+            n_bases = const_slot + 1
+            plan.bases = torch.empty(n_bases, dtype=torch.int64, device=device)
+            plan.staging = [torch.empty(n_bases, dtype=torch.int64).pin_memory() for _ in range(_STAGING_DEPTH)]
+            plan.stage_events, plan.stage_next = [None] * _STAGING_DEPTH, 0
         if zp_entries:
             zrows, zstart, plan.zp_words = zero_point_rows(zp_entries)
             plan.zp_rows, plan.zp_start = zrows.to(device), zstart.to(device)
-        plan.total_bytes = off
-        plan.metadata = meta
-        plan.late_copies = late
-        plan.device = device
-        # The table holds the addresses of the inputs, not references: a cached plan is used again only when a later
-        # bucket presents tensors with the same names, shapes, strides AND addresses, and it keeps no weight alive.
+        # The layout holds no address of an input and no reference to one: it serves every later bucket with the same
+        # names, shapes, strides and dtypes wherever its tensors live, and it keeps no weight alive.
         return plan
+
+    def _resolve(self, plan: _Layout, ptrs) -> bool:
+        """The bucket's tensors are not where the resolved table says: upload their addresses (8 bytes each, through
+        pinned staging) and let the GPU add them to the template.  -> False when an input the kernels need aligned
+        is not (the cached routing does not apply to these tensors)."""
+        arr = np.asarray(ptrs, dtype=np.int64)
+        bases = arr[plan.slot_src]
+        if np.any(bases & plan.align):
+            return False
+        k = plan.stage_next
+        plan.stage_next = (k + 1) % _STAGING_DEPTH
+        if plan.stage_events[k] is not None:
+            plan.stage_events[k].synchronize()          # the upload that last used this staging buffer has finished
+        host = plan.staging[k]
+        h = host.numpy()
+        h[:-1] = bases
+        h[-1] = plan.const_base
+        stream = torch.cuda.current_stream(plan.device)
+        with torch.cuda.device(plan.device):
+            plan.bases.copy_(host, non_blocking=True)
+            ev = torch.cuda.Event()
+            ev.record(stream)
+            plan.stage_events[k] = ev
+            rc = _lib.load().wq_bucket_resolve_items(plan.template.data_ptr(), plan.owner.data_ptr(), plan.bases.data_ptr(),
+                                                     plan.n_items, plan.width, plan.items.data_ptr(), stream.cuda_stream)
+        _lib.check(rc, "BucketConverter: resolving the work-item table")
+        plan.resolved_ptrs = ptrs
+        self.resolves += 1
+        return True
 
     # ------------------------------------------------------------------ run
 
     def convert(self, params, out: torch.Tensor | None = None, bucket_id=None) -> FlattenedBucket:
         """``bucket_id`` (any hashable, e.g. the bucket's index in the weight-sync loop) is a promise that every call
-        with this id presents the same names, shapes, strides and dtypes; then only the addresses are compared with
-        the cached table's (0.2 us per tensor instead of 4 us for the full identity), and a bucket whose tensors
-        moved gets a new table."""
+        with this id presents the same names, shapes, strides and dtypes; the layout is then found by the id alone
+        (without it, by the full identity of the bucket: about 3 us per tensor).  Where the tensors live may change
+        from call to call: a moved bucket costs one upload of its addresses and one small launch."""
+        params = [(mn, conv if type(conv) is list else list(conv)) for mn, conv in params]
+        ptrs = [t.data_ptr() for _, conv in params for _, t in conv]
+        if not ptrs:
+            return flatten_named_tensors([])
         if bucket_id is not None:
-            key = ("id", bucket_id, tuple([t.data_ptr() for _, conv in params for _, t in conv]), ue8m0_requant_enabled())
-            if not key[2]:
-                return flatten_named_tensors([])
+            key = ("id", bucket_id, ue8m0_requant_enabled())
         else:
-            params = [(mn, list(conv)) for mn, conv in params]
-            if not any(conv for _, conv in params):
-                return flatten_named_tensors([])
             key = (self._key(params), self._config_key, self.transform_ue8m0, ue8m0_requant_enabled())
-        plan = self._plans.get(key)
-        if plan is None:
-            params = [(mn, list(conv)) for mn, conv in params]
-            plan = self._build(params)
-            self._plans[key] = plan
-            while len(self._plans) > self._max:
-                self._plans.popitem(last=False)
-        else:
-            self._plans.move_to_end(key)
+        plan = self._layouts.get(key)
+        if plan is not None and plan.n_tensors != len(ptrs):
+            plan = None                                  # not the bucket this id stood for
+        for _ in range(2):
+            if plan is None:
+                plan = self._build(params)
+                self._layouts[key] = plan
+                while len(self._layouts) > self._max:
+                    self._layouts.popitem(last=False)
+            else:
+                self._layouts.move_to_end(key)
+            if plan.fallback:
+                # back-to-back packing puts a tensor at an offset that is not a multiple of its element size:
+                # the per-parameter loop and a plain concatenation, exactly as the reference builds the buffer
+                return flatten_named_tensors(per_param_loop(self.args, params, self.config, self.transform_ue8m0))
+            if not plan.n_items or ptrs == plan.resolved_ptrs or self._resolve(plan, ptrs):
+                break
+            plan = None                                  # an input lost the alignment the cached routing relied on
         device = plan.device
         if out is None:
             out = torch.empty(plan.total_bytes, dtype=torch.uint8, device=device)
@@ -368,7 +460,7 @@ class BucketConverter:
         for mi, pi, ci, out_name in plan.late_copies:
             m = plan.metadata[mi]
             mn, conv = params[pi]
-            name, t = (conv if isinstance(conv, (list, tuple)) else list(conv))[ci]
+            name, t = conv[ci]
             if out_name is None:
                 src = t
             else:

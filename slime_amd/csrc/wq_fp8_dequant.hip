@@ -26,6 +26,10 @@ constexpr int kSteps = kSegsPerWg / 4;           // loads in flight per lane
 constexpr int kDeqItemsPerXcdRun = 32;
 constexpr int kDeqWindow = 4;                          // steps whose loads are in flight (kSteps = all)
 constexpr unsigned kDeqOccupancyPadBytes = 27 * 1024;  // unused dynamic LDS: at most 5 workgroups per CU
+// A launch of at most this many work items ([4096, 4096] is 2048) fits the chip at full occupancy in one wave of
+// workgroups; capped at 5 per CU it would run as one full wave and a partial one.  Such launches run uncapped
+// ([4096, 4096], launches back to back: 12.3 -> 11.0 us; larger launches do not change).
+constexpr int64_t kDeqSmallLaunchItems = 2048;
 static_assert(kSeg == 512 && kSegsPerWg % 4 == 0, "a segment is 64 lanes x 8 codes; four waves per workgroup");
 
 struct DeqArgs {
@@ -207,6 +211,7 @@ template <int GROUPED>
 static int launch_deq(const DeqArgs& a, int64_t work, int mode, int out_dtype, hipStream_t st)
 {
     const dim3 g = grid_for_items(work);
+    const unsigned kDeqOccupancyPadBytes = work <= kDeqSmallLaunchItems ? 0u : wq::kDeqOccupancyPadBytes;
     if (mode == WQ_DEQ_MODE_F32SCALE) {
         if (out_dtype == WQ_DTYPE_BF16) fp8_block_dequant_kernel<WQ_DEQ_MODE_F32SCALE, GROUPED, WQ_DTYPE_BF16><<<g, 256, kDeqOccupancyPadBytes, st>>>(a, work);
         else if (out_dtype == WQ_DTYPE_F16) fp8_block_dequant_kernel<WQ_DEQ_MODE_F32SCALE, GROUPED, WQ_DTYPE_F16><<<g, 256, kDeqOccupancyPadBytes, st>>>(a, work);

@@ -38,6 +38,15 @@ constexpr unsigned kOccupancyPadBytes = 36 * 1024;  // unused dynamic LDS: caps 
 // workgroups per CU (84 %): fewer bytes in flight per CU suit the memory system, and the window gets part of that while
 // four workgroups keep the arithmetic overlapped.
 constexpr int kTileWindow = 2;
+// Launches of at most kSmallLaunchTiles tiles put fewer than two workgroups on a CU: nothing else is there to overlap a
+// workgroup's load latency, so these issue all eight loads of a lane at once and run without the residency pad
+// ([2048, 2048], 256 tiles, launches back to back: 6.0 -> 5.1 us).  From one workgroup per CU slot upwards the windowed
+// form is as fast or faster ([4096, 4096], 1024 tiles: 10.7 us windowed, 11.2 us all at once; 2048 tiles: 19.2 - 20.2 us in
+// every combination of window and pad), and a launch of that size is within 1.5 us of launch gap (1.6 us between two
+// empty kernels on one stream) + the time its bytes take at the rate the plain copy reaches.
+constexpr int64_t kSmallLaunchTiles = 512;
+constexpr int kSmallTileWindow = 8;
+constexpr unsigned kSmallOccupancyPadBytes = 0;
 constexpr int kRowSlots = kTileThreads / 16;   // rows covered by one load step of the workgroup
 constexpr int kTileLoads = 128 / kRowSlots;    // 16-byte loads per lane
 constexpr int kTileWaves = kTileThreads / 64;
@@ -59,7 +68,7 @@ __device__ __forceinline__ bool desc_vector_ok(const wq_fp8_quant_desc& d)
            d.sy_m >= 0 && d.sy_m < (1 << 22);
 }
 
-template <int MODE>
+template <int MODE, int WINDOW>
 __device__ __forceinline__ void quant_tile_vec128(const wq_fp8_quant_desc& d, int64_t tm, int64_t tn, int kt,
                                                   uint32_t* lds)
 {
@@ -80,15 +89,17 @@ __device__ __forceinline__ void quant_tile_vec128(const wq_fp8_quant_desc& d, in
     uint32_t m = 0;
     if (full) {
 #pragma unroll
-        for (int i = 0; i < kTileWindow && i < kTileLoads; ++i) v[i] = ldg_nt<u32x4>(xt + (xoff + i * xstep));
+        for (int i = 0; i < WINDOW && i < kTileLoads; ++i) v[i] = ldg_nt<u32x4>(xt + (xoff + i * xstep));
 #pragma unroll
         for (int i = 0; i < kTileLoads; ++i) {
             m = pk_absmax(m, v[i].x);
             m = pk_absmax(m, v[i].y);
             m = pk_absmax(m, v[i].z);
             m = pk_absmax(m, v[i].w);
-            __builtin_amdgcn_sched_barrier(0);      // keep the next load behind this step's use of its data
-            if (i + kTileWindow < kTileLoads) v[i + kTileWindow] = ldg_nt<u32x4>(xt + (xoff + (i + kTileWindow) * xstep));
+            if (WINDOW < kTileLoads) {
+                __builtin_amdgcn_sched_barrier(0);      // keep the next load behind this step's use of its data
+                if (i + WINDOW < kTileLoads) v[i + WINDOW] = ldg_nt<u32x4>(xt + (xoff + (i + WINDOW) * xstep));
+            }
         }
     } else {
         // Edge tile: every lane loads from a valid address - its row and piece clamped into the tile - and the lanes
@@ -182,7 +193,8 @@ __device__ __forceinline__ void quant_tile_generic(const wq_fp8_quant_desc& d, i
 
 // GROUPED: 0 = one tensor in the kernel arguments, 1 = descriptor array + prefix sums (the owner of a tile is
 // searched), 2 = one descriptor per tile, already moved to the tile's origin (a single scalar load, no search)
-template <int MODE, int GROUPED>
+// SMALL: the single-wave form (see kSmallLaunchTiles)
+template <int MODE, int GROUPED, bool SMALL = false>
 __global__ __launch_bounds__(kTileThreads) void fp8_block_quant_kernel(const Fp8QuantArgs a, const int64_t total_tiles)
 {
     __shared__ __attribute__((aligned(16))) uint32_t lds[kRowSlots];
@@ -213,7 +225,7 @@ __global__ __launch_bounds__(kTileThreads) void fp8_block_quant_kernel(const Fp8
     const int kt = GROUPED == 2 ? 1 : (int)((d.N + a.bn - 1) / a.bn);
     const int64_t tm = local / kt, tn = local - tm * kt;
     if (a.bm == 128 && a.bn == 128 && desc_vector_ok(d))
-        quant_tile_vec128<MODE>(d, tm, tn, kt, lds);
+        quant_tile_vec128<MODE, SMALL ? kSmallTileWindow : kTileWindow>(d, tm, tn, kt, lds);
     else
         quant_tile_generic<MODE>(d, tm, tn, kt, a.bm, a.bn, lds);
 }
@@ -652,18 +664,23 @@ static bool known_mode(int mode)
            mode == WQ_FP8_MODE_UE8M0;
 }
 
+template <int MODE, int GROUPED>
+static void launch_block_quant_mode(const Fp8QuantArgs& a, int64_t tiles, hipStream_t st)
+{
+    const dim3 g = grid_for_items(tiles);
+    if (tiles <= kSmallLaunchTiles)
+        fp8_block_quant_kernel<MODE, GROUPED, true><<<g, kTileThreads, kSmallOccupancyPadBytes, st>>>(a, tiles);
+    else
+        fp8_block_quant_kernel<MODE, GROUPED, false><<<g, kTileThreads, kOccupancyPadBytes, st>>>(a, tiles);
+}
+
 template <int GROUPED>
 static void launch_block_quant(const Fp8QuantArgs& a, int64_t tiles, int mode, hipStream_t st)
 {
-    const dim3 g = grid_for_items(tiles);
-    if (mode == WQ_FP8_MODE_TORCH)
-        fp8_block_quant_kernel<WQ_FP8_MODE_TORCH, GROUPED><<<g, kTileThreads, kOccupancyPadBytes, st>>>(a, tiles);
-    else if (mode == WQ_FP8_MODE_TORCH_DEVICE)
-        fp8_block_quant_kernel<WQ_FP8_MODE_TORCH_DEVICE, GROUPED><<<g, kTileThreads, kOccupancyPadBytes, st>>>(a, tiles);
-    else if (mode == WQ_FP8_MODE_UE8M0)
-        fp8_block_quant_kernel<WQ_FP8_MODE_UE8M0, GROUPED><<<g, kTileThreads, kOccupancyPadBytes, st>>>(a, tiles);
-    else
-        fp8_block_quant_kernel<WQ_FP8_MODE_TRITON, GROUPED><<<g, kTileThreads, kOccupancyPadBytes, st>>>(a, tiles);
+    if (mode == WQ_FP8_MODE_TORCH) launch_block_quant_mode<WQ_FP8_MODE_TORCH, GROUPED>(a, tiles, st);
+    else if (mode == WQ_FP8_MODE_TORCH_DEVICE) launch_block_quant_mode<WQ_FP8_MODE_TORCH_DEVICE, GROUPED>(a, tiles, st);
+    else if (mode == WQ_FP8_MODE_UE8M0) launch_block_quant_mode<WQ_FP8_MODE_UE8M0, GROUPED>(a, tiles, st);
+    else launch_block_quant_mode<WQ_FP8_MODE_TRITON, GROUPED>(a, tiles, st);
 }
 
 static int check_desc_host(const void* x, int64_t M, int64_t N, const void* y, const float* s, int bm, int bn, int mode)

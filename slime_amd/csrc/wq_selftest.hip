@@ -1,5 +1,7 @@
-// On-device self-checks of the element functions and of the hardware number-format conversions the
-// production kernels rely on, plus the plain copy kernel used to calibrate hardware counters.
+// libslime_amd_wq_test.so: on-device self-checks of the element functions and of the hardware number-format
+// conversions the production kernels rely on, plus the compute-free kernels (copy, 2:1 / 4:1 streams, an empty launch)
+// that hardware counters and achieved bandwidths are scaled against.  Instruments of the tests and the benchmark; the
+// product library holds none of this.
 //
 // The production element functions replace the reference's per-element IEEE division by a
 // reciprocal-and-refine sequence and its software casts by gfx950 conversion instructions.  These
@@ -7,6 +9,7 @@
 // software round-to-nearest-even), so that the shortcut is licensed by exhaustion, not by argument.
 
 #include "wq_common.h"
+#include "../../include/slime_amd_wq_test.h"
 
 namespace wq {
 
@@ -176,27 +179,13 @@ __global__ __launch_bounds__(256) void fold_kernel(const u32x4* __restrict__ src
     }
 }
 
+__global__ void empty_kernel() {}
+
 }  // namespace wq
 
 using namespace wq;
 
-WQ_EXPORT int wq_abi_version(void) { return WQ_ABI_VERSION; }
-
-WQ_EXPORT const char* wq_error_string(int code)
-{
-    switch (code) {
-    case WQ_OK: return "success";
-    case WQ_ERR_NULL: return "a required pointer is NULL";
-    case WQ_ERR_SHAPE: return "invalid shape, block or group size";
-    case WQ_ERR_MODE: return "unknown mode or dtype selector";
-    case WQ_ERR_UNSUPPORTED: return "configuration not supported by this library";
-    case WQ_ERR_ALIGN: return "pointer or stride alignment requirement violated";
-    case WQ_ERR_TOO_LARGE: return "count exceeds the limits of this entry point";
-    default: break;
-    }
-    if (code > 0) return hipGetErrorString((hipError_t)code);
-    return "unknown error";
-}
+WQ_EXPORT int wq_test_abi_version(void) { return WQ_ABI_VERSION; }
 
 WQ_EXPORT int wq_selftest_fp8_elem(uint32_t amax_lo, uint32_t amax_hi, int mode, uint64_t* out, void* stream)
 {
@@ -295,6 +284,14 @@ WQ_EXPORT int wq_stream_fold_bytes(const void* src, void* dst, int64_t n_out_byt
         const int64_t items = n_out_bytes / (kFoldSteps4 * 4096);
         fold_kernel<4, kFoldSteps4><<<grid_for_items(items), 256, kFoldPadBytes4, st>>>((const u32x4*)src, (u32x4*)dst, items);
     }
+    WQ_LAUNCH_CHECK();
+    return WQ_OK;
+}
+
+WQ_EXPORT int wq_empty_launch(int64_t workgroups, int threads, void* stream)
+{
+    if (workgroups <= 0 || workgroups > (1ll << 30) || threads <= 0 || threads > 1024) return WQ_ERR_SHAPE;
+    empty_kernel<<<grid_for_items(workgroups), threads, 0, (hipStream_t)stream>>>();
     WQ_LAUNCH_CHECK();
     return WQ_OK;
 }

@@ -7,16 +7,25 @@ import re
 
 import pytest
 
+import wq_testlib
 from slime_amd import _lib
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 HEADER = os.path.join(ROOT, "include", "slime_amd_wq.h")
+TEST_HEADER = os.path.join(ROOT, "include", "slime_amd_wq_test.h")
 
 
-def _declared_symbols():
-    text = open(HEADER).read()
+def _declared_symbols(header=HEADER):
+    text = open(header).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(wq_[a-z0-9_]+)\s*\(", text)))
+
+
+def _exported_symbols(path):
+    import subprocess
+
+    out = subprocess.check_output(["nm", "-D", "--defined-only", path], text=True)
+    return sorted(ln.split()[-1] for ln in out.splitlines() if " T " in ln and ln.split()[-1].startswith("wq_"))
 
 
 def test_header_symbols_are_exported_and_bound():
@@ -27,6 +36,18 @@ def test_header_symbols_are_exported_and_bound():
         assert hasattr(lib, n), f"{n} declared in the header but not exported"
         assert n in _lib.SIGNATURES, f"{n} has no ctypes signature"
     assert sorted(_lib.SIGNATURES) == names
+    assert _exported_symbols(_lib.LIB_PATH) == names        # nothing exported that the header does not declare
+
+
+def test_product_library_holds_no_instruments():
+    """Self-checks and calibration kernels live in a library of their own: the product header declares only entry points
+    that replace a reference interface (plus the no-allocation variant), and the two libraries share no symbol."""
+    product, instruments = _declared_symbols(), _declared_symbols(TEST_HEADER)
+    assert not [n for n in product if "selftest" in n or n in ("wq_copy_bytes", "wq_stream_fold_bytes", "wq_empty_launch")]
+    assert not set(product) & set(instruments)
+    assert sorted(wq_testlib.SIGNATURES) == instruments == _exported_symbols(wq_testlib.LIB_PATH)
+    lib = wq_testlib.load()
+    assert lib.wq_test_abi_version() == _lib.ABI_VERSION
 
 
 def test_abi_version_and_error_strings():
@@ -79,8 +100,9 @@ def test_argument_validation_without_launch():
     assert lib.wq_int4_fake_quant_ste(None, None, 4, 96, 96, 0, None) == U
     assert lib.wq_int4_fake_quant_ste(None, None, 4, 128, 128, 5, None) == M_
     assert lib.wq_int4_fake_quant_ste(None, None, 4, 128, 128, 1, None) == N_
-    assert lib.wq_copy_bytes(None, None, 24, None) == S
-    assert lib.wq_selftest_fp8_elem(0, 0x9000, 0, ctypes.c_void_p(8), None) == S
+    tlib = wq_testlib.load()
+    assert tlib.wq_copy_bytes(None, None, 24, None) == S
+    assert tlib.wq_selftest_fp8_elem(0, 0x9000, 0, ctypes.c_void_p(8), None) == S
 
 
 def test_check_raises_runtime_error():

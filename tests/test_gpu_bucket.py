@@ -76,33 +76,112 @@ def test_fp8_bucket_equals_per_param_loop_and_oracle(cuda):
     params[1][1][0][1].mul_(3)
     out2 = conv.convert(params)
     assert conv.plan_builds == 1 and out2.get_flattened_tensor().data_ptr() != out.get_flattened_tensor().data_ptr()
+    assert conv.resolves == 1
     _same_as_loop(out2, B.per_param_loop(None, params, FP8_CFG))
-    # same shapes at other addresses: a new table
+    # same shapes at other addresses: the layout is kept, only the addresses are resolved again (on the GPU)
     moved = [(mn, [(n, t.clone()) for n, t in cv]) for mn, cv in params]
     _same_as_loop(conv.convert(moved), B.per_param_loop(None, moved, FP8_CFG))
-    assert conv.plan_builds == 2
+    assert conv.plan_builds == 1 and conv.resolves == 2
     # into a caller-owned buffer
     buf = torch.empty(out.get_flattened_tensor().numel() + 64, dtype=torch.uint8, device=cuda)
     out3 = conv.convert(moved, out=buf)
     assert out3.get_flattened_tensor().data_ptr() == buf.data_ptr()
     _same_as_loop(out3, B.per_param_loop(None, moved, FP8_CFG))
+    assert conv.plan_builds == 1 and conv.resolves == 2
+
+
+@pytest.mark.parametrize("cfg", ["fp8", "int4", "int4_asym"])
+def test_bucket_inputs_reallocated_every_sync(cuda, cfg):
+    """What a sharded model presents: the same names and shapes every sync, each time in freshly allocated tensors
+    (gathered partitions, concatenated experts).  The layout is built once; every sync after that uploads the new
+    addresses and resolves the work-item table on the GPU - bytes equal to the per-parameter loop and to the oracle."""
+    config = {"fp8": FP8_CFG, "int4": INT4_CFG,
+              "int4_asym": {**INT4_CFG, "config_groups": {"group_0": {"weights": {"group_size": 128, "symmetric": False}}}}}[cfg]
+    conv = B.BucketConverter(None, config)
+    keep = []                                     # earlier syncs' tensors stay allocated: the new ones cannot reuse their addresses
+    for sync in range(4):
+        params = _moe_layer(0, cuda, 900 + sync) + _moe_layer(1, cuda, 950 + sync)
+        keep.append(params)
+        out = conv.convert(params, bucket_id="layers 0-1")
+        _same_as_loop(out, B.per_param_loop(None, params, config))
+        assert conv.plan_builds == 1 and conv.resolves == sync + 1
+        named = dict(out.reconstruct_tensors())
+        n, t = params[4][1][0]                   # an expert's gate projection: a chunk view of its fc1 weight
+        assert n.endswith("experts.0.gate_proj.weight")
+        if cfg == "fp8":
+            qo, so = C.fp8_block_quant(t.cpu().contiguous(), (128, 128), 1)
+            assert torch.equal(named[n].cpu().view(torch.uint8), qo)
+            assert torch.equal(named[n.replace(".weight", ".weight_scale_inv")].cpu().view(torch.int32), so.view(torch.int32))
+        else:
+            po, so, zo = C.int4_pack_layer(t.cpu().contiguous(), 128, cfg == "int4")
+            assert torch.equal(named[n.replace(".weight", ".weight_packed")].cpu(), po)
+            assert I.same_bits(named[n.replace(".weight", ".weight_scale")].cpu(), so)
+    # the first sync's tensors again (another move), without the id: found by the layout's identity
+    again = conv.convert(keep[0])
+    _same_as_loop(again, B.per_param_loop(None, keep[0], config))
+    assert conv.plan_builds == 2 and conv.convert(keep[0]).launches == again.launches and conv.plan_builds == 2
+
+
+def test_int4_bucket_input_that_lost_its_alignment(cuda):
+    """The cached routing of an INT4 bucket sends 16-byte aligned weights to the one-launch kernel.  The same bucket
+    with a weight at an address that is not (a view into a larger allocation) must not reuse it."""
+    w = I.weights(64, 512, seed=11).to(cuda)
+    name = [(L.format(0) + "mlp.experts.linear_fc2.weight0", "model.layers.0.mlp.experts.0.down_proj.weight")]
+    params = [(name[0][0], [(name[0][1], w)])]
+    conv = B.BucketConverter(None, INT4_CFG)
+    _same_as_loop(conv.convert(params, bucket_id=0), B.per_param_loop(None, params, INT4_CFG))
+    big = torch.zeros(64 * 512 + 4, dtype=torch.bfloat16, device=cuda)
+    shifted = big[4:].view(64, 512)
+    shifted.copy_(w)
+    assert shifted.data_ptr() % 16 == 8
+    params2 = [(name[0][0], [(name[0][1], shifted)])]
+    out = conv.convert(params2, bucket_id=0)
+    _same_as_loop(out, B.per_param_loop(None, params, INT4_CFG))
+    assert conv.plan_builds == 2
+
+
+def test_bucket_with_an_odd_sized_member_is_the_plain_concatenation(cuda):
+    """FlattenedTensorBucket packs back to back without padding.  When that puts a wider tensor at an offset that is not
+    a multiple of its element size, the converter must still produce exactly that buffer (no gap bytes, cumulative
+    offsets): it runs the per-parameter loop and concatenates."""
+    params = [("module.module.x.flags", [("flags", torch.arange(7, device=cuda, dtype=torch.uint8))]),
+              (L.format(0) + "self_attention.linear_proj.weight", [("model.layers.0.self_attn.o_proj.weight", I.weights(256, 128, seed=1).to(cuda))]),
+              ("module.module.x.norm", [("model.norm.weight", I.weights(1, 64, seed=2)[0].to(cuda))])]
+    conv = B.BucketConverter(None, FP8_CFG)
+    want = B.per_param_loop(None, params, FP8_CFG)
+    for _ in range(2):
+        out = conv.convert(params)
+        flat = B.flatten_named_tensors(want)
+        assert torch.equal(out.get_flattened_tensor(), flat.get_flattened_tensor())
+        assert [(m.name, m.start_idx, m.end_idx) for m in out.metadata] == [(m.name, m.start_idx, m.end_idx) for m in flat.metadata]
+        assert out.metadata[1].start_idx == 7 and out.metadata[2].start_idx == 7 + 256 * 128      # the scale sits at an odd offset
+    assert conv.plan_builds == 1
+
+
+def test_bucket_accepts_generators(cuda):
+    params = _moe_layer(0, cuda, 990, experts=1)
+    want = B.per_param_loop(None, params, FP8_CFG)
+    conv = B.BucketConverter(None, FP8_CFG)
+    for _ in range(2):
+        lazy = ((mn, ((n, t) for n, t in cv)) for mn, cv in params)
+        _same_as_loop(conv.convert(lazy, bucket_id="lazy"), want)
 
 
 def test_fp8_bucket_odd_members(cuda):
     # ragged shapes, a strided quantised member (generic tiles), a non-contiguous pass-through, members whose byte
-    # sizes put the next one at odd offsets (4-byte and 2-byte aligned destinations), an empty tensor, an fp32 weight
-    # and a *_scale entry that the expert rule drops
+    # sizes put the next one at 4-byte and 2-byte aligned offsets (every tensor still at a multiple of its element
+    # size), an empty tensor, an fp32 weight and a *_scale entry that the expert rule drops
     w = I.weights(300, 200, seed=1).to(cuda)
     wide = I.weights(264, 520, seed=2).to(cuda)
     params = [
         ("module.module.decoder.layers.0.mlp.router.expert_bias", [("model.layers.0.mlp.gate.e_score_correction_bias", torch.arange(3, device=cuda, dtype=torch.float32))]),
         (L.format(0) + "self_attention.linear_proj.weight", [("model.layers.0.self_attn.o_proj.weight", w)]),
         ("module.module.x.odd", [("odd.bf16", I.weights(1, 3, seed=3)[0].to(cuda))]),
-        (L.format(0) + "mlp.linear_fc2.weight", [("model.layers.0.mlp.down_proj.weight", wide[:, 8:][:, ::2])]),
+        (L.format(0) + "mlp.linear_fc2.weight", [("model.layers.0.mlp.down_proj.weight", wide[:263, 8:516][:, ::2])]),
         ("module.module.x.strided", [("strided.pass", wide.t())]),
         ("module.module.x.empty", [("empty", torch.empty(0, 4, device=cuda, dtype=torch.bfloat16))]),
         (L.format(0) + "mlp.linear_fc1.weight", [("model.layers.0.mlp.gate_proj.weight", I.weights(7, 7168, seed=4).to(cuda)),
-                                                 ("model.layers.0.mlp.up_proj.weight", I.weights(129, 127, seed=5).to(cuda).float())]),
+                                                 ("model.layers.0.mlp.up_proj.weight", I.weights(129, 128, seed=5).to(cuda).float())]),
         (L.format(0) + "mlp.experts.linear_fc1.weight0", [("model.layers.0.mlp.experts.0.gate_proj.weight", I.weights(128, 128, seed=6).to(cuda)),
                                                          ("model.layers.0.mlp.experts.0.gate_proj.weight_scale", torch.ones(1, device=cuda))]),
     ]
@@ -112,8 +191,12 @@ def test_fp8_bucket_odd_members(cuda):
     for _ in range(2):
         _same_as_loop(conv.convert(params), want)
     assert conv.plan_builds == 1
-    o, so = C.fp8_block_quant(wide[:, 8:][:, ::2].cpu(), (128, 128), 1)
-    named = dict(conv.convert(params).reconstruct_tensors())
+    o, so = C.fp8_block_quant(wide[:263, 8:516][:, ::2].cpu(), (128, 128), 1)
+    out = conv.convert(params)
+    assert out.launches > 1 and not conv._layouts[next(iter(conv._layouts))].fallback       # the one-launch path plus the late members
+    starts = {m.name: m.start_idx for m in out.metadata}
+    assert starts["model.layers.0.mlp.down_proj.weight"] % 4 == 2 and starts["model.layers.0.self_attn.o_proj.weight"] % 16 == 12
+    named = dict(out.reconstruct_tensors())
     assert torch.equal(named["model.layers.0.mlp.down_proj.weight"].cpu().view(torch.uint8), o)
 
 
