@@ -103,6 +103,16 @@ typedef struct wq_fp8_quant_desc {
 int wq_fp8_block_quant_grouped(const wq_fp8_quant_desc *descs, const int64_t *tile_start, int n_desc,
                                int64_t total_tiles, int bm, int bn, int mode, void *stream);
 
+/* The grouped launch for up to WQ_FP8_FEW_MAX tensors, with the descriptors in the kernel arguments: `descs` is a
+ * HOST array that the call reads before it returns - no device table to build, upload, cache or keep valid.  Meant for
+ * the q/k/v or gate/up group of ONE weight-sync parameter (quantize_params_fp8, quantizer_fp8.py:69-95, calls
+ * _quantize_param once per tensor of the group), whose tensors are fresh allocations on every sync.  With out_base
+ * non-NULL the y and s fields are byte offsets from it (one allocation for all outputs of the group).  Descriptors
+ * with M == 0 or N == 0 are skipped. */
+#define WQ_FP8_FEW_MAX 4
+int wq_fp8_block_quant_few(const wq_fp8_quant_desc *descs, int n_desc, void *out_base, int bm, int bn, int mode,
+                           void *stream);
+
 /* The same launch with every tile resolved beforehand: `tiles` is a DEVICE array with one descriptor per
  * (bm x bn) tile, moved to the tile's origin - x and y point at the tile's first element, s at the tile's scale,
  * M and N are the rows and columns of the tensor from there on (the kernel uses min(bm, M) x min(bn, N)), strides

@@ -26,6 +26,7 @@ DEQ_SEG, DEQ_SEGS_PER_WG = 512, 16
 INT4_GROUPS_PER_WG = 64
 INT4_DEQ_WORDS_PER_ITEM = 512
 BUCKET_COPY_MARK, BUCKET_COPY_BYTES = -1, 32768
+FP8_FEW_MAX = 4
 
 _i64, _int, _vp, _u32, _u64 = ctypes.c_int64, ctypes.c_int, ctypes.c_void_p, ctypes.c_uint32, ctypes.c_uint64
 
@@ -36,6 +37,7 @@ SIGNATURES = {
     "wq_fp8_block_quant": [_vp, _i64, _i64, _i64, _i64, _vp, _i64, _vp, _int, _int, _int, _vp],
     "wq_fp8_block_quant_grouped": [_vp, _vp, _int, _i64, _int, _int, _int, _vp],
     "wq_fp8_block_quant_tiles": [_vp, _i64, _int, _int, _int, _vp],
+    "wq_fp8_block_quant_few": [_vp, _int, _vp, _int, _int, _int, _vp],
     "wq_fp8_bucket_convert": [_vp, _i64, _vp, _int, _int, _int, _vp],
     "wq_int4_bucket_convert": [_vp, _i64, _vp, _int, _vp],
     "wq_bucket_resolve_items": [_vp, _vp, _vp, _i64, _int, _vp, _vp],

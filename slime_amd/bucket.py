@@ -35,11 +35,13 @@ import numpy as np
 import torch
 
 from . import _lib
+from ._tables import ResolvedTable
 from .fp8 import FP8_DTYPE, ceildiv, tile_table
 from .int4 import item_table, zero_point_rows
 from .processors import _fp8_route, _is_ignored, quantize_params, ue8m0_requant_enabled
 
 _COPY = _lib.BUCKET_COPY_BYTES
+_ELEMENT_SIZE: dict = {}
 
 
 @dataclasses.dataclass(frozen=True)
@@ -93,13 +95,9 @@ def flatten_named_tensors(named_tensors) -> FlattenedBucket:
 
 class _Layout:
     """Everything about a bucket that does not depend on where its inputs live this sync."""
-    __slots__ = ("kind", "block", "group", "device", "metadata", "total_bytes", "n_tensors", "n_items", "width",
-                 "template", "owner", "items", "bases", "slot_src", "align", "const_base", "resolved_ptrs", "staging",
-                 "stage_events", "stage_next", "keepalive", "late_copies", "zero_bytes", "zp_rows", "zp_start",
+    __slots__ = ("kind", "block", "group", "device", "metadata", "total_bytes", "n_tensors", "n_items", "table",
+                 "slot_src", "align", "const_base", "keepalive", "late_copies", "zero_bytes", "zp_rows", "zp_start",
                  "zp_words", "n_zp", "fallback")
-
-
-_STAGING_DEPTH = 4
 
 
 class BucketConverter:
@@ -216,7 +214,7 @@ class BucketConverter:
         def place(name, shape, dtype):
             """The next tensor of the flat buffer, back to back as FlattenedTensorBucket packs them."""
             nonlocal off
-            esz = torch.empty((), dtype=dtype).element_size()
+            esz = _ELEMENT_SIZE.get(dtype) or _ELEMENT_SIZE.setdefault(dtype, torch.empty((), dtype=dtype).element_size())
             if off % esz:
                 # an odd-sized tensor ahead of a wider one: neither the kernels nor a consumer's .view(dtype) can
                 # address the wider tensor at this offset, and padding would not be the reference's layout
@@ -274,8 +272,7 @@ class BucketConverter:
         plan.late_copies = late
         plan.device = device
         plan.keepalive = []
-        plan.resolved_ptrs = None
-        plan.n_items, plan.template, plan.owner, plan.items = 0, None, None, None
+        plan.n_items, plan.table = 0, None
         plan.zero_bytes, plan.n_zp = zero_off, len(zp_entries)
         if plan.fallback:
             return plan
@@ -330,16 +327,10 @@ class BucketConverter:
             perm = torch.argsort(torch.cat(order), stable=True)
             table = torch.cat(blocks, dim=0)[perm].contiguous()
             assert table.shape[1] == width
-            plan.n_items, plan.width = table.shape[0], width
-            plan.template = table.to(device)
-            plan.owner = torch.cat(owners)[perm].to(torch.int32).contiguous().to(device)
-            plan.items = torch.empty_like(plan.template)
+            plan.n_items = table.shape[0]
+            plan.table = ResolvedTable(table, torch.cat(owners)[perm], const_slot + 1, device)
             plan.slot_src = np.asarray(slot_src, dtype=np.int64)
             plan.align = np.asarray(align, dtype=np.int64)
-            n_bases = const_slot + 1
-            plan.bases = torch.empty(n_bases, dtype=torch.int64, device=device)
-            plan.staging = [torch.empty(n_bases, dtype=torch.int64).pin_memory() for _ in range(_STAGING_DEPTH)]
-            plan.stage_events, plan.stage_next = [None] * _STAGING_DEPTH, 0
         if zp_entries:
             zrows, zstart, plan.zp_words = zero_point_rows(zp_entries)
             plan.zp_rows, plan.zp_start = zrows.to(device), zstart.to(device)
@@ -355,24 +346,7 @@ class BucketConverter:
         bases = arr[plan.slot_src]
         if np.any(bases & plan.align):
             return False
-        k = plan.stage_next
-        plan.stage_next = (k + 1) % _STAGING_DEPTH
-        if plan.stage_events[k] is not None:
-            plan.stage_events[k].synchronize()          # the upload that last used this staging buffer has finished
-        host = plan.staging[k]
-        h = host.numpy()
-        h[:-1] = bases
-        h[-1] = plan.const_base
-        stream = torch.cuda.current_stream(plan.device)
-        with torch.cuda.device(plan.device):
-            plan.bases.copy_(host, non_blocking=True)
-            ev = torch.cuda.Event()
-            ev.record(stream)
-            plan.stage_events[k] = ev
-            rc = _lib.load().wq_bucket_resolve_items(plan.template.data_ptr(), plan.owner.data_ptr(), plan.bases.data_ptr(),
-                                                     plan.n_items, plan.width, plan.items.data_ptr(), stream.cuda_stream)
-        _lib.check(rc, "BucketConverter: resolving the work-item table")
-        plan.resolved_ptrs = ptrs
+        plan.table.resolve(np.append(bases, plan.const_base), tag=ptrs)
         self.resolves += 1
         return True
 
@@ -406,7 +380,7 @@ class BucketConverter:
                 # back-to-back packing puts a tensor at an offset that is not a multiple of its element size:
                 # the per-parameter loop and a plain concatenation, exactly as the reference builds the buffer
                 return flatten_named_tensors(per_param_loop(self.args, params, self.config, self.transform_ue8m0))
-            if not plan.n_items or ptrs == plan.resolved_ptrs or self._resolve(plan, ptrs):
+            if not plan.n_items or ptrs == plan.table.resolved_for or self._resolve(plan, ptrs):
                 break
             plan = None                                  # an input lost the alignment the cached routing relied on
         device = plan.device
@@ -423,13 +397,13 @@ class BucketConverter:
                 ev[0].record(torch.cuda.current_stream(device))
             with torch.cuda.device(device):
                 if plan.kind == "fp8":
-                    rc = lib.wq_fp8_bucket_convert(plan.items.data_ptr(), plan.n_items, out.data_ptr(), plan.block[0],
+                    rc = lib.wq_fp8_bucket_convert(plan.table.items.data_ptr(), plan.n_items, out.data_ptr(), plan.block[0],
                                                    plan.block[1], _lib.FP8_MODE_TRITON, _lib.stream_ptr(device))
                 elif plan.kind == "int4_asym":
                     # the pack kernel leaves every group's zero point in a scratch buffer; a second launch packs them
                     # eight rows to a word into their place in the bucket
                     zero = torch.empty(max(plan.zero_bytes, 16), dtype=torch.uint8, device=device)
-                    rc = lib.wq_int4_group_quant_pack_asym_items(plan.items.data_ptr(), plan.n_items, out.data_ptr(),
+                    rc = lib.wq_int4_group_quant_pack_asym_items(plan.table.items.data_ptr(), plan.n_items, out.data_ptr(),
                                                                  zero.data_ptr(), plan.group, _lib.stream_ptr(device))
                     if rc == 0 and plan.n_zp:
                         rc = lib.wq_int4_zero_point_pack_grouped(plan.zp_rows.data_ptr(), plan.zp_start.data_ptr(), plan.n_zp,
@@ -437,7 +411,7 @@ class BucketConverter:
                                                                  _lib.stream_ptr(device))
                         launches += 1
                 else:
-                    rc = lib.wq_int4_bucket_convert(plan.items.data_ptr(), plan.n_items, out.data_ptr(), plan.group,
+                    rc = lib.wq_int4_bucket_convert(plan.table.items.data_ptr(), plan.n_items, out.data_ptr(), plan.group,
                                                     _lib.stream_ptr(device))
             _lib.check(rc, "BucketConverter.convert")
             launches += 1

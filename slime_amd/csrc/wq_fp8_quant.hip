@@ -230,6 +230,47 @@ __global__ __launch_bounds__(kTileThreads) void fp8_block_quant_kernel(const Fp8
         quant_tile_generic<MODE>(d, tm, tn, kt, a.bm, a.bn, lds);
 }
 
+// Up to WQ_FP8_FEW_MAX tensors with their descriptors in the kernel arguments: no device table to build, upload or keep.
+// The owner of a tile is found by comparing against the (at most three) interior prefix sums and the descriptor is
+// selected field by field, so everything stays in scalar registers (indexing the argument array with a run-time value
+// would move it to scratch memory).
+constexpr int kFewMax = WQ_FP8_FEW_MAX;
+struct Fp8FewArgs {
+    wq_fp8_quant_desc d[kFewMax];
+    int64_t tile_start[kFewMax + 1];
+    int32_t n_desc, bm, bn;
+    char* out_base;      // when set, y and s of every descriptor are byte offsets from here
+};
+
+template <int MODE, bool SMALL>
+__global__ __launch_bounds__(kTileThreads) void fp8_block_quant_few_kernel(const Fp8FewArgs a, const int64_t total_tiles)
+{
+    __shared__ __attribute__((aligned(16))) uint32_t lds[kRowSlots];
+    const int64_t slot = (int64_t)blockIdx.x + (int64_t)blockIdx.y * gridDim.x;
+    if (slot >= total_tiles) return;  // uniform per workgroup
+    const int64_t tile = xcd_chunked_item(slot, total_tiles, kTilesPerXcdRun);
+    wq_fp8_quant_desc d = a.d[0];
+    int64_t first = 0;
+#pragma unroll
+    for (int k = 1; k < kFewMax; ++k) {
+        if (k < a.n_desc && tile >= a.tile_start[k]) {
+            d = a.d[k];
+            first = a.tile_start[k];
+        }
+    }
+    if (a.out_base) {
+        d.y = a.out_base + (uintptr_t)d.y;
+        d.s = (float*)(a.out_base + (uintptr_t)d.s);
+    }
+    const int64_t local = tile - first;
+    const int kt = (int)((d.N + a.bn - 1) / a.bn);
+    const int64_t tm = local / kt, tn = local - tm * kt;
+    if (a.bm == 128 && a.bn == 128 && desc_vector_ok(d))
+        quant_tile_vec128<MODE, SMALL ? kSmallTileWindow : kTileWindow>(d, tm, tn, kt, lds);
+    else
+        quant_tile_generic<MODE>(d, tm, tn, kt, a.bm, a.bn, lds);
+}
+
 // ---- per-row (channel) and per-tensor scaling -------------------------------------------------
 
 // The row and tensor forms exist only in the torch formulation; the scale rule is a run-time choice there.
@@ -683,6 +724,16 @@ static void launch_block_quant(const Fp8QuantArgs& a, int64_t tiles, int mode, h
     else launch_block_quant_mode<WQ_FP8_MODE_TRITON, GROUPED>(a, tiles, st);
 }
 
+template <int MODE>
+static void launch_block_quant_few_mode(const Fp8FewArgs& a, int64_t tiles, hipStream_t st)
+{
+    const dim3 g = grid_for_items(tiles);
+    if (tiles <= kSmallLaunchTiles)
+        fp8_block_quant_few_kernel<MODE, true><<<g, kTileThreads, kSmallOccupancyPadBytes, st>>>(a, tiles);
+    else
+        fp8_block_quant_few_kernel<MODE, false><<<g, kTileThreads, kOccupancyPadBytes, st>>>(a, tiles);
+}
+
 static int check_desc_host(const void* x, int64_t M, int64_t N, const void* y, const float* s, int bm, int bn, int mode)
 {
     if (M < 0 || N < 0 || bm <= 0 || bn <= 0) return WQ_ERR_SHAPE;
@@ -851,6 +902,42 @@ WQ_EXPORT int wq_fp8_block_quant_tiles(const wq_fp8_quant_desc* tiles, int64_t n
     a.bm = bm;
     a.bn = bn;
     launch_block_quant<2>(a, n_tiles, mode, (hipStream_t)stream);
+    WQ_LAUNCH_CHECK();
+    return WQ_OK;
+}
+
+WQ_EXPORT int wq_fp8_block_quant_few(const wq_fp8_quant_desc* descs, int n_desc, void* out_base, int bm, int bn, int mode,
+                                     void* stream)
+{
+    if (n_desc < 0 || n_desc > kFewMax || bm <= 0 || bn <= 0) return WQ_ERR_SHAPE;
+    if (!known_mode(mode)) return WQ_ERR_MODE;
+    if (n_desc == 0) return WQ_OK;
+    if (!descs) return WQ_ERR_NULL;
+    if ((int64_t)bm * bn > (1 << 30)) return WQ_ERR_TOO_LARGE;
+    Fp8FewArgs a{};
+    int64_t tiles = 0;
+    int n = 0;
+    for (int i = 0; i < n_desc; ++i) {          // `descs` is host memory: checked and copied into the kernel arguments
+        const wq_fp8_quant_desc& d = descs[i];
+        if (d.M < 0 || d.N < 0) return WQ_ERR_SHAPE;
+        if (d.M == 0 || d.N == 0) continue;
+        if (!d.x || (!out_base && (!d.y || !d.s))) return WQ_ERR_NULL;
+        a.d[n] = d;
+        a.tile_start[n] = tiles;
+        tiles += cdiv64(d.M, bm) * cdiv64(d.N, bn);
+        ++n;
+    }
+    if (n == 0) return WQ_OK;
+    for (int i = n; i <= kFewMax; ++i) a.tile_start[i] = tiles;
+    a.n_desc = n;
+    a.bm = bm;
+    a.bn = bn;
+    a.out_base = (char*)out_base;
+    hipStream_t st = (hipStream_t)stream;
+    if (mode == WQ_FP8_MODE_TORCH) launch_block_quant_few_mode<WQ_FP8_MODE_TORCH>(a, tiles, st);
+    else if (mode == WQ_FP8_MODE_TORCH_DEVICE) launch_block_quant_few_mode<WQ_FP8_MODE_TORCH_DEVICE>(a, tiles, st);
+    else if (mode == WQ_FP8_MODE_UE8M0) launch_block_quant_few_mode<WQ_FP8_MODE_UE8M0>(a, tiles, st);
+    else launch_block_quant_few_mode<WQ_FP8_MODE_TRITON>(a, tiles, st);
     WQ_LAUNCH_CHECK();
     return WQ_OK;
 }

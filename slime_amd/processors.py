@@ -16,13 +16,16 @@ the reference whenever that path is off.
 
 from __future__ import annotations
 
+import ctypes
 import re
 import threading
 from collections import OrderedDict
 
+import numpy as np
 import torch
 
 from . import _lib
+from ._tables import ResolvedTable
 from .fp8 import (FP8_DTYPE, blockwise_cast_to_fp8_triton, ceildiv, quant_weight_ue8m0, tensor_fp8, tile_table,
                   transform_scale_ue8m0)
 from .int4 import pack_layer
@@ -136,60 +139,57 @@ def quantize_params_fp8(args, megatron_name, converted_named_params, quantizatio
     return result
 
 
-_GROUP_TABLES: OrderedDict = OrderedDict()
-_GROUP_LOCK = threading.Lock()
-_GROUP_STATS = {"builds": 0, "hits": 0, "bytes": 0}
-# The cache is bounded by the device memory its tables take, not by a count: an MoE model presents one gate/up pair per
-# expert and layer (6 144 for 48 x 128 experts, 12 KiB of table each) in the same order on every sync, and a
-# least-recently-used list shorter than that cycle would miss every time.
-_GROUP_MAX_BYTES = 512 << 20
-
-
-def plan_cache_info() -> dict:
-    """Counters of the descriptor-table cache behind the grouped launch of ``quantize_params_fp8``."""
-    return dict(_GROUP_STATS, entries=len(_GROUP_TABLES))
+class _QuantDesc(ctypes.Structure):
+    """``wq_fp8_quant_desc``."""
+    _fields_ = [("x", ctypes.c_void_p), ("y", ctypes.c_void_p), ("s", ctypes.c_void_p), ("M", ctypes.c_int64),
+                ("N", ctypes.c_int64), ("sx_m", ctypes.c_int64), ("sx_n", ctypes.c_int64), ("sy_m", ctypes.c_int64)]
 
 
 def _group_cast(weights, block_size):
-    """``blockwise_cast_to_fp8_triton`` over a few tensors with one launch -> [(qweight, scale)], fresh outputs (slices
-    of one new allocation).  The per-tile table depends only on the addresses, shapes and strides of the inputs and is
-    cached: a parameter that comes back at the same addresses on the next sync costs no host-side table work."""
+    """``blockwise_cast_to_fp8_triton`` over the few tensors of one parameter with one launch -> [(qweight, scale)],
+    fresh outputs (slices of one new allocation).  The descriptors travel in the kernel arguments
+    (``wq_fp8_block_quant_few``): nothing is cached and nothing depends on where the inputs live, so a parameter
+    that is gathered into fresh tensors on every sync costs the same as one that stays put."""
     bm, bn = int(block_size[0]), int(block_size[1])
     device = weights[0].device
-    key = (bm, bn, device.index, tuple((w.data_ptr(), tuple(w.shape), w.stride()) for w in weights))
-    with _GROUP_LOCK:
-        entry = _GROUP_TABLES.get(key)
-        if entry is not None:
-            _GROUP_TABLES.move_to_end(key)
-            _GROUP_STATS["hits"] += 1
-    if entry is None:
-        rows, layout, off = [], [], 0
-        for w in weights:
+    results = []
+    lib = _lib.load()
+    for g0 in range(0, len(weights), _lib.FP8_FEW_MAX):
+        group = weights[g0:g0 + _lib.FP8_FEW_MAX]
+        descs = (_QuantDesc * len(group))()
+        layout, off = [], 0
+        for d, w in zip(descs, group):
             M, N = w.shape
             tm, tn = ceildiv(M, bm), ceildiv(N, bn)
             q0 = off
             s0 = (q0 + M * N + 15) // 16 * 16
             off = (s0 + 4 * tm * tn + 15) // 16 * 16
-            rows.append([w.data_ptr(), q0, s0, M, N, w.stride(0), w.stride(1), N])
+            d.x, d.y, d.s, d.M, d.N, d.sx_m, d.sx_n, d.sy_m = w.data_ptr(), q0, s0, M, N, w.stride(0), w.stride(1), N
             layout.append((q0, M, N, s0, tm, tn))
-        table, _, _ = tile_table(rows, bm, bn)
-        entry = (table.contiguous().to(device), table.shape[0], layout, off)
-        with _GROUP_LOCK:
-            if key not in _GROUP_TABLES:
-                _GROUP_STATS["bytes"] += entry[0].numel() * 8
-            _GROUP_TABLES[key] = entry
-            _GROUP_STATS["builds"] += 1
-            while _GROUP_STATS["bytes"] > _GROUP_MAX_BYTES and len(_GROUP_TABLES) > 1:
-                _, old = _GROUP_TABLES.popitem(last=False)
-                _GROUP_STATS["bytes"] -= old[0].numel() * 8
-    table, n_tiles, layout, total = entry
-    flat = torch.empty(total, dtype=torch.uint8, device=device)
-    with torch.cuda.device(device):
-        rc = _lib.load().wq_fp8_bucket_convert(table.data_ptr(), n_tiles, flat.data_ptr(), bm, bn, _lib.FP8_MODE_TRITON,
-                                               _lib.stream_ptr(device))
-    _lib.check(rc, "quantize_params_fp8")
-    return [(flat[q0:q0 + M * N].view(FP8_DTYPE).view(M, N), flat[s0:s0 + 4 * tm * tn].view(torch.float32).view(tm, tn))
-            for q0, M, N, s0, tm, tn in layout]
+        flat = torch.empty(off, dtype=torch.uint8, device=device)
+        with torch.cuda.device(device):
+            rc = lib.wq_fp8_block_quant_few(descs, len(group), flat.data_ptr(), bm, bn, _lib.FP8_MODE_TRITON,
+                                            _lib.stream_ptr(device))
+        _lib.check(rc, "quantize_params_fp8")
+        results += [(flat[q0:q0 + M * N].view(FP8_DTYPE).view(M, N), flat[s0:s0 + 4 * tm * tn].view(torch.float32).view(tm, tn))
+                    for q0, M, N, s0, tm, tn in layout]
+    return results
+
+
+# Work-item tables of quantize_grouped_weights, one per (expert count, shape, strides, block, device): address-free
+# templates (see _tables.ResolvedTable), so the number of entries is the number of distinct grouped linears, not the
+# number of allocations they have lived in.
+_GROUP_TABLES: OrderedDict = OrderedDict()
+_GROUP_LOCK = threading.Lock()
+_GROUP_STATS = {"builds": 0, "hits": 0, "resolves": 0, "bytes": 0}
+_GROUP_MAX_ENTRIES = 64
+_GROUP_MAX_BYTES = 512 << 20
+
+
+def plan_cache_info() -> dict:
+    """Counters of the work-item table cache behind ``quantize_grouped_weights``: layouts built on the host, calls
+    that found theirs, calls whose weights had moved (one address upload and one small launch each), device bytes held."""
+    return dict(_GROUP_STATS, entries=len(_GROUP_TABLES))
 
 
 def quantize_grouped_weights(weights, block_size=(128, 128), use_ue8m0: bool = False):
@@ -200,8 +200,9 @@ def quantize_grouped_weights(weights, block_size=(128, 128), use_ue8m0: bool = F
     deepgemm_moe_forward.py:1383-1428), which calls ``ops.quantize_weight(weight, (128, 128))`` - that is
     ``blockwise_cast_to_fp8_triton``, or sglang's ``quant_weight_ue8m0`` with ``use_ue8m0`` - once per expert and copies
     every result into the stacked tensors: E launches, 2 E copies and a second pass over the quantised bytes.  Same
-    bytes; the per-tile table is cached on the addresses of the weights (a training step presents the same parameters
-    again).  All weights: 2-D bf16 on one GPU, one shape.  The reference's later ``requant_weight_ue8m0`` of the stacked
+    bytes.  The per-tile table is cached per layout (expert count, shape, strides), not per address: weights that come
+    back somewhere else cost one upload of E addresses and one small launch.  Calls must be ordered on one stream.
+    All weights: 2-D bf16 on one GPU, one shape.  The reference's later ``requant_weight_ue8m0`` of the stacked
     tensors (sglang, Blackwell only) is not provided."""
     weights = list(weights)
     if not weights:
@@ -221,30 +222,31 @@ def quantize_grouped_weights(weights, block_size=(128, 128), use_ue8m0: bool = F
     if E * M * N == 0:
         return (torch.empty((E, M, N), dtype=FP8_DTYPE, device=device),
                 torch.empty((E, tm, tn), dtype=torch.float32, device=device))
-    key = ("stacked", bm, bn, device.index, tuple((w.data_ptr(), w.stride()) for w in weights), shape)
+    key = ("stacked", bm, bn, device.index, shape, tuple(w.stride() for w in weights))
+    ptrs = [w.data_ptr() for w in weights]
+    s_base = (E * M * N + 15) // 16 * 16
     with _GROUP_LOCK:
-        entry = _GROUP_TABLES.get(key)
-        if entry is not None:
+        table = _GROUP_TABLES.get(key)
+        if table is not None:
             _GROUP_TABLES.move_to_end(key)
             _GROUP_STATS["hits"] += 1
-    s_base = (E * M * N + 15) // 16 * 16
-    if entry is None:
-        rows = [[w.data_ptr(), e * M * N, s_base + 4 * e * tm * tn, M, N, w.stride(0), w.stride(1), N]
-                for e, w in enumerate(weights)]
-        table, _, _ = tile_table(rows, bm, bn)
-        entry = (table.contiguous().to(device), table.shape[0], None, s_base + 4 * E * tm * tn)
-        with _GROUP_LOCK:
-            if key not in _GROUP_TABLES:
-                _GROUP_STATS["bytes"] += entry[0].numel() * 8
-            _GROUP_TABLES[key] = entry
+        else:
+            rows = [[0, e * M * N, s_base + 4 * e * tm * tn, M, N, w.stride(0), w.stride(1), N] for e, w in enumerate(weights)]
+            template, owner, _ = tile_table(rows, bm, bn)
+            table = ResolvedTable(template, owner, E, device)
+            _GROUP_TABLES[key] = table
             _GROUP_STATS["builds"] += 1
-            while _GROUP_STATS["bytes"] > _GROUP_MAX_BYTES and len(_GROUP_TABLES) > 1:
+            _GROUP_STATS["bytes"] += table.device_bytes
+            while (len(_GROUP_TABLES) > _GROUP_MAX_ENTRIES or _GROUP_STATS["bytes"] > _GROUP_MAX_BYTES) and len(_GROUP_TABLES) > 1:
                 _, old = _GROUP_TABLES.popitem(last=False)
-                _GROUP_STATS["bytes"] -= old[0].numel() * 8
-    table, n_tiles, _, total = entry
-    flat = torch.empty(total, dtype=torch.uint8, device=device)
-    with torch.cuda.device(device):
-        rc = _lib.load().wq_fp8_bucket_convert(table.data_ptr(), n_tiles, flat.data_ptr(), bm, bn, mode, _lib.stream_ptr(device))
+                _GROUP_STATS["bytes"] -= old.device_bytes
+        if table.resolved_for != ptrs:
+            table.resolve(np.asarray(ptrs, dtype=np.int64), tag=ptrs)
+            _GROUP_STATS["resolves"] += 1
+        flat = torch.empty(s_base + 4 * E * tm * tn, dtype=torch.uint8, device=device)
+        with torch.cuda.device(device):
+            rc = _lib.load().wq_fp8_bucket_convert(table.items.data_ptr(), table.n_items, flat.data_ptr(), bm, bn, mode,
+                                                   _lib.stream_ptr(device))
     _lib.check(rc, "quantize_grouped_weights")
     return (flat[:E * M * N].view(FP8_DTYPE).view(E, M, N),
             flat[s_base:s_base + 4 * E * tm * tn].view(torch.float32).view(E, tm, tn))

@@ -72,6 +72,12 @@ def test_argument_validation_without_launch():
     assert lib.wq_fp8_block_quant_tiles(None, 4, 128, 128, 9, None) == M_
     assert lib.wq_fp8_block_quant_tiles(None, 0, 128, 128, 0, None) == 0
     assert lib.wq_fp8_block_quant(None, 4, 4, 4, 1, None, 4, None, 128, 128, 2, None) == N_
+    assert lib.wq_fp8_block_quant_few(None, 5, None, 128, 128, 1, None) == S           # more than WQ_FP8_FEW_MAX
+    assert lib.wq_fp8_block_quant_few(None, 2, None, 128, 128, 1, None) == N_
+    assert lib.wq_fp8_block_quant_few(None, 0, None, 128, 128, 1, None) == 0
+    assert lib.wq_bucket_resolve_items(None, None, None, 3, 8, None, None) == N_
+    assert lib.wq_bucket_resolve_items(None, None, None, 3, 0, None, None) == S
+    assert lib.wq_bucket_resolve_items(ctypes.c_void_p(64), ctypes.c_void_p(64), ctypes.c_void_p(64), 3, 8, ctypes.c_void_p(64), None) == U
     assert lib.wq_fp8_row_quant(None, -1, 4, 4, 1, None, 4, None, 0, None) == S
     assert lib.wq_fp8_row_quant(None, 4, 4, 4, 1, None, 4, None, 1, None) == M_         # no Triton row form
     assert lib.wq_fp8_tensor_quant(None, 4, 4, 4, 1, None, 4, None, None, 2, None) == N_

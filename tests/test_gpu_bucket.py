@@ -266,18 +266,26 @@ def test_int4_bucket_asymmetric_and_other_groups(cuda):
     _same_as_loop(B.BucketConverter(None, g256).convert(one), B.per_param_loop(None, one, g256))
 
 
-def test_quantize_params_fp8_caches_its_table(cuda):
-    # the per-parameter entry point groups q/k/v (or gate/up) of one parameter into one launch; the same tensors
-    # presented again reuse the cached descriptor table
+def test_quantize_params_fp8_groups_one_parameter_into_one_launch(cuda):
+    # the per-parameter entry point puts q/k/v (or gate/up) of one parameter into one launch whose descriptors travel
+    # in the kernel arguments: no table, nothing cached, and the same bytes wherever the tensors live
     from slime_amd import processors
 
     params = _moe_layer(0, cuda, 700, experts=1)
-    mn, cv = params[1]
-    first = processors.quantize_params_fp8(None, mn, cv, FP8_CFG)
-    builds = processors.plan_cache_info()["builds"]
-    again = processors.quantize_params_fp8(None, mn, cv, FP8_CFG)
-    assert processors.plan_cache_info()["builds"] == builds
-    for (n0, a), (n1, b), (_, t) in zip(first[::2], again[::2], cv):
-        qo, _ = C.fp8_block_quant(t.cpu(), (128, 128), 1)
-        assert n0 == n1 and torch.equal(a.cpu().view(torch.uint8), qo) and torch.equal(b.cpu().view(torch.uint8), qo)
-        assert a.data_ptr() != b.data_ptr()          # fresh outputs on every call, like the reference
+    for mn, cv in (params[1], params[4]):                     # q/k/v (3 tensors), gate/up (2 chunk views)
+        first = processors.quantize_params_fp8(None, mn, cv, FP8_CFG)
+        moved = [(n, t.clone()) for n, t in cv]
+        again = processors.quantize_params_fp8(None, mn, moved, FP8_CFG)
+        assert [n for n, _ in first] == [n for n, _ in again] and len(first) == 2 * len(cv)
+        for (n0, a), (_, sa), (n1, b), (_, sb), (_, t) in zip(first[::2], first[1::2], again[::2], again[1::2], cv):
+            qo, so = C.fp8_block_quant(t.cpu().contiguous(), (128, 128), 1)
+            assert n0 == n1 and torch.equal(a.cpu().view(torch.uint8), qo) and torch.equal(b.cpu().view(torch.uint8), qo)
+            assert torch.equal(sa.cpu().view(torch.int32), so.view(torch.int32)) and I.same_bits(sa, sb)
+            assert a.data_ptr() != b.data_ptr()          # fresh outputs on every call, like the reference
+    # more tensors than one launch's kernel arguments hold: split over launches, same results
+    many = [(f"model.layers.0.self_attn.p{i}.weight", I.weights(130 + i, 264, seed=i).to(cuda)) for i in range(6)]
+    outs = processors.quantize_params_fp8(None, L.format(0) + "self_attention.linear_qkv.weight", many, FP8_CFG)
+    for (n, t), (nq, q), (ns, s) in zip(many, outs[::2], outs[1::2]):
+        qo, so = C.fp8_block_quant(t.cpu(), (128, 128), 1)
+        assert nq == n and ns == n.replace(".weight", ".weight_scale_inv")
+        assert torch.equal(q.cpu().view(torch.uint8), qo) and torch.equal(s.cpu().view(torch.int32), so.view(torch.int32))

@@ -87,10 +87,19 @@ def test_quantize_grouped_weights_equals_the_per_expert_loop(cuda, shape, ue8m0)
         assert I.same_bits(q[e].view(torch.uint8), qe.view(torch.uint8)) and I.same_bits(s[e], se), e
         qo, so = C.fp8_block_quant(w.cpu().contiguous(), (128, 128), 3 if ue8m0 else 1)
         assert torch.equal(q[e].cpu().view(torch.uint8), qo) and I.same_bits(s[e].cpu(), so), e
-    builds = processors.plan_cache_info()["builds"]
+    info = processors.plan_cache_info()
     q2, _ = slime_amd.quantize_grouped_weights(views, (128, 128), use_ue8m0=ue8m0)
-    assert processors.plan_cache_info()["builds"] == builds and I.same_bits(q2.view(torch.uint8), q.view(torch.uint8))
+    after = processors.plan_cache_info()
+    assert (after["builds"], after["resolves"]) == (info["builds"], info["resolves"])      # same weights: nothing to do
+    assert I.same_bits(q2.view(torch.uint8), q.view(torch.uint8))
     assert q2.data_ptr() != q.data_ptr()                              # fresh outputs on every call
+    # the same grouped linear somewhere else (freshly gathered weights): the layout is reused, the addresses resolved again
+    moved = [w.clone(memory_format=torch.preserve_format) for w in views]
+    assert [w.stride() for w in moved] == [w.stride() for w in views] and moved[0].data_ptr() != views[0].data_ptr()
+    q3, s3 = slime_amd.quantize_grouped_weights(moved, (128, 128), use_ue8m0=ue8m0)
+    last = processors.plan_cache_info()
+    assert last["builds"] == info["builds"] and last["resolves"] == info["resolves"] + 1
+    assert I.same_bits(q3.view(torch.uint8), q.view(torch.uint8)) and I.same_bits(s3, s)
 
 
 def test_quantize_grouped_weights_argument_errors(cuda):
