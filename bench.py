@@ -27,6 +27,7 @@ if os.path.join(ROOT, "tests") not in sys.path:
     sys.path.append(os.path.join(ROOT, "tests"))         # wq_testlib: the binding of the calibration kernels
 
 HBM_PEAK_GBS = 8000.0
+HEADLINE_FP8_MODE = 0          # WQ_FP8_MODE_TORCH: block_fp8 as the reference's test and the CPU baseline evaluate it
 
 QWEN3_4B_LAYER = [("q_proj", 4096, 2560), ("k_proj", 1024, 2560), ("v_proj", 1024, 2560), ("o_proj", 2560, 4096),
                   ("gate_proj", 9728, 2560), ("up_proj", 9728, 2560), ("down_proj", 2560, 9728)]
@@ -162,7 +163,9 @@ def bench_north_star(dev, steps, warmup, layers):
     from oracle import c_oracle
 
     weights, expert_weights = _moe_state_dict(dev, layers)
-    fp8_plan = slime_amd.Fp8QuantPlan(weights, (128, 128))
+    # The headline computes block_fp8 as the reference's own test runs it and as the CPU baseline beside it does: torch's
+    # CPU evaluation (WQ_FP8_MODE_TORCH = 0).  The two other arithmetic variants are timed on the same tensors below.
+    fp8_plan = slime_amd.Fp8QuantPlan(weights, (128, 128), mode=HEADLINE_FP8_MODE)
     int4_plan = slime_amd.Int4PackPlan(expert_weights, 128)
     wall_ms, mean, mn = _time_step([fp8_plan.run, int4_plan.run], steps, warmup)
 
@@ -170,14 +173,18 @@ def bench_north_star(dev, steps, warmup, layers):
     el_int4 = sum(w.numel() for w in expert_weights)
     algo_fp8 = 3 * el_fp8 + 4 * fp8_plan.total_tiles
     algo_int4 = 2 * el_int4 + el_int4 // 2 + el_int4 // 128 * 2
+    fp8_sample = (0, 2, 385, len(weights) - 1)
+
+    def check_fp8(plan):
+        for idx in fp8_sample:
+            q, s = plan.outputs[idx]
+            qo, so = c_oracle.fp8_block_quant(weights[idx].cpu().contiguous(), (128, 128), plan.mode)
+            assert torch.equal(q.cpu().view(torch.uint8), qo), f"FP8 parity failure on tensor {idx} (mode {plan.mode})"
+            assert torch.equal(s.cpu().view(torch.int32), so.view(torch.int32)), f"FP8 scale parity failure on tensor {idx} (mode {plan.mode})"
+        return len(fp8_sample)
+
     # parity on a sample of the very tensors that were timed
-    checked = 0
-    for idx in (0, 2, 385, len(weights) - 1):
-        q, s = fp8_plan.outputs[idx]
-        qo, so = c_oracle.fp8_block_quant(weights[idx].cpu().contiguous(), (128, 128), fp8_plan.mode)
-        assert torch.equal(q.cpu().view(torch.uint8), qo), f"FP8 parity failure on tensor {idx}"
-        assert torch.equal(s.cpu().view(torch.int32), so.view(torch.int32)), f"FP8 scale parity failure on tensor {idx}"
-        checked += 1
+    checked = check_fp8(fp8_plan)
     for idx in (0, 2, len(expert_weights) - 1):
         p, s = int4_plan.outputs[idx]
         po, so, _ = c_oracle.int4_pack_layer(expert_weights[idx].cpu().contiguous(), 128, True)
@@ -189,7 +196,25 @@ def bench_north_star(dev, steps, warmup, layers):
            "fp8": {"kernel_ms": mean[0], "kernel_ms_min": mn[0], "elements": el_fp8, "blocks": fp8_plan.total_tiles,
                    "algo_bytes": algo_fp8, "mode": fp8_plan.mode},
            "int4": {"kernel_ms": mean[1], "kernel_ms_min": mn[1], "elements": el_int4, "algo_bytes": algo_int4}}
-    del fp8_plan, int4_plan, weights, expert_weights
+    del fp8_plan, int4_plan
+    torch.cuda.empty_cache()
+    # the FP8 launch of the step in the two other arithmetic variants, same tensors, each checked against the oracle in
+    # its own mode: 1 = the weight-sync cast (blockwise_cast_to_fp8_triton), 2 = block_fp8 as torch evaluates it on GPU tensors
+    modes = {}
+    for mode, label in ((1, "weight-sync cast: fp32 amax floored at 1e-10, x * (1 / scale)"),
+                        (2, "block_fp8 as torch evaluates it on GPU tensors: scale = amax * RN(1/448), IEEE x / scale")):
+        plan = slime_amd.Fp8QuantPlan(weights, (128, 128), mode=mode)
+        _, ev_ms, ev_min = _time_launches(plan.run, steps, warmup)
+        n = check_fp8(plan)
+        modes[str(mode)] = {"arithmetic": label, "kernel_ms": ev_ms, "kernel_ms_min": ev_min,
+                            "hbm_frac": algo_fp8 / ev_ms / 1e6 / HBM_PEAK_GBS, "parity_tensors_checked": n}
+        del plan
+        torch.cuda.empty_cache()
+    modes[str(HEADLINE_FP8_MODE)] = {"arithmetic": "block_fp8 as torch evaluates it on CPU tensors (the headline): scale = amax / 448, IEEE x / scale",
+                                     "kernel_ms": mean[0], "kernel_ms_min": mn[0],
+                                     "hbm_frac": algo_fp8 / mean[0] / 1e6 / HBM_PEAK_GBS, "parity_tensors_checked": len(fp8_sample)}
+    out["fp8_modes"] = modes
+    del weights, expert_weights
     torch.cuda.empty_cache()
     return out
 
@@ -309,7 +334,7 @@ def bench_cfg1(dev, steps, warmup, n_buffers=8):
     return out
 
 
-def bench_fp8_quant_moe(dev, steps, warmup, layers):
+def bench_fp8_quant_moe(dev, steps, warmup, layers, mode=HEADLINE_FP8_MODE):
     """Block-FP8 quant of every linear weight of a Qwen3-30B-A3B-shaped state dict (48 layers: 128 experts x
     gate/up [768,2048], down [2048,768]; attention q [4096,2048], k/v [512,2048], o [2048,4096]), one grouped launch."""
     import torch
@@ -318,7 +343,7 @@ def bench_fp8_quant_moe(dev, steps, warmup, layers):
     from oracle import c_oracle
 
     weights, _ = _moe_state_dict(dev, layers)
-    plan = slime_amd.Fp8QuantPlan(weights, (128, 128))
+    plan = slime_amd.Fp8QuantPlan(weights, (128, 128), mode=mode)
     wall_ms, ev_ms, ev_min = _time_launches(plan.run, steps, warmup)
     elements = sum(w.numel() for w in weights)
     algo_bytes = 3 * elements + 4 * plan.total_tiles
@@ -327,8 +352,8 @@ def bench_fp8_quant_moe(dev, steps, warmup, layers):
         qo, so = c_oracle.fp8_block_quant(weights[idx].cpu().contiguous(), (128, 128), plan.mode)
         assert torch.equal(q.cpu().view(torch.uint8), qo) and torch.equal(s.cpu().view(torch.int32), so.view(torch.int32))
     out = {"workload": f"Qwen3-30B-A3B-shaped state dict, {layers} layers x (128 experts x gate, up [768,2048], down "
-                       "[2048,768] + q, k, v, o), block-FP8 128x128, one grouped launch",
-           "tensors": len(weights), "bf16_GB": 2 * elements / 1e9, "kernel_ms": ev_ms, "wall_ms": wall_ms,
+                       f"[2048,768] + q, k, v, o), block-FP8 128x128 (arithmetic mode {mode}), one grouped launch",
+           "mode": mode, "tensors": len(weights), "bf16_GB": 2 * elements / 1e9, "kernel_ms": ev_ms, "wall_ms": wall_ms,
            "bf16_GBps": 2 * elements / ev_ms / 1e6, "algo_GBps": algo_bytes / ev_ms / 1e6,
            "hbm_frac": algo_bytes / ev_ms / 1e6 / HBM_PEAK_GBS, "parity_tensors_checked": 4}
     del plan, weights
@@ -1000,6 +1025,8 @@ def main():
                     help="run just one of the other legs and print its record: a kernel for profiling, the plain copy "
                          "kernel that hardware counters are calibrated against, or the host-resident streaming run "
                          "(64 x 1 GiB buckets, PCIe-bound)")
+    ap.add_argument("--fp8-mode", type=int, default=HEADLINE_FP8_MODE, choices=[0, 1, 2],
+                    help="arithmetic of `--only fp8moe`: 0 block_fp8 on CPU tensors (the headline), 1 weight-sync cast, 2 block_fp8 on GPU tensors")
     ap.add_argument("--stream-buckets", type=int, default=64)
     ap.add_argument("--stream-bucket-mib", type=int, default=1024)
     ap.add_argument("--stream-no-download", action="store_true")
@@ -1031,7 +1058,7 @@ def main():
         print(json.dumps(bench_bucket(dev, args.steps, args.warmup, args.int4_layers)))
         return
     if args.only == "fp8moe":
-        print(json.dumps(bench_fp8_quant_moe(dev, args.steps, args.warmup, args.int4_layers)))
+        print(json.dumps(bench_fp8_quant_moe(dev, args.steps, args.warmup, args.int4_layers, args.fp8_mode)))
         return
     if args.only == "int4":
         print(json.dumps(bench_int4_pack(dev, args.steps, args.warmup, args.int4_layers)))
@@ -1061,7 +1088,7 @@ def main():
 
     r = bench_north_star(dev, args.steps, args.warmup, args.int4_layers)
     kernels = {}
-    for key, name, profile, src in (("fp8", "fp8_block_quant_kernel<TORCH_DEVICE, per-tile descriptors>",
+    for key, name, profile, src in (("fp8", "fp8_block_quant_kernel<TORCH, per-tile descriptors>",
                                      "fp8_block_quant_qwen3_30b_a3b_state_dict.txt", "fp8_block_quant"),
                                     ("int4", "int4_pack_kernel<128, per-item descriptors>",
                                      "int4_pack_qwen3_30b_a3b_experts.txt", "int4_pack")):
@@ -1084,14 +1111,18 @@ def main():
         "config": {"workload": f"Qwen3-30B-A3B-shaped bf16 state dict ({r['layers']} layers x (128 experts x gate, up "
                                "[768,2048], down [2048,768] + q, k, v, o), N(0, 0.02) with rare x20 outliers), resident in "
                                f"HBM: block-FP8 128x128 quant of all {r['tensors_fp8']} linear weights (block_fp8 arithmetic "
-                               f"as torch evaluates it on GPU tensors), then INT4 sym group-128 pack of the {r['tensors_int4']} "
+                               f"as torch evaluates it on CPU tensors), then INT4 sym group-128 pack of the {r['tensors_int4']} "
                                "expert weights; one grouped launch each",
+                   "fp8_mode": r["fp8"]["mode"],
+                   "fp8_mode_meaning": "WQ_FP8_MODE_TORCH (0): amax clamped at bf16(1e-12), scale = f32(amax) / 448, q = f32(x) / scale, "
+                                       "both IEEE divisions - tools/convert_hf_to_fp8.py:41-75 on CPU tensors, what cpu_baseline computes",
                    "launches_per_step": 2, "bf16_GB_fp8": 2 * r["fp8"]["elements"] / 1e9,
                    "bf16_GB_int4": 2 * r["int4"]["elements"] / 1e9, "fp8_blocks": r["fp8"]["blocks"],
                    "parity_tensors_checked": r["parity_tensors_checked"]},
         "pct_hbm_peak": 100.0 * lower["frac"],
         "roofline": lower,
         "roofline_kernels": kernels,
+        "fp8_arithmetic_modes": r["fp8_modes"],
     }
     if not args.no_cpu:
         line["cpu_baseline"], line["cpu_baseline_legs"] = cpu_baselines(
@@ -1111,6 +1142,9 @@ def main():
         extras["delta_xor"] = bench_delta(dev, args.steps, args.warmup)
         extras["single_tensor_forms"] = bench_single_tensor_forms(dev, args.steps, args.warmup)
         extras["grouped_expert_weights"] = bench_grouped_experts(dev, args.steps, args.warmup)
+        # config 5's streaming leg: host-resident weights, PCIe-bound by construction (never part of `value`)
+        extras["host_resident_stream"] = bench_stream(dev, args.stream_buckets, args.stream_bucket_mib << 20,
+                                                      not args.stream_no_download)
         # the practical ceilings of 1:1, 2:1 and 4:1 read:write streams on this very box, measured in this very run
         cal = bench_copy(dev, args.steps, args.warmup)
         extras["copy_kernel_calibration"] = cal

@@ -114,3 +114,47 @@ def test_deepseek_v3_layer_dequant(cuda):
     x, s, y = xs[5], ss[5], outs[5]
     back = (y.float() / s.repeat_interleave(128, 0).repeat_interleave(128, 1)).to(E4M3)
     assert torch.equal(back.view(torch.uint8) & 0x7F, x.view(torch.uint8) & 0x7F)
+
+
+@pytest.mark.parametrize("mode", [0, 2])
+def test_qwen3_30b_a3b_state_dict_block_fp8(cuda, mode):
+    """The FP8 launch of the benchmark's headline step at its full size: all 18 624 linear weights of the
+    Qwen3-30B-A3B-shaped state dict (59.8 GB of bf16) through ONE launch, in the arithmetic the reference's own test
+    runs (mode 0) and the one its tool runs on GPU tensors (mode 2)."""
+    g = torch.Generator(device=cuda).manual_seed(3)
+    cg = torch.Generator().manual_seed(3 + mode)
+    layers, experts = 48, 128
+    ws, attention = [], []
+    for _ in range(layers):
+        gate, up = _gen((experts, 768, 2048), cuda, g, True), _gen((experts, 768, 2048), cuda, g, True)
+        down = _gen((experts, 2048, 768), cuda, g, True)
+        for e in range(experts):
+            ws += [gate[e], up[e], down[e]]
+        for sh in ((4096, 2048), (512, 2048), (512, 2048), (2048, 4096)):
+            attention.append(len(ws))
+            ws.append(_gen(sh, cuda, g, False))
+    plan = slime_amd.Fp8QuantPlan(ws, (128, 128), mode=mode)
+    outs = plan.run()
+    assert len(outs) == 18624 and plan.total_tiles == 1824768 and plan.bf16_bytes == 59793997824
+    # oracle on whole expert tensors and on stripes of attention weights; the bucket launch equals the single call
+    picks = torch.randint(0, len(ws), (20,), generator=cg).tolist() + [0, 1, 2, len(ws) - 5]
+    picks += [attention[i] for i in torch.randint(0, len(attention), (8,), generator=cg).tolist()] + [len(ws) - 1]
+    with slime_amd.torch_arithmetic("cpu" if mode == 0 else "device"):
+        for i in picks:
+            w, (q, s) = ws[i], outs[i]
+            for r0 in _stripe_rows(w.shape[0], cg, n=2):
+                qo, so = C.fp8_block_quant(w[r0:r0 + 128].cpu().contiguous(), (128, 128), mode)
+                assert torch.equal(q[r0:r0 + 128].cpu().view(torch.uint8), qo), (i, r0)
+                assert torch.equal(s[r0 // 128].cpu().view(torch.int32), so[0].view(torch.int32)), (i, r0)
+            q1, s1 = slime_amd.block_fp8(w, (128, 128))
+            assert torch.equal(q1.view(torch.uint8), q.view(torch.uint8)) and torch.equal(s1, s), i
+    # reconstruction bound over every tensor of three layers (first, middle, last)
+    per_layer = 3 * experts + 4
+    for layer in (0, layers // 2, layers - 1):
+        for i in range(layer * per_layer, (layer + 1) * per_layer):
+            w, (q, s) = ws[i], outs[i]
+            step = s.repeat_interleave(128, 0)[: w.shape[0]].repeat_interleave(128, 1)[:, : w.shape[1]] * 32
+            assert ((q.float() * step / 32 - w.float()).abs() <= step / 2 * 1.001).all(), i
+    # nothing outside the sampled tensors was left unwritten: every scale of the bucket is a positive finite number
+    scales = torch.cat([s.reshape(-1) for _, s in outs])
+    assert scales.numel() == plan.total_tiles and bool(((scales > 0) & torch.isfinite(scales)).all())
