@@ -334,6 +334,66 @@ def bench_cfg1(dev, steps, warmup, n_buffers=8):
     return out
 
 
+def bench_launch_sizes(dev, shapes=((2048, 2048), (4096, 4096), (8192, 4096), (8192, 8192), (16384, 8192), (32768, 8192),
+                                    (65536, 8192), (131072, 8192))):
+    """How the achieved fraction of the HBM peak grows with the size of ONE launch: a single bf16 matrix through
+    wq_fp8_block_quant and its codes through wq_fp8_block_dequant, launches back to back over enough distinct buffers
+    to stay out of the last-level cache.  Every launch pays a fixed cost - the gap between two kernels on a stream,
+    the first bytes' latency, the tail in which the last workgroups drain - that only multi-gigabyte launches
+    amortise; the sub-millisecond legs of this benchmark sit on this curve."""
+    import torch
+
+    import wq_testlib
+    from slime_amd import _lib
+
+    lib, tl = _lib.load(), wq_testlib.load()
+    st = _lib.stream_ptr(dev)
+    empty_b2b = _time_back_to_back(lambda: tl.wq_empty_launch(1024, 256, st), 64)
+    rows = []
+    for M, N in shapes:
+        touched = 2 * (3 * M * N)                                   # bytes of one quant + one dequant
+        n = max(2, min(16, (600 << 20) // touched + 1))             # >= 600 MB cycled, or two buffers of the largest
+        ws = [torch.empty((M, N), dtype=torch.bfloat16, device=dev).normal_(0, 0.02) for _ in range(n)]
+        qs = [torch.empty((M, N), dtype=torch.uint8, device=dev) for _ in ws]
+        ss = [torch.empty((M // 128, N // 128), dtype=torch.float32, device=dev) for _ in ws]
+        ys = [torch.empty((M, N), dtype=torch.bfloat16, device=dev) for _ in ws]
+        k = {"i": 0}
+
+        def quant():
+            k["i"] = (k["i"] + 1) % n
+            i = k["i"]
+            _lib.check(lib.wq_fp8_block_quant(ws[i].data_ptr(), M, N, N, 1, qs[i].data_ptr(), N, ss[i].data_ptr(), 128, 128,
+                                              HEADLINE_FP8_MODE, st), "quant")
+
+        def dequant():
+            k["i"] = (k["i"] + 1) % n
+            i = k["i"]
+            _lib.check(lib.wq_fp8_block_dequant(qs[i].data_ptr(), ss[i].data_ptr(), ys[i].data_ptr(), _lib.DTYPE_BF16, M, N,
+                                                128, _lib.DEQ_MODE_F32SCALE, st), "dequant")
+
+        for _ in range(n):
+            quant()
+        launches = max(8, min(64, (8 << 30) // touched))
+        q_us = _time_back_to_back(quant, launches)
+        d_us = _time_back_to_back(dequant, launches)
+        algo = 3 * M * N + 4 * (M // 128) * (N // 128)
+        rows.append({"shape": [M, N], "algorithmic_MB": algo / 1e6, "quant_us": q_us, "dequant_us": d_us,
+                     "quant_hbm_frac": algo / q_us / 1e3 / HBM_PEAK_GBS, "dequant_hbm_frac": algo / d_us / 1e3 / HBM_PEAK_GBS,
+                     # what is left of a launch when its bytes are charged at the rate of the largest launch of this sweep
+                     "buffers_cycled": n})
+        del ws, qs, ss, ys
+        torch.cuda.empty_cache()
+    best_q = max(r["quant_hbm_frac"] for r in rows)
+    best_d = max(r["dequant_hbm_frac"] for r in rows)
+    for r in rows:
+        r["quant_fixed_us"] = r["quant_us"] - r["algorithmic_MB"] / (best_q * HBM_PEAK_GBS) * 1e3
+        r["dequant_fixed_us"] = r["dequant_us"] - r["algorithmic_MB"] / (best_d * HBM_PEAK_GBS) * 1e3
+    return {"workload": "one bf16 [M, N] matrix per launch, block-FP8 quant (headline arithmetic) and dequant, launches back to "
+                        "back between one pair of events, cold buffers; *_fixed_us = time of a launch beyond its bytes at the "
+                        "rate of the best launch of the sweep",
+            "empty_launch_us_back_to_back": empty_b2b, "rows": rows}
+
+
 def bench_fp8_quant_moe(dev, steps, warmup, layers, mode=HEADLINE_FP8_MODE):
     """Block-FP8 quant of every linear weight of a Qwen3-30B-A3B-shaped state dict (48 layers: 128 experts x
     gate/up [768,2048], down [2048,768]; attention q [4096,2048], k/v [512,2048], o [2048,4096]), one grouped launch."""
@@ -486,7 +546,22 @@ def bench_bucket(dev, steps, warmup, layers):
     expert_el = sum(t.numel() for n, t in quantised if ".experts." in n)
     passed = sum(t.numel() * t.element_size() for _, cv in whole for n, t in cv if ".experts." not in n)
     algo4 = int(expert_el * 2.515625) + 2 * passed
-    del named4, conv4
+    del named4
+    # the same conversion as ONE bucket: one launch instead of 48, so one start-up and one tail instead of 48
+    conv4.time_kernels = False
+
+    def int4_one_bucket():
+        state["out"] = None
+        state["out"] = conv4.convert(whole, bucket_id="all")
+
+    wall4a, _, _ = _time_launches(int4_one_bucket, steps, warmup)
+    conv4.time_kernels = True
+    for _ in range(steps):
+        int4_one_bucket()
+    torch.cuda.synchronize()
+    ev4a = conv4.kernel_ms() / steps
+    launches4a = state["out"].launches
+    del conv4
     state["out"] = None
     # the loop this replaces, on this build's own per-tensor kernels (so the difference is launches and copies, not
     # arithmetic): quantize_params per Megatron parameter, then the flatten copy; two layers, scaled to all of them
@@ -515,6 +590,9 @@ def bench_bucket(dev, steps, warmup, layers):
                                              "weights packed (sym, group 128), attention / norms / router copied through",
                                      "launches_per_sync": launches4, "ms_per_sync_kernels": ev4, "ms_per_sync_wall": wall4,
                                      "hbm_frac": algo4 / ev4 / 1e6 / HBM_PEAK_GBS, "bf16_GBps": 2 * expert_el / ev4 / 1e6},
+           "int4_one_bucket": {"what": "the INT4 branch with the whole state dict as one bucket",
+                               "launches_per_sync": launches4a, "ms_per_sync_kernels": ev4a, "ms_per_sync_wall": wall4a,
+                               "hbm_frac": algo4 / ev4a / 1e6 / HBM_PEAK_GBS, "bf16_GBps": 2 * expert_el / ev4a / 1e6},
            "per_parameter_loop_then_flatten": {
                "what": "quantize_params once per Megatron parameter (one cached-table launch each) followed by the flatten "
                        "copy into one buffer, per layer bucket - the shape of the reference's loop, on this build's kernels",
@@ -1021,7 +1099,7 @@ def main():
     ap.add_argument("--dequant-experts", type=int, default=256)
     ap.add_argument("--no-extras", action="store_true", help="headline step only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
-    ap.add_argument("--only", choices=["fp8", "cfg1", "bucket", "fp8moe", "int4", "dequant", "int4deq", "ste", "delta", "forms", "experts", "copy", "stream", "hashes"], default=None,
+    ap.add_argument("--only", choices=["fp8", "cfg1", "bucket", "fp8moe", "int4", "dequant", "int4deq", "ste", "delta", "forms", "experts", "copy", "stream", "sizes", "hashes"], default=None,
                     help="run just one of the other legs and print its record: a kernel for profiling, the plain copy "
                          "kernel that hardware counters are calibrated against, or the host-resident streaming run "
                          "(64 x 1 GiB buckets, PCIe-bound)")
@@ -1080,6 +1158,9 @@ def main():
         return
     if args.only == "copy":
         print(json.dumps(bench_copy(dev, args.steps, args.warmup)))
+        return
+    if args.only == "sizes":
+        print(json.dumps(bench_launch_sizes(dev)))
         return
     if args.only == "stream":
         print(json.dumps(bench_stream(dev, args.stream_buckets, args.stream_bucket_mib << 20,
@@ -1142,6 +1223,7 @@ def main():
         extras["delta_xor"] = bench_delta(dev, args.steps, args.warmup)
         extras["single_tensor_forms"] = bench_single_tensor_forms(dev, args.steps, args.warmup)
         extras["grouped_expert_weights"] = bench_grouped_experts(dev, args.steps, args.warmup)
+        extras["launch_size_curve"] = bench_launch_sizes(dev)
         # config 5's streaming leg: host-resident weights, PCIe-bound by construction (never part of `value`)
         extras["host_resident_stream"] = bench_stream(dev, args.stream_buckets, args.stream_bucket_mib << 20,
                                                       not args.stream_no_download)

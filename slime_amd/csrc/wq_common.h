@@ -403,10 +403,14 @@ __device__ __forceinline__ float rcp_refined(float s)
 }
 
 // acc's byte BYTE <- low byte of (q + magic): v_add_f32_sdwa with the other bytes of the destination preserved.
+// `s_nop 0`: on this family a VALU instruction that writes part of a register (dst_sel other than DWORD) needs one wait
+// state before a VALU instruction that reads the register - the next add into the same word (UNUSED_PRESERVE reads the
+// destination) or the final shift-or.  The compiler's hazard recogniser does not look inside inline assembly, so the
+// helper carries the wait state itself, like the DPP helpers above.
 #define WQ_ADD_TO_BYTE(BYTE)                                                                                        \
     __device__ __forceinline__ void add_magic_to_byte##BYTE(uint32_t& acc, float q, float magic)                    \
     {                                                                                                               \
-        asm("v_add_f32_sdwa %0, %1, %2 dst_sel:BYTE_" #BYTE " dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD" \
+        asm("v_add_f32_sdwa %0, %1, %2 dst_sel:BYTE_" #BYTE " dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD\n\ts_nop 0" \
             : "+v"(acc) : "v"(q), "v"(magic));                                                                      \
     }
 WQ_ADD_TO_BYTE(1)

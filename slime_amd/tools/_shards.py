@@ -51,6 +51,25 @@ def list_shards(input_path: str) -> list:
     return sorted(f for f in os.listdir(input_path) if f.endswith(".safetensors"))
 
 
+def locate_tensors(checkpoint_dir: str) -> dict:
+    """{tensor name: shard file name} of a HF checkpoint directory.  ``model.safetensors.index.json`` decides when it
+    exists; otherwise every shard's header is read (in sorted order, so a name stored twice resolves to the last
+    shard).  FileNotFoundError when the directory holds neither."""
+    index = os.path.join(checkpoint_dir, "model.safetensors.index.json")
+    if os.path.isfile(index):
+        with open(index) as f:
+            return dict(json.load(f)["weight_map"])
+    shards = list_shards(checkpoint_dir)
+    if not shards:
+        raise FileNotFoundError(f"No safetensors checkpoint found in {checkpoint_dir}")
+    where = {}
+    for shard in shards:
+        with safe_open(os.path.join(checkpoint_dir, shard), framework="pt", device="cpu") as f:
+            for key in f.keys():
+                where[key] = shard
+    return where
+
+
 class ConversionResult:
     """Thread-safe accumulator of the output index.  ``param_count`` reproduces the reference's quirk: it adds
     ``len(tensor)`` - the first dimension - of every output tensor (tools/convert_hf_to_fp8.py:110-114), and

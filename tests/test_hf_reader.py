@@ -49,9 +49,28 @@ def test_reader_dequantizes_block_scaled_fp8(tmp_path, cuda):
 
     loaded = SafetensorReader(tmp_path).get_tensor("weight")
 
-    assert loaded.dtype == torch.bfloat16
-    assert torch.equal(loaded.cpu(), weight.to(torch.bfloat16) * 2)
-    assert SafetensorReader(tmp_path, device="cpu").get_tensor("weight").device.type == "cpu"
+    assert loaded.dtype == torch.bfloat16 and loaded.device.type == "cpu"          # host tensors, like the reference's reader
+    assert torch.equal(loaded, weight.to(torch.bfloat16) * 2)
+    on_gpu = SafetensorReader(tmp_path, device="cuda").get_tensor("weight")
+    assert on_gpu.is_cuda and torch.equal(on_gpu.cpu(), loaded)
+
+
+@pytest.mark.gpu
+def test_reader_partly_quantised_checkpoint_and_other_one_byte_dtypes(tmp_path, cuda):
+    """modules_to_not_convert leaves bf16 weights next to FP8 ones: both come back on the host and can be concatenated.
+    A one-byte tensor that is not float8_e4m3fn is not reinterpreted: without a scale it is returned as stored, with a
+    scale it is refused."""
+    codes = I.fp8_codes(128, 256, seed=3)
+    scale = I.log_uniform_scales(1, 2, seed=4)
+    save_file({"q.weight": codes.view(E4M3), "q.weight_scale_inv": scale, "k.weight": torch.ones(64, 256, dtype=torch.bfloat16),
+               "flags": torch.arange(5, dtype=torch.int8), "odd.weight": torch.zeros(128, 128, dtype=torch.int8),
+               "odd.weight_scale_inv": torch.ones(1, 1)}, tmp_path / "model.safetensors")
+    reader = SafetensorReader(tmp_path)
+    qk = torch.cat([reader.get_tensor("q.weight"), reader.get_tensor("k.weight")], dim=0)
+    assert qk.shape == (192, 256) and I.same_bits(qk[:128], C.fp8_block_dequant(codes, scale, 128, 1))
+    assert reader.get_tensor("flags").dtype == torch.int8
+    with pytest.raises(TypeError, match="float8_e4m3fn"):
+        reader.get_tensor("odd.weight")
 
 
 @pytest.mark.gpu
@@ -67,7 +86,7 @@ def test_reader_ragged_shapes_and_scale_in_another_shard(tmp_path, cuda):
     first["l0.norm.weight"] = torch.ones(8, dtype=torch.bfloat16)
     save_file(first, tmp_path / "model-00001-of-00002.safetensors")
     save_file(second, tmp_path / "model-00002-of-00002.safetensors")
-    reader = SafetensorReader(tmp_path)
+    reader = SafetensorReader(tmp_path, device="cuda")
     for name, w in want.items():
         got = reader.get_tensor(name)
         assert got.is_cuda and got.dtype == torch.bfloat16 and got.shape == w.shape and I.same_bits(got.cpu(), w), name

@@ -394,6 +394,20 @@ def test_ue8m0_scale_is_the_smallest_power_of_two_not_below_amax_over_448_for_ev
     assert int(exact.sum()) > 100
 
 
+def test_ue8m0_literal_log2_ceil_pow_expression_for_every_bf16_amax():
+    """sglang evaluates the scale as ``2 ** ceil(log2(amax / 448))`` in fp32; the C oracle (and the kernel) round the
+    exponent up by bit manipulation.  The literal torch expression, evaluated here on all 32 639 finite non-zero bf16
+    amax values, gives the oracle's scale bits for every one of them - fp32 log2 never lands on the wrong side of an
+    integer for these inputs."""
+    bits = torch.arange(1, 0x7F80, dtype=torch.int32)
+    amax = bits.to(torch.int16).view(torch.bfloat16).float().clamp(1e-4)
+    literal = torch.pow(2.0, torch.ceil(torch.log2(amax / 448.0)))
+    w = torch.zeros(128, 128 * bits.numel(), dtype=torch.bfloat16)
+    w[5, 3::128] = -bits.to(torch.int16).view(torch.bfloat16)
+    _, so = C.fp8_block_quant(w, (128, 128), 3)
+    assert torch.equal(literal.view(torch.int32), so.view(-1).view(torch.int32))
+
+
 def test_ue8m0_codes_are_one_rounding_of_an_exact_scaling():
     w = I.zero_blocks(I.weights(300, 520, seed=3), 0.2, seed=1)
     w[200:, 300:] = I.subnormal_block(100, 220, seed=2)
