@@ -134,6 +134,13 @@ __global__ __launch_bounds__(256) void int4_pack_kernel(const Int4PackArgs a, co
     const char* xb = (const char*)d.x + base * (16 * L);
     char* pb = (char*)d.packed + base * (4 * L);
     char* sb = (char*)d.scale + base * 2;
+    // Where the item's words do not start on a 128-byte line - a bucket packs its tensors back to back, and every INT4
+    // weight is followed by its 8-byte weight_shape - each wavefront's 256-byte store would begin and end in the middle of
+    // a line, and such streams lose 7 points of bandwidth on this part (81 -> 74 % of HBM peak on 16 layers of experts).
+    // Those items collect their words in LDS and write them out as whole lines: 16-byte stores, a wavefront per KiB
+    // starting on a line boundary, single words only before the first and after the last boundary (80 %).
+    __shared__ uint32_t stage[kGroupsPerWg * L];
+    const bool staged = GROUPED == 2 && ((uintptr_t)pb & 127u) != 0;          // uniform per workgroup
 
     // Rolling window: at most kPackWindow 16-byte loads per lane are in flight; the load of step i + window
     // is issued just before step i is processed (with the window as long as the item, all of them are issued up front).
@@ -158,10 +165,26 @@ __global__ __launch_bounds__(256) void int4_pack_kernel(const Int4PackArgs a, co
         const uint32_t sb_bits = bf16_bits_hw(scale);
         if (sb_bits >= kLiteralChainScaleBits) w = pack8_literal(xs, scale, u2f(sb_bits << 16));
         if (g < rem) {
-            stg_nt<uint32_t>(pb + (uint32_t)((g * L + ll) * 4), w);
+            if (staged) stage[g * L + ll] = w;
+            else stg_nt<uint32_t>(pb + (uint32_t)((g * L + ll) * 4), w);
             if (ll == 0) stg<uint16_t>(sb + (uint32_t)(g * 2), (uint16_t)sb_bits);
         }
         __builtin_amdgcn_sched_barrier(0);
+    }
+    if (staged) {
+        __syncthreads();
+        const int n_words = rem * L;
+        const int head = min((int)(((128u - ((uintptr_t)pb & 127u)) & 127u) >> 2), n_words);   // words before the first line
+        const int pieces = (n_words - head) >> 2;                                              // whole 16-byte pieces from there
+        const int t = threadIdx.x;
+        if (t < head) stg_nt<uint32_t>(pb + (uint32_t)(t * 4), stage[t]);
+        for (int p = t; p < pieces; p += 256) {
+            const int w0 = head + 4 * p;
+            const u32x4 o = {stage[w0], stage[w0 + 1], stage[w0 + 2], stage[w0 + 3]};
+            stg_nt<u32x4>(pb + (uint32_t)(w0 * 4), o);
+        }
+        const int tail = head + 4 * pieces + t;
+        if (tail < n_words) stg_nt<uint32_t>(pb + (uint32_t)(tail * 4), stage[tail]);
     }
 }
 

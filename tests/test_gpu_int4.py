@@ -490,3 +490,39 @@ def test_int4_dequant_plan(cuda):
         slime_amd.Int4DequantPlan([trip[0][0].to(cuda)], [trip[0][1].to(cuda)], [shapes[0]], 96)
     with pytest.raises(ValueError):
         slime_amd.Int4DequantPlan([trip[0][0].to(cuda)], [trip[0][1].to(cuda)], [(96, 512)], 32)
+
+
+@pytest.mark.parametrize("group", [128, 64, 32])
+def test_bucket_form_with_destinations_at_every_word_offset_of_a_line(cuda, group):
+    """A bucket packs its outputs back to back, so the packed words of a tensor start wherever the previous tensor
+    ended.  Items whose words do not start on a 128-byte line are collected in LDS and written out as whole lines:
+    every 4-byte offset inside a line, with full, short and one-group items, against the oracle - and the bytes around
+    every output must stay untouched."""
+    from slime_amd import _lib
+    from slime_amd.int4 import item_table
+
+    shapes = [(64, 128), (1, 128), (63, 128), (65, 128), (3, 1024), (130, 256), (16, 2048), (7, 384)]
+    ws = [I.weights(*sh, seed=900 + i) for i, sh in enumerate(shapes)]
+    wg = [w.to(cuda) for w in ws]
+    for shift in range(0, 128, 4):
+        rows, places, off = [], [], 128 + shift
+        for w in wg:
+            M, N = w.shape
+            p0 = off
+            s0 = p0 + M * N // 2
+            off = -(-(s0 + M * N // group * 2) // 4) * 4 + 8   # the weight_shape entry of a bucket: the next tensor lands 8 bytes further
+            rows.append([w.data_ptr(), p0, s0, M * N // group])
+            places.append((p0, s0, M, N))
+        table, _, _ = item_table(rows, group)
+        out = torch.full((off + 256,), 0xA5, dtype=torch.uint8, device=cuda)
+        rc = _lib.load().wq_int4_bucket_convert(table.contiguous().to(cuda).data_ptr(), table.shape[0], out.data_ptr(), group,
+                                                _lib.stream_ptr(cuda))
+        _lib.check(rc, "bucket form")
+        host = out.cpu()
+        written = torch.zeros(host.numel(), dtype=torch.bool)
+        for w, (p0, s0, M, N) in zip(ws, places):
+            po, so, _ = C.int4_pack_layer(w, group, True)
+            assert torch.equal(host[p0:p0 + M * N // 2].clone().view(torch.int32).view(M, N // 8), po), (shift, M, N)
+            assert torch.equal(host[s0:s0 + M * N // group * 2].clone().view(torch.int16), so.view(torch.int16).reshape(-1)), (shift, M, N)
+            written[p0:s0 + M * N // group * 2] = True
+        assert bool((host[~written] == 0xA5).all()), shift
