@@ -93,6 +93,24 @@ __device__ __forceinline__ uint32_t pack8_literal(const float (&x)[8], float sca
     return w;
 }
 
+// Writes n_words words collected in LDS to dst (4-byte aligned, not on a 128-byte line) as whole lines: single words up to
+// the first line boundary and after the last 16-byte piece, 16-byte stores in between - a wavefront per KiB, starting on a
+// line.  All threads of the workgroup call it after a barrier.
+__device__ __forceinline__ void store_words_by_lines(char* dst, const uint32_t* stage, int n_words)
+{
+    const int head = min((int)(((128u - ((uintptr_t)dst & 127u)) & 127u) >> 2), n_words);   // words before the first line
+    const int pieces = (n_words - head) >> 2;                                               // whole 16-byte pieces from there
+    const int t = threadIdx.x;
+    if (t < head) stg_nt<uint32_t>(dst + (uint32_t)(t * 4), stage[t]);
+    for (int p = t; p < pieces; p += 256) {
+        const int w0 = head + 4 * p;
+        const u32x4 o = {stage[w0], stage[w0 + 1], stage[w0 + 2], stage[w0 + 3]};
+        stg_nt<u32x4>(dst + (uint32_t)(w0 * 4), o);
+    }
+    const int tail = head + 4 * pieces + t;
+    if (tail < n_words) stg_nt<uint32_t>(dst + (uint32_t)(tail * 4), stage[tail]);
+}
+
 // Contiguous tensors only: group g of the tensor starts at x + g*G, its packed words at
 // packed + g*L, its scale at scale[g].
 // GROUPED: 0 = one tensor in the kernel arguments, 1 = descriptor array + prefix sums (the owner of a work item is
@@ -173,18 +191,7 @@ __global__ __launch_bounds__(256) void int4_pack_kernel(const Int4PackArgs a, co
     }
     if (staged) {
         __syncthreads();
-        const int n_words = rem * L;
-        const int head = min((int)(((128u - ((uintptr_t)pb & 127u)) & 127u) >> 2), n_words);   // words before the first line
-        const int pieces = (n_words - head) >> 2;                                              // whole 16-byte pieces from there
-        const int t = threadIdx.x;
-        if (t < head) stg_nt<uint32_t>(pb + (uint32_t)(t * 4), stage[t]);
-        for (int p = t; p < pieces; p += 256) {
-            const int w0 = head + 4 * p;
-            const u32x4 o = {stage[w0], stage[w0 + 1], stage[w0 + 2], stage[w0 + 3]};
-            stg_nt<u32x4>(pb + (uint32_t)(w0 * 4), o);
-        }
-        const int tail = head + 4 * pieces + t;
-        if (tail < n_words) stg_nt<uint32_t>(pb + (uint32_t)(tail * 4), stage[tail]);
+        store_words_by_lines(pb, stage, rem * L);
     }
 }
 
@@ -450,6 +457,9 @@ __global__ __launch_bounds__(256) void int4_pack_asym_kernel(const uint16_t* __r
             return;
         }
     }
+    // items whose words do not start on a 128-byte line: collected in LDS, written as whole lines (see int4_pack_kernel)
+    __shared__ uint32_t stage[ITEMS ? kFakeGroupsPerWg * L : 1];
+    const bool staged = ITEMS && ((uintptr_t)packed & 127u) != 0;          // uniform per workgroup
     u32x4 v[STEPS];
 #pragma unroll
     for (int i = 0; i < STEPS; ++i) {
@@ -501,12 +511,17 @@ __global__ __launch_bounds__(256) void int4_pack_asym_kernel(const uint16_t* __r
             for (int j = 0; j < 8; ++j) word += code_literal_asym(q[j], zero, sb) << (4 * j);
         }
         if (g < n_groups) {
-            stg_nt<uint32_t>(packed + g * L + ll, word);
+            if (staged) stage[(int)g * L + ll] = word;
+            else stg_nt<uint32_t>(packed + g * L + ll, word);
             if (ll == 0) {
                 stg<uint16_t>(scale_out + g, (uint16_t)sb_bits);
                 stg<uint16_t>(zero_out + g, (uint16_t)f32_to_bf16_bits(zero));
             }
         }
+    }
+    if (staged) {
+        __syncthreads();
+        store_words_by_lines((char*)packed, stage, (int)min(n_groups, (int64_t)kFakeGroupsPerWg) * L);
     }
 }
 

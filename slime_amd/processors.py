@@ -162,8 +162,8 @@ def _group_cast(weights, block_size):
             M, N = w.shape
             tm, tn = ceildiv(M, bm), ceildiv(N, bn)
             q0 = off
-            s0 = (q0 + M * N + 15) // 16 * 16
-            off = (s0 + 4 * tm * tn + 15) // 16 * 16
+            s0 = (q0 + M * N + 127) // 128 * 128          # codes of every tensor start on a 128-byte line
+            off = (s0 + 4 * tm * tn + 127) // 128 * 128
             d.x, d.y, d.s, d.M, d.N, d.sx_m, d.sx_n, d.sy_m = w.data_ptr(), q0, s0, M, N, w.stride(0), w.stride(1), N
             layout.append((q0, M, N, s0, tm, tn))
         flat = torch.empty(off, dtype=torch.uint8, device=device)

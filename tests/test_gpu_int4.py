@@ -526,3 +526,43 @@ def test_bucket_form_with_destinations_at_every_word_offset_of_a_line(cuda, grou
             assert torch.equal(host[s0:s0 + M * N // group * 2].clone().view(torch.int16), so.view(torch.int16).reshape(-1)), (shift, M, N)
             written[p0:s0 + M * N // group * 2] = True
         assert bool((host[~written] == 0xA5).all()), shift
+
+
+def test_asym_bucket_form_with_destinations_off_a_line(cuda):
+    """The asymmetric items kernel with packed words starting at every fourth word offset of a 128-byte line."""
+    from slime_amd import _lib
+    from slime_amd.int4 import item_table
+
+    group = 128
+    shapes = [(64, 128), (8, 128), (72, 256), (16, 2048), (136, 384)]
+    ws = [I.weights(*sh, seed=950 + i) + 0.01 for i, sh in enumerate(shapes)]
+    wg = [w.to(cuda) for w in ws]
+    for shift in range(0, 128, 16):
+        rows, places, off, zoff = [], [], 128 + shift + 4, 0
+        for w in wg:
+            M, N = w.shape
+            p0 = off
+            s0 = p0 + M * N // 2
+            off = -(-(s0 + M * N // group * 2) // 4) * 4 + 8
+            rows.append([w.data_ptr(), p0, s0, zoff, M * N // group])
+            places.append((p0, s0, zoff, M, N))
+            zoff += (2 * M * N // group + 15) // 16 * 16
+        full = torch.tensor(rows, dtype=torch.int64)
+        table4, owner, local = item_table(full[:, [0, 1, 2, 4]], group)
+        zcol = full[owner, 3] + local * (_lib.INT4_GROUPS_PER_WG * 2)
+        table = torch.cat([table4[:, :3], zcol.unsqueeze(1), table4[:, 3:]], dim=1).contiguous().to(cuda)
+        out = torch.full((off + 256,), 0x5A, dtype=torch.uint8, device=cuda)
+        zero = torch.zeros(zoff + 16, dtype=torch.uint8, device=cuda)
+        rc = _lib.load().wq_int4_group_quant_pack_asym_items(table.data_ptr(), table.shape[0], out.data_ptr(), zero.data_ptr(),
+                                                             group, _lib.stream_ptr(cuda))
+        _lib.check(rc, "asym items")
+        host, zhost = out.cpu(), zero.cpu()
+        written = torch.zeros(host.numel(), dtype=torch.bool)
+        for w, (p0, s0, z0, M, N) in zip(ws, places):
+            po, so, _ = C.int4_pack_layer(w, group, False)
+            _, _, zo = C.int4_fake_quant(w, (1, group), False)
+            assert torch.equal(host[p0:p0 + M * N // 2].clone().view(torch.int32).view(M, N // 8), po), (shift, M, N)
+            assert torch.equal(host[s0:s0 + M * N // group * 2].clone().view(torch.int16), so.view(torch.int16).reshape(-1)), (shift, M, N)
+            assert torch.equal(zhost[z0:z0 + M * N // group * 2].clone().view(torch.int16), zo.view(torch.int16).reshape(-1)), (shift, M, N)
+            written[p0:s0 + M * N // group * 2] = True
+        assert bool((host[~written] == 0x5A).all()), shift
