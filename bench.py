@@ -268,7 +268,7 @@ def bench_cfg1(dev, steps, warmup, n_buffers=8):
     qs = [torch.empty((M, N), dtype=torch.uint8, device=dev) for _ in ws]
     ss = [torch.empty((M // 128, N // 128), dtype=torch.float32, device=dev) for _ in ws]
     ys = [torch.empty((M, N), dtype=torch.bfloat16, device=dev) for _ in ws]
-    mode = slime_amd.arith.fp8_torch_mode()
+    mode = HEADLINE_FP8_MODE
     st = _lib.stream_ptr(dev)
     state = {"i": 0}
 
