@@ -26,10 +26,9 @@ converted by the per-parameter loop and concatenated with ``torch.cat``, as the 
 
 from __future__ import annotations
 
-import dataclasses
 import json
 from collections import OrderedDict
-from typing import Sequence
+from typing import NamedTuple, Sequence
 
 import numpy as np
 import torch
@@ -44,10 +43,10 @@ _COPY = _lib.BUCKET_COPY_BYTES
 _ELEMENT_SIZE: dict = {}
 
 
-@dataclasses.dataclass(frozen=True)
-class FlattenedTensorMetadata:
+class FlattenedTensorMetadata(NamedTuple):
     """One entry of ``FlattenedTensorBucket.get_metadata()``: the tensor is
-    ``flattened_tensor[start_idx:end_idx].view(dtype).reshape(shape)``; ``numel`` counts bytes."""
+    ``flattened_tensor[start_idx:end_idx].view(dtype).reshape(shape)``; ``numel`` counts bytes.  (An immutable record
+    with the fields of sglang's dataclass; a named tuple because a bucket builds tens of thousands of them.)"""
     name: str
     shape: torch.Size
     dtype: torch.dtype
@@ -229,7 +228,7 @@ class BucketConverter:
             nbytes = esz
             for d in shape:
                 nbytes *= int(d)
-            meta.append(FlattenedTensorMetadata(name, torch.Size(shape), dtype, off, off + nbytes, nbytes))
+            meta.append(FlattenedTensorMetadata(name, shape if type(shape) is torch.Size else torch.Size(shape), dtype, off, off + nbytes, nbytes))
             start = off
             off += nbytes
             return start, nbytes
