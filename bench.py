@@ -610,6 +610,57 @@ def bench_bucket(dev, steps, warmup, layers):
     return out
 
 
+def bench_bucket_off_lines(dev, steps, warmup, layers=6):
+    """A DeepSeek-V3-shaped (MLA) FP8 weight-sync bucket: kv_a_proj_with_mqa [576, 7168] has 280 tiles, so its 1120 bytes
+    of scales leave every tensor packed after it 96 bytes off the 128-byte lines of the flat buffer.  Those tensors take the
+    converter's second launch (plain stores); the record says what the bucket costs and checks a tensor from each launch."""
+    import torch
+
+    from oracle import c_oracle
+    from slime_amd import bucket as B
+
+    cfg = {"quant_method": "fp8", "fmt": "e4m3", "activation_scheme": "dynamic", "weight_block_size": [128, 128]}
+    params = []
+    for layer in range(layers):
+        L, hf = f"module.module.decoder.layers.{layer}.", f"model.layers.{layer}."
+        params += [(L + "self_attention.linear_q_down_proj.weight", [(hf + "self_attn.q_a_proj.weight", _gen_bf16((1536, 7168), dev))]),
+                   (L + "self_attention.linear_q_up_proj.weight", [(hf + "self_attn.q_b_proj.weight", _gen_bf16((24576, 1536), dev))]),
+                   (L + "self_attention.linear_kv_down_proj.weight", [(hf + "self_attn.kv_a_proj_with_mqa.weight", _gen_bf16((576, 7168), dev))]),
+                   (L + "self_attention.linear_kv_up_proj.weight", [(hf + "self_attn.kv_b_proj.weight", _gen_bf16((32768, 512), dev))]),
+                   (L + "self_attention.linear_proj.weight", [(hf + "self_attn.o_proj.weight", _gen_bf16((7168, 16384), dev))])]
+        for e in range(16):
+            params.append((L + f"mlp.experts.linear_fc2.weight{e}",
+                           [(hf + f"mlp.experts.{e}.down_proj.weight", _gen_bf16((7168, 2048), dev, outliers=True))]))
+    tensors = [(n, t) for _, cv in params for n, t in cv]
+    elements = sum(t.numel() for _, t in tensors)
+    algo = 3 * elements + 4 * sum((-(-t.shape[0] // 128)) * (-(-t.shape[1] // 128)) for _, t in tensors)
+    conv = B.BucketConverter(None, cfg)
+    state = {}
+
+    def run():
+        state["out"] = None
+        state["out"] = conv.convert(params, bucket_id="mla")
+
+    wall, _, _ = _time_launches(run, steps, warmup)
+    conv.time_kernels = True
+    for _ in range(steps):
+        run()
+    torch.cuda.synchronize()
+    ev = conv.kernel_ms() / steps
+    out = state["out"]
+    off = sum(1 for m in out.metadata if m.dtype == torch.float8_e4m3fn and m.start_idx % 64)
+    named = dict(out.reconstruct_tensors())
+    for n, t in (tensors[0], tensors[3], tensors[-1]):                 # before and after the tensor that shifts the rest
+        qo, so = c_oracle.fp8_block_quant(t.cpu().contiguous(), (128, 128), 1)
+        assert torch.equal(named[n].cpu().view(torch.uint8), qo), f"off-line bucket: parity failure on {n}"
+        assert torch.equal(named[n.replace(".weight", ".weight_scale_inv")].cpu().view(torch.int32), so.view(torch.int32))
+    return {"workload": f"{layers} layers x (q_a [1536,7168], q_b [24576,1536], kv_a [576,7168], kv_b [32768,512], o [7168,16384], 16 experts' "
+                        "down [7168,2048]) bf16 -> block-FP8 through BucketConverter, packed back to back",
+            "tensors": len(tensors), "tensors_off_the_lines": off, "launches_per_sync": out.launches, "ms_per_sync_kernels": ev,
+            "ms_per_sync_wall": wall, "hbm_frac": algo / ev / 1e6 / HBM_PEAK_GBS, "bf16_GBps": 2 * elements / ev / 1e6,
+            "parity_tensors_checked": 3}
+
+
 def bench_grouped_experts(dev, steps, warmup, experts=128):
     """The stacked expert weights of one MoE layer's grouped linears (fc1 = gate+up [1536, 2048], fc2 [2048, 768]) as the
     FP8-aligned MoE forward quantises them on every step: one launch per grouped linear against the loop it replaces."""
@@ -1105,7 +1156,7 @@ def main():
     ap.add_argument("--dequant-experts", type=int, default=256)
     ap.add_argument("--no-extras", action="store_true", help="headline step only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
-    ap.add_argument("--only", choices=["fp8", "cfg1", "bucket", "fp8moe", "int4", "dequant", "int4deq", "ste", "delta", "forms", "experts", "copy", "stream", "sizes", "hashes"], default=None,
+    ap.add_argument("--only", choices=["fp8", "cfg1", "bucket", "fp8moe", "int4", "dequant", "int4deq", "ste", "delta", "forms", "experts", "copy", "stream", "sizes", "mla", "hashes"], default=None,
                     help="run just one of the other legs and print its record: a kernel for profiling, the plain copy "
                          "kernel that hardware counters are calibrated against, or the host-resident streaming run "
                          "(64 x 1 GiB buckets, PCIe-bound)")
@@ -1165,6 +1216,9 @@ def main():
     if args.only == "copy":
         print(json.dumps(bench_copy(dev, args.steps, args.warmup)))
         return
+    if args.only == "mla":
+        print(json.dumps(bench_bucket_off_lines(dev, args.steps, args.warmup)))
+        return
     if args.only == "sizes":
         print(json.dumps(bench_launch_sizes(dev)))
         return
@@ -1223,6 +1277,7 @@ def main():
             extras["weight_sync_bucket"] = bench_bucket(dev, args.steps, args.warmup, args.int4_layers)
         extras["delta_xor"] = bench_delta(dev, args.steps, args.warmup)
         extras["single_tensor_forms"] = bench_single_tensor_forms(dev, args.steps, args.warmup)
+        extras["weight_sync_bucket_off_lines"] = bench_bucket_off_lines(dev, args.steps, args.warmup)
         extras["grouped_expert_weights"] = bench_grouped_experts(dev, args.steps, args.warmup)
         extras["launch_size_curve"] = bench_launch_sizes(dev)
         # config 5's streaming leg: host-resident weights, PCIe-bound by construction (never part of `value`)

@@ -133,6 +133,15 @@ int wq_fp8_block_quant_tiles(const wq_fp8_quant_desc *tiles, int64_t n_tiles, in
 int wq_fp8_bucket_convert(const wq_fp8_quant_desc *items, int64_t n_items, void *out_base, int bm, int bn, int mode,
                           void *stream);
 
+/* wq_fp8_bucket_convert for items whose code rows do NOT start on 64-byte boundaries (out_base + y or sy_m not a multiple of
+ * 64): same items, same results, plain instead of streaming stores, so that the two tiles that share every 128-byte line of
+ * such a tensor have their halves merged in the L2 (65-70 % of HBM peak wherever the rows start, where the streaming form
+ * falls to 44-55 %; for aligned rows the streaming form's 80 % is 8-10 points ahead).  A caller that packs tensors back to
+ * back, as FlattenedTensorBucket does (update_weight_from_tensor.py:30-48), knows every offset when it builds its tables and
+ * puts the items of each kind into the launch made for it. */
+int wq_fp8_bucket_convert_rows_off_lines(const wq_fp8_quant_desc *items, int64_t n_items, void *out_base, int bm, int bn,
+                                         int mode, void *stream);
+
 /* The bucket tables above hold the ADDRESS of every item's input, while the inputs of a weight-sync bucket are fresh
  * tensors on every sync as soon as the model is sharded: all_gather_param fills torch.empty_like partitions and
  * concatenates them (slime/backends/megatron_utils/update_weight/common.py:97,120) before

@@ -39,6 +39,7 @@ SIGNATURES = {
     "wq_fp8_block_quant_tiles": [_vp, _i64, _int, _int, _int, _vp],
     "wq_fp8_block_quant_few": [_vp, _int, _vp, _int, _int, _int, _vp],
     "wq_fp8_bucket_convert": [_vp, _i64, _vp, _int, _int, _int, _vp],
+    "wq_fp8_bucket_convert_rows_off_lines": [_vp, _i64, _vp, _int, _int, _int, _vp],
     "wq_int4_bucket_convert": [_vp, _i64, _vp, _int, _vp],
     "wq_bucket_resolve_items": [_vp, _vp, _vp, _i64, _int, _vp, _vp],
     "wq_fp8_block_quant_any": [_vp, _int, _i64, _i64, _i64, _i64, _vp, _i64, _vp, _int, _int, _int, _vp],

@@ -95,7 +95,7 @@ def flatten_named_tensors(named_tensors) -> FlattenedBucket:
 class _Layout:
     """Everything about a bucket that does not depend on where its inputs live this sync."""
     __slots__ = ("kind", "block", "group", "device", "metadata", "total_bytes", "n_tensors", "n_items", "table",
-                 "slot_src", "align", "const_base", "keepalive", "late_copies", "zero_bytes", "zp_rows", "zp_start",
+                 "table_off_lines", "slot_src", "align", "const_base", "keepalive", "late_copies", "zero_bytes", "zp_rows", "zp_start",
                  "zp_words", "n_zp", "fallback")
 
 
@@ -278,7 +278,7 @@ class BucketConverter:
         plan.late_copies = late
         plan.device = device
         plan.keepalive = []
-        plan.n_items, plan.table = 0, None
+        plan.n_items, plan.table, plan.table_off_lines = 0, None, None
         plan.zero_bytes, plan.n_zp = zero_off, len(zp_entries)
         if plan.fallback:
             return plan
@@ -332,9 +332,18 @@ class BucketConverter:
         if blocks:
             perm = torch.argsort(torch.cat(order), stable=True)
             table = torch.cat(blocks, dim=0)[perm].contiguous()
+            owner_all = torch.cat(owners)[perm]
             assert table.shape[1] == width
             plan.n_items = table.shape[0]
-            plan.table = ResolvedTable(table, torch.cat(owners)[perm], const_slot + 1, device)
+            if fp8:
+                # FP8 tiles whose code rows do not start on 64-byte boundaries of the buffer (an earlier tensor of the bucket
+                # left them there: back-to-back packing decides every address) go to the launch with plain stores, where
+                # the two tiles that share each 128-byte line get their halves merged in the L2
+                off_lines = (table[:, 5] != _lib.BUCKET_COPY_MARK) & (((table[:, 1] | table[:, 7]) & 63) != 0)
+                if bool(off_lines.any()):
+                    plan.table_off_lines = ResolvedTable(table[off_lines].contiguous(), owner_all[off_lines], const_slot + 1, device)
+                    table, owner_all = table[~off_lines].contiguous(), owner_all[~off_lines]
+            plan.table = ResolvedTable(table, owner_all, const_slot + 1, device) if table.shape[0] else None
             plan.slot_src = np.asarray(slot_src, dtype=np.int64)
             plan.align = np.asarray(align, dtype=np.int64)
         if zp_entries:
@@ -352,7 +361,10 @@ class BucketConverter:
         bases = arr[plan.slot_src]
         if np.any(bases & plan.align):
             return False
-        plan.table.resolve(np.append(bases, plan.const_base), tag=ptrs)
+        bases = np.append(bases, plan.const_base)
+        for table in (plan.table, plan.table_off_lines):
+            if table is not None:
+                table.resolve(bases, tag=ptrs)
         self.resolves += 1
         return True
 
@@ -386,15 +398,15 @@ class BucketConverter:
                 # back-to-back packing puts a tensor at an offset that is not a multiple of its element size:
                 # the per-parameter loop and a plain concatenation, exactly as the reference builds the buffer
                 return flatten_named_tensors(per_param_loop(self.args, params, self.config, self.transform_ue8m0))
-            if not plan.n_items or ptrs == plan.table.resolved_for or self._resolve(plan, ptrs):
+            if not plan.n_items or ptrs == (plan.table or plan.table_off_lines).resolved_for or self._resolve(plan, ptrs):
                 break
             plan = None                                  # an input lost the alignment the cached routing relied on
         device = plan.device
         if out is None:
             out = torch.empty(plan.total_bytes, dtype=torch.uint8, device=device)
         elif out.dtype != torch.uint8 or out.dim() != 1 or out.numel() < plan.total_bytes or not out.is_contiguous() \
-                or out.device != device or out.data_ptr() % 16:
-            raise ValueError(f"out must be a contiguous 16-byte aligned uint8 vector of at least {plan.total_bytes} bytes on {device}")
+                or out.device != device or out.data_ptr() % 128:
+            raise ValueError(f"out must be a contiguous 128-byte aligned uint8 vector of at least {plan.total_bytes} bytes on {device}")
         launches = 0
         if plan.n_items:
             lib = _lib.load()
@@ -403,8 +415,15 @@ class BucketConverter:
                 ev[0].record(torch.cuda.current_stream(device))
             with torch.cuda.device(device):
                 if plan.kind == "fp8":
-                    rc = lib.wq_fp8_bucket_convert(plan.table.items.data_ptr(), plan.n_items, out.data_ptr(), plan.block[0],
-                                                   plan.block[1], _lib.FP8_MODE_TRITON, _lib.stream_ptr(device))
+                    rc = 0
+                    if plan.table is not None:
+                        rc = lib.wq_fp8_bucket_convert(plan.table.items.data_ptr(), plan.table.n_items, out.data_ptr(),
+                                                       plan.block[0], plan.block[1], _lib.FP8_MODE_TRITON, _lib.stream_ptr(device))
+                    if rc == 0 and plan.table_off_lines is not None:
+                        rc = lib.wq_fp8_bucket_convert_rows_off_lines(
+                            plan.table_off_lines.items.data_ptr(), plan.table_off_lines.n_items, out.data_ptr(),
+                            plan.block[0], plan.block[1], _lib.FP8_MODE_TRITON, _lib.stream_ptr(device))
+                        launches += plan.table is not None
                 elif plan.kind == "int4_asym":
                     # the pack kernel leaves every group's zero point in a scratch buffer; a second launch packs them
                     # eight rows to a word into their place in the bucket

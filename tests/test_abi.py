@@ -220,6 +220,8 @@ def test_ue8m0_requests_are_not_ignored():
     assert lib_rc("wq_int4_dequant_any", None, None, 7, None, 4, 8, 8, None) == -3
     assert lib_rc("wq_int4_dequant_any", None, None, 0, None, 4, 8, 3, None) == -2
     assert lib_rc("wq_fp8_bucket_convert", None, 3, None, 128, 128, 1, None) == -1
+    assert lib_rc("wq_fp8_bucket_convert_rows_off_lines", None, 3, None, 128, 128, 1, None) == -1
+    assert lib_rc("wq_fp8_bucket_convert_rows_off_lines", None, 3, None, 128, 128, 9, None) == -3
     assert lib_rc("wq_int4_bucket_convert", None, 3, None, 48, None) == -4
     assert lib_rc("wq_delta_xor_noalloc", None, None, None, (4 << 30) + 1, 0, None, None) == -6
 

@@ -61,7 +61,7 @@ def test_fp8_bucket_equals_per_param_loop_and_oracle(cuda):
     out = conv.convert(params)
     want = B.per_param_loop(None, params, FP8_CFG)
     _same_as_loop(out, want)
-    assert out.launches == 1 and conv.plan_builds == 1
+    assert out.launches == 2 and conv.plan_builds == 1      # these small matrices leave their successors 32 bytes off a line (below)
     # every size here is a multiple of its successor's element size: the buffer is the plain concatenation
     assert torch.equal(out.get_flattened_tensor(), B.flatten_named_tensors(want).get_flattened_tensor())
     # quantised members against the CPU oracle (weight-sync arithmetic = mode 1)
@@ -289,3 +289,33 @@ def test_quantize_params_fp8_groups_one_parameter_into_one_launch(cuda):
         qo, so = C.fp8_block_quant(t.cpu(), (128, 128), 1)
         assert nq == n and ns == n.replace(".weight", ".weight_scale_inv")
         assert torch.equal(q.cpu().view(torch.uint8), qo) and torch.equal(s.cpu().view(torch.int32), so.view(torch.int32))
+
+
+def test_fp8_bucket_tensors_off_the_lines_take_the_plain_store_launch(cuda):
+    """Back-to-back packing decides where every tensor starts.  While code rows start on 64-byte boundaries the bucket is ONE
+    launch; a matrix whose scales are not a multiple of 64 bytes long (280 tiles here, the shape class of DeepSeek-V3's
+    [576, 7168] kv_a_proj_with_mqa) moves everything after it off the lines, and those tensors go through the launch with
+    plain stores - same bytes, two launches."""
+    name = lambda i: (L.format(0) + f"mlp.experts.linear_fc2.weight{i}", f"model.layers.0.mlp.experts.{i}.down_proj.weight")
+    friendly = [(name(i)[0], [(name(i)[1], I.weights(256, 2048, seed=40 + i).to(cuda))]) for i in range(3)]
+    conv = B.BucketConverter(None, FP8_CFG)
+    out = conv.convert(friendly)
+    assert out.launches == 1 and all(m.start_idx % 64 == 0 for m in out.metadata)
+    _same_as_loop(out, B.per_param_loop(None, friendly, FP8_CFG))
+    shifting = friendly[:1] + [(name(7)[0], [(name(7)[1], I.weights(576, 1024, seed=47).to(cuda))])] + friendly[1:]
+    out = conv.convert(shifting)
+    starts = [m.start_idx % 64 for m in out.metadata]
+    assert out.launches == 2 and starts[:4] == [0, 0, 0, 0] and starts[4] == 32          # 5 x 8 tiles: 160 bytes of scales
+    want = B.per_param_loop(None, shifting, FP8_CFG)
+    _same_as_loop(out, want)
+    named = dict(out.reconstruct_tensors())
+    for mn, cv in shifting:
+        for n, t in cv:
+            qo, so = C.fp8_block_quant(t.cpu(), (128, 128), 1)
+            assert torch.equal(named[n].cpu().view(torch.uint8), qo), n
+            assert torch.equal(named[n.replace(".weight", ".weight_scale_inv")].cpu().view(torch.int32), so.view(torch.int32)), n
+    # 8 bytes of a pass-through tensor ahead: every tile of the matrix is off the lines, the copy item stays in the first launch
+    ahead = [("module.module.x.pair", [("pair.f32", torch.ones(2, device=cuda))])] + friendly[:1]
+    out = conv.convert(ahead)
+    assert out.launches == 2 and out.metadata[1].start_idx == 8
+    _same_as_loop(out, B.per_param_loop(None, ahead, FP8_CFG))
