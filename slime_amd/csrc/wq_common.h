@@ -28,6 +28,23 @@ __device__ __forceinline__ uint32_t f2u(float f) { return __builtin_bit_cast(uin
 template <typename T> __device__ __forceinline__ T ldg_nt(const void* p) { return __builtin_nontemporal_load((const WQ_GLOBAL T*)p); }
 template <typename T> __device__ __forceinline__ T ldg(const void* p) { return *(const WQ_GLOBAL T*)p; }
 template <typename T> __device__ __forceinline__ void stg_nt(void* p, T v) { __builtin_nontemporal_store(v, (WQ_GLOBAL T*)p); }
+// The same with `sc1` next to `nt` (the compiler's non-temporal store emits `nt` only, hence the assembly; 4-, 8- and
+// 16-byte forms).  Which of the two streams faster depends on the kernel's read:write mix - measured per kernel, two
+// alternating pairs of builds in one session, % of HBM peak `nt` -> `nt sc1`: delta pass (1:1) 77.8 -> 82.1, QAT forward
+// (1:1) 79.8 -> 82.1, fake INT4 (1:1) 75.9-77.1 -> 77.4-78.5, FP8-aligned weight (1:1) 73.9 -> 75.0, block-FP8 quantiser (2:1)
+// 79.9-80.0 -> 80.6-81.4 and 76.2 -> 76.9 on the Qwen3-4B shapes; but INT4 packer (4:1) 81.5-82.3 -> 81.2-81.4, FP8 -> bf16
+// (1:2) 80.1 -> 79.6, INT4 -> bf16 (1:4) 79.0 -> 76.6, per-row FP8 77.3 -> 75.8.  Each kernel uses the one that won.
+template <typename T> __device__ __forceinline__ void stg_nt_sc1(void* p, T v)
+{
+    WQ_GLOBAL T* gp = (WQ_GLOBAL T*)p;
+    static_assert(sizeof(T) == 4 || sizeof(T) == 8 || sizeof(T) == 16, "dword, dwordx2 and dwordx4 stores");
+    if constexpr (sizeof(T) == 4) asm volatile("global_store_dword %0, %1, off nt sc1" :: "v"(gp), "v"(v) : "memory");
+    else if constexpr (sizeof(T) == 8) asm volatile("global_store_dwordx2 %0, %1, off nt sc1" :: "v"(gp), "v"(v) : "memory");
+    // A store of more than 8 bytes still reads its data registers after it has issued: a VALU instruction that overwrites
+    // them needs two wait states behind it on this family.  The compiler's hazard recogniser adds them for its own stores
+    // but does not look inside assembly (without them the FP8-aligned weight of a ragged matrix came out wrong).
+    else asm volatile("global_store_dwordx4 %0, %1, off nt sc1\n\ts_nop 1" :: "v"(gp), "v"(v) : "memory");
+}
 template <typename T> __device__ __forceinline__ void stg(void* p, T v) { *(WQ_GLOBAL T*)p = v; }
 
 // A dword holds two bf16: element 2k in the low half, 2k+1 in the high half.

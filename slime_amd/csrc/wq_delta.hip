@@ -139,8 +139,8 @@ __device__ __forceinline__ void delta_xor_chunk(const uint8_t* __restrict__ nw, 
         if (XXH3)
             xxh3_lane_terms(((uint64_t)a[i].y << 32) | a[i].x, ((uint64_t)a[i].w << 32) | a[i].z, k0, k1, xs0[i], xs1[i]);
         if (valid == 16) {
-            if (DIFF) stg_nt<u32x4>(diff + off, d);
-            if (UPDATE) stg_nt<u32x4>(old + off, a[i]);
+            if (DIFF) stg_nt_sc1<u32x4>(diff + off, d);
+            if (UPDATE) stg_nt_sc1<u32x4>(old + off, a[i]);
         } else if (valid > 0) {
             if (DIFF) store_tail(diff + off, d, valid);
             if (UPDATE) store_tail(old + off, a[i], valid);

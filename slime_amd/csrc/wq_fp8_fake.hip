@@ -122,7 +122,7 @@ __device__ __forceinline__ void fake_tile_vec128(const FakeArgs& a, int64_t tm, 
             const u32x2 hi = expand4(fp8_quant4_fast<MODE>(v[i].z, v[i].w, p), p.scale);
             const u32x4 o = {lo.x, lo.y, hi.x, hi.y};
             if (full || (col_ok && rb + kFakeRowSlots * i < rows))
-                stg_nt<u32x4>(yt + ((uint32_t)(rb + kFakeRowSlots * i) * yrow + (uint32_t)cc * 16u), o);
+                stg_nt_sc1<u32x4>(yt + ((uint32_t)(rb + kFakeRowSlots * i) * yrow + (uint32_t)cc * 16u), o);
         }
     } else {
         // NaN / Inf block (rare): the literal element functions; rows are re-read so that the register copy of the

@@ -149,7 +149,7 @@ __device__ __forceinline__ void quant_tile_vec128(const wq_fp8_quant_desc& d, in
             o.y = fp8_quant4_fast<MODE>(v[i].z, v[i].w, p);
             if (full || (col_ok && kRowSlots * i < rows_left)) {
                 if (PLAIN) stg<u32x2>(yt + (yoff + i * ystep), o);
-                else stg_nt<u32x2>(yt + (yoff + i * ystep), o);
+                else stg_nt_sc1<u32x2>(yt + (yoff + i * ystep), o);
             }
         }
     } else {

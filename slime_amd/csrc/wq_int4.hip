@@ -400,7 +400,7 @@ __global__ __launch_bounds__(256) void int4_fake_quant_vec_kernel(const uint16_t
             u32x4 r = {pack2_bf16_hw(o[0], o[1]), pack2_bf16_hw(o[2], o[3]), pack2_bf16_hw(o[4], o[5]),
                        pack2_bf16_hw(o[6], o[7])};
             if (restore_sign) r = (r & 0x7FFF7FFFu) | (v[i] & 0x80008000u);
-            stg_nt<u32x4>(q + g * (8 * L) + ll * 8, r);
+            stg_nt_sc1<u32x4>(q + g * (8 * L) + ll * 8, r);
             if (ll == 0) {
                 stg<uint16_t>(scale_out + g, (uint16_t)f32_to_bf16_bits(scale));
                 stg<uint16_t>(zero_out + g, (uint16_t)f32_to_bf16_bits(zero));

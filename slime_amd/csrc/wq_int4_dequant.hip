@@ -187,7 +187,7 @@ __global__ __launch_bounds__(256) void int4_fake_ste_kernel(const uint16_t* __re
         if (g < n_groups) {
             u32x4 r = {pack2_bf16(o[0], o[1]), pack2_bf16(o[2], o[3]), pack2_bf16(o[4], o[5]), pack2_bf16(o[6], o[7])};
             if (fast) r = (r & 0x7FFF7FFFu) | (v[i] & 0x80008000u);
-            stg_nt<u32x4>(y + g * (8 * L) + ll * 8, r);
+            stg_nt_sc1<u32x4>(y + g * (8 * L) + ll * 8, r);
         }
     }
 }
