@@ -1231,7 +1231,8 @@ def main():
     kernels = {}
     for key, name, profile, src in (("fp8", "fp8_block_quant_kernel<TORCH, per-tile descriptors>",
                                      "fp8_block_quant_qwen3_30b_a3b_state_dict.txt", "fp8_block_quant"),
-                                    ("int4", "int4_pack_kernel<128, per-item descriptors>",
+                                    ("int4", "int4_pack_kernel<128, per-item descriptors> (one call = ceil(items / 2^18) dispatches "
+                                             "over consecutive parts of the item table; kernel_ms is the call)",
                                      "int4_pack_qwen3_30b_a3b_experts.txt", "int4_pack")):
         k = r[key]
         achieved = k["algo_bytes"] / k["kernel_ms"] / 1e6      # GB/s
@@ -1253,11 +1254,11 @@ def main():
                                "[768,2048], down [2048,768] + q, k, v, o), N(0, 0.02) with rare x20 outliers), resident in "
                                f"HBM: block-FP8 128x128 quant of all {r['tensors_fp8']} linear weights (block_fp8 arithmetic "
                                f"as torch evaluates it on CPU tensors), then INT4 sym group-128 pack of the {r['tensors_int4']} "
-                               "expert weights; one grouped launch each",
+                               "expert weights; one call of the library each (the INT4 call is 14 dispatches of one kernel)",
                    "fp8_mode": r["fp8"]["mode"],
                    "fp8_mode_meaning": "WQ_FP8_MODE_TORCH (0): amax clamped at bf16(1e-12), scale = f32(amax) / 448, q = f32(x) / scale, "
                                        "both IEEE divisions - tools/convert_hf_to_fp8.py:41-75 on CPU tensors, what cpu_baseline computes",
-                   "launches_per_step": 2, "bf16_GB_fp8": 2 * r["fp8"]["elements"] / 1e9,
+                   "library_calls_per_step": 2, "bf16_GB_fp8": 2 * r["fp8"]["elements"] / 1e9,
                    "bf16_GB_int4": 2 * r["int4"]["elements"] / 1e9, "fp8_blocks": r["fp8"]["blocks"],
                    "parity_tensors_checked": r["parity_tensors_checked"]},
         "pct_hbm_peak": 100.0 * lower["frac"],
