@@ -114,3 +114,39 @@ def test_quantize_grouped_weights_argument_errors(cuda):
         slime_amd.quantize_grouped_weights([])
     q, s = slime_amd.quantize_grouped_weights([w[:0], w[:0]])
     assert q.shape == (2, 0, 256) and s.shape == (2, 0, 2)
+
+
+@pytest.mark.parametrize("mode", [0, 1, 2, 3])
+def test_few_tensor_launch_through_the_c_abi(cuda, mode):
+    """wq_fp8_block_quant_few: up to four descriptors in the kernel arguments - ragged and strided members, an empty one
+    in the middle, absolute output addresses (out_base NULL) and offsets from a base, every arithmetic mode."""
+    import ctypes
+
+    from slime_amd import _lib
+    from slime_amd.processors import _QuantDesc
+
+    ws = [I.weights(300, 520, seed=61), I.weights(128, 128, seed=62), I.weights(0, 256, seed=63), I.weights(264, 512, seed=64)[:, ::2]]
+    wg = [w.to(cuda) for w in ws[:3]] + [I.weights(264, 512, seed=64).to(cuda)[:, ::2]]
+    lib = _lib.load()
+    for with_base in (False, True):
+        outs, descs, off = [], (_QuantDesc * 4)(), 0
+        flat = torch.full((1 << 20,), 0xEE, dtype=torch.uint8, device=cuda)
+        for d, w in zip(descs, wg):
+            M, N = w.shape
+            tm, tn = -(-M // 128), -(-N // 128)
+            q0, s0 = off, (off + M * N + 127) // 128 * 128
+            off = (s0 + 4 * tm * tn + 127) // 128 * 128
+            base = 0 if with_base else flat.data_ptr()
+            d.x, d.y, d.s, d.M, d.N, d.sx_m, d.sx_n, d.sy_m = w.data_ptr() if M else 0, base + q0, base + s0, M, N, w.stride(0), w.stride(1), N
+            outs.append((q0, s0, M, N, tm, tn))
+        rc = lib.wq_fp8_block_quant_few(descs, 4, flat.data_ptr() if with_base else None, 128, 128, mode, _lib.stream_ptr(cuda))
+        _lib.check(rc, "few")
+        host = flat.cpu()
+        for w, (q0, s0, M, N, tm, tn) in zip(ws, outs):
+            if M == 0:
+                continue
+            qo, so = C.fp8_block_quant(w.contiguous(), (128, 128), mode)
+            assert torch.equal(host[q0:q0 + M * N].view(M, N), qo), (mode, with_base, M, N)
+            assert torch.equal(host[s0:s0 + 4 * tm * tn].clone().view(torch.int32).view(tm, tn), so.view(torch.int32)), (mode, with_base, M, N)
+        assert bool((host[off:] == 0xEE).all())
+    assert lib.wq_fp8_block_quant_few(descs, 5, None, 128, 128, mode, None) == -2
