@@ -319,3 +319,31 @@ def test_fp8_bucket_tensors_off_the_lines_take_the_plain_store_launch(cuda):
     out = conv.convert(ahead)
     assert out.launches == 2 and out.metadata[1].start_idx == 8
     _same_as_loop(out, B.per_param_loop(None, ahead, FP8_CFG))
+
+
+@pytest.mark.parametrize("width", [4, 5, 8])
+def test_resolve_items_through_the_c_abi(cuda, width):
+    """wq_bucket_resolve_items: items = template with bases[owner] added to word 0, nothing else touched."""
+    from slime_amd import _lib
+    from slime_amd._tables import ResolvedTable
+
+    g = I.gen(width)
+    n, n_bases = 10_007, 37
+    template = torch.randint(-2 ** 40, 2 ** 40, (n, width), generator=g, dtype=torch.int64)
+    owner = torch.randint(0, n_bases, (n,), generator=g, dtype=torch.int64)
+    bases = torch.randint(0, 2 ** 47, (n_bases,), generator=g, dtype=torch.int64)
+    want = template.clone()
+    want[:, 0] += bases[owner]
+    table = ResolvedTable(template, owner, n_bases, cuda)
+    table.resolve(bases.numpy(), tag="a")
+    assert torch.equal(table.items.cpu(), want) and torch.equal(table.template.cpu(), template) and table.resolved_for == "a"
+    other = bases + 4096                                        # the same inputs somewhere else: five resolves cycle the staging
+    for _ in range(5):
+        table.resolve(other.numpy(), tag="b")
+    want[:, 0] += 4096
+    assert torch.equal(table.items.cpu(), want) and table.resolves == 6
+    lib = _lib.load()
+    assert lib.wq_bucket_resolve_items(table.template.data_ptr(), table.owner.data_ptr(), table.bases.data_ptr(), n, width,
+                                       table.template.data_ptr(), None) == -4          # in place: refused
+    assert lib.wq_bucket_resolve_items(table.template.data_ptr(), table.owner.data_ptr(), table.bases.data_ptr(), n, 17,
+                                       table.items.data_ptr(), None) == -2
