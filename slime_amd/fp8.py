@@ -8,7 +8,8 @@ Function names, argument meaning, return layouts and error behaviour follow the 
 * ``weight_dequant``                                                - tools/fp8_cast_bf16.py:31-41
 * ``weight_dequant_bf16_scale``                                     - slime/backends/megatron_utils/hf_to_megatron/common.py:42-56
 
-All arithmetic runs in the HIP kernels of ``libslime_amd_wq.so``; inputs must live on the GPU.
+All arithmetic runs in the HIP kernels of ``libslime_amd_wq.so``.  Inputs live on the GPU; the three torch-formulated
+quantisers also take host tensors, as the reference's do, by way of the GPU (see ``_host_tensor_through_gpu``).
 ``Fp8QuantPlan`` / ``Fp8DequantPlan`` quantise many tensors with ONE kernel launch and write into
 one flat output buffer - the shape a weight-sync bucket wants.
 """
@@ -39,6 +40,19 @@ def _check_weight(w: torch.Tensor, what: str) -> None:
 
 
 _OTHER_FLOAT_DTYPES = {torch.float16: _lib.DTYPE_F16, torch.float32: _lib.DTYPE_F32}
+
+
+def _host_tensor_through_gpu(fn, weight: torch.Tensor, what: str, *args):
+    """The reference's ``block_fp8`` / ``channel_fp8`` / ``tensor_fp8`` are plain torch ops and take host tensors (its own
+    test, tests/test_block_fp8_zero_block.py, runs them on the CPU).  A host tensor is uploaded, quantised by the same
+    kernels in the arithmetic torch uses on CPU tensors - which is what the reference computes for such an input - and the
+    results are handed back on the host.  No GPU: RuntimeError, as for every entry point of the package."""
+    if not torch.cuda.is_available():
+        _lib.require_gpu(weight, what)
+    device = torch.device("cuda", torch.cuda.current_device())
+    with arith.torch_arithmetic("cpu"):
+        q, s = fn(weight.to(device), *args)
+    return q.cpu(), s.cpu()
 
 
 def _block_quant(w: torch.Tensor, bm: int, bn: int, mode: int, what: str):
@@ -73,7 +87,10 @@ def block_fp8(weight: torch.Tensor, block_size) -> tuple[torch.Tensor, torch.Ten
 
     Arithmetic of tools/convert_hf_to_fp8.py:41-75: zero padding of edge blocks, amax clamped at
     1e-12 in the weight dtype, scale = f32(amax)/448, q = clamp(f32(w)/scale), RNE to e4m3fn.  `/448` is
-    evaluated as torch does on GPU tensors unless ``arith.set_torch_arithmetic("cpu")`` is in force."""
+    evaluated as torch does on GPU tensors unless ``arith.set_torch_arithmetic("cpu")`` is in force.  A host tensor is
+    quantised on the GPU in the CPU evaluation and comes back on the host."""
+    if isinstance(weight, torch.Tensor) and not weight.is_cuda:
+        return _host_tensor_through_gpu(block_fp8, weight, "block_fp8", block_size)
     return _block_quant(weight, int(block_size[0]), int(block_size[1]), arith.fp8_torch_mode(), "block_fp8")
 
 
@@ -81,6 +98,8 @@ def channel_fp8(weight: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
     """Per-row scaling, tools/convert_hf_to_fp8.py:78-83 -> (qweight [M,N], scale float32 [M,1]).  bf16 rows take the
     bandwidth-tuned kernels; fp16 / fp32 weights are quantised as blocks of one row (the same arithmetic: both
     divide by a dimensioned float32 scale)."""
+    if isinstance(weight, torch.Tensor) and not weight.is_cuda:
+        return _host_tensor_through_gpu(channel_fp8, weight, "channel_fp8")
     if weight.dtype in _OTHER_FLOAT_DTYPES and weight.dim() == 2:
         return _block_quant(weight, 1, max(int(weight.shape[1]), 1), arith.fp8_torch_mode(), "channel_fp8")
     _check_weight(weight, "channel_fp8")
@@ -100,6 +119,8 @@ def tensor_fp8(weight: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
     """Per-tensor scaling, tools/convert_hf_to_fp8.py:86-91 -> (qweight [M,N], scale float32 [1]).  The quotient is
     rounded to the weight's dtype before the clamp, as torch's type promotion with a 0-dim scale makes it (bf16 and
     fp16 weights round twice, fp32 weights once); fp16 / fp32 weights take plain two-pass kernels."""
+    if isinstance(weight, torch.Tensor) and not weight.is_cuda:
+        return _host_tensor_through_gpu(tensor_fp8, weight, "tensor_fp8")
     other = weight.dtype in _OTHER_FLOAT_DTYPES and weight.dim() == 2
     if other:
         _lib.require_gpu(weight, "tensor_fp8")

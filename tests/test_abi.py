@@ -122,12 +122,17 @@ def test_cpu_tensors_are_refused():
     import slime_amd
 
     w = torch.zeros(128, 128, dtype=torch.bfloat16)
-    for fn in (lambda: slime_amd.block_fp8(w, (128, 128)), lambda: slime_amd.channel_fp8(w),
-               lambda: slime_amd.tensor_fp8(w), lambda: slime_amd.blockwise_cast_to_fp8_triton(w),
+    # what is a Triton kernel or a CUDA extension in the reference takes GPU tensors only, there and here
+    for fn in (lambda: slime_amd.blockwise_cast_to_fp8_triton(w),
                lambda: slime_amd.pack_layer(w, 128), lambda: slime_amd.fake_int4_quant_cuda(w, (1, 128), True),
                lambda: slime_amd.weight_dequant(w.view(torch.uint8)[:, :128].contiguous(), torch.ones(1, 1))):
         with pytest.raises(RuntimeError, match="GPU"):
             fn()
+    # the torch-formulated quantisers take host tensors like the reference's - by way of the GPU, so without one they refuse
+    if not torch.cuda.is_available():
+        for fn in (lambda: slime_amd.block_fp8(w, (128, 128)), lambda: slime_amd.channel_fp8(w), lambda: slime_amd.tensor_fp8(w)):
+            with pytest.raises(RuntimeError, match="GPU"):
+                fn()
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):

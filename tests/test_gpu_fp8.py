@@ -173,6 +173,37 @@ def test_reference_suite_invariants_on_gpu(cuda):
     assert not torch.isnan(q.float()).any() and (deq - w.float()).abs().max() < 0.5
 
 
+def test_reference_suite_on_host_tensors(cuda):
+    """The reference's own test file (tests/test_block_fp8_zero_block.py:38-75) hands CPU tensors to block_fp8.  Host tensors
+    go through the same kernels in the arithmetic torch uses on CPU tensors and come back on the host: the three cases of
+    that file verbatim, the bytes of the CPU oracle (mode 0), and the per-row / per-tensor forms."""
+    weight = torch.zeros(256, 256, dtype=torch.bfloat16)
+    weight[0, 0] = 1.0
+    qweight, scale = slime_amd.block_fp8(weight, (128, 128))
+    assert not qweight.is_cuda and not scale.is_cuda and qweight.dtype == torch.float8_e4m3fn
+    assert not torch.isnan(qweight.float()).any() and not torch.isinf(qweight.float()).any() and (scale > 0).all()
+    assert _bits32(scale)[0, 1].item() == 0x27212492                      # the zero-block scale of the CPU evaluation
+    qweight, scale = slime_amd.block_fp8(torch.zeros(128, 128, dtype=torch.bfloat16), (128, 128))
+    assert ((qweight.float() * scale.float()) == 0).all()
+    torch.manual_seed(0)
+    weight = torch.randn(256, 256, dtype=torch.float32).to(torch.bfloat16)
+    qweight, scale = slime_amd.block_fp8(weight, (128, 128))
+    dequantized = qweight.float() * scale.repeat_interleave(128, dim=0).repeat_interleave(128, dim=1).float()
+    assert not torch.isnan(qweight.float()).any() and (dequantized - weight.float()).abs().max() < 0.5
+    qo, so = C.fp8_block_quant(weight, (128, 128), 0)
+    assert torch.equal(_codes(qweight), qo) and torch.equal(_bits32(scale), _bits32(so))
+    w = I.weights(37, 520, seed=4)
+    for fn, ora in ((slime_amd.channel_fp8, C.fp8_channel_quant), (slime_amd.tensor_fp8, C.fp8_tensor_quant)):
+        q, s = fn(w)
+        qo, so = ora(w, 0)
+        assert not q.is_cuda and torch.equal(_codes(q), qo) and torch.equal(_bits32(s), _bits32(so))
+    q, s = slime_amd.quant_fp8(w, "block", (128, 128))
+    assert not q.is_cuda and tuple(s.shape) == (1, 5)
+    assert slime_amd.get_torch_arithmetic() == "device"                     # the caller's setting is untouched
+    with pytest.raises(RuntimeError, match="GPU"):
+        slime_amd.blockwise_cast_to_fp8_triton(w)                           # a Triton kernel in the reference: GPU tensors only
+
+
 @pytest.mark.parametrize("shape", [(64, 256), (3, 1000), (257, 129), (1024, 2560), (7, 7168), (130, 9728), (5, 20000),
                                    (33, 8200), (1, 8), (300, 16384), (2, 16392)])
 def test_channel_and_tensor_quant(cuda, shape):
