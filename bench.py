@@ -1017,6 +1017,19 @@ def bench_copy(dev, steps, warmup, nbytes=4 << 30):
         assert torch.equal(dst[:piece], want)
         rec[f"compute_free_{ratio}_to_1"] = {"bytes_read": nbytes, "bytes_written": n_out, "kernel_ms": f_ms, "kernel_ms_min": f_min,
                                               "hbm_frac": (nbytes + n_out) / f_ms / 1e6 / HBM_PEAK_GBS}
+    # and for the dequantisers' mixes: compute-free 1:2 and 1:4 streams (1 GiB read, 2 / 4 GiB written)
+    n_in = nbytes // 4
+    for ratio in (2, 4):
+
+        def expand():
+            _lib.check(wq_testlib.load().wq_stream_expand_bytes(src.data_ptr(), dst.data_ptr(), n_in, ratio, _lib.stream_ptr(dev)), "expand")
+
+        _, x_ms, x_min = _time_launches(expand, steps, warmup)
+        head = dst[:ratio * 4096].view(torch.int32).view(ratio, 1024)
+        first = src[:4096].view(torch.int32)
+        assert all(torch.equal(head[w], first + w) for w in range(ratio))
+        rec[f"compute_free_1_to_{ratio}"] = {"bytes_read": n_in, "bytes_written": ratio * n_in, "kernel_ms": x_ms, "kernel_ms_min": x_min,
+                                              "hbm_frac": (1 + ratio) * n_in / x_ms / 1e6 / HBM_PEAK_GBS}
     return rec
 
 
@@ -1284,14 +1297,16 @@ def main():
         # config 5's streaming leg: host-resident weights, PCIe-bound by construction (never part of `value`)
         extras["host_resident_stream"] = bench_stream(dev, args.stream_buckets, args.stream_bucket_mib << 20,
                                                       not args.stream_no_download)
-        # the practical ceilings of 1:1, 2:1 and 4:1 read:write streams on this very box, measured in this very run
+        # the practical ceilings of 1:1, 2:1, 4:1, 1:2 and 1:4 read:write streams on this very box, measured in this very run
         cal = bench_copy(dev, args.steps, args.warmup)
         extras["copy_kernel_calibration"] = cal
         line["roofline"]["same_run_compute_free_streams"] = {
             "note": "fraction of the 8 TB/s peak that kernels with no arithmetic reach on this box in this run: plain copy, and the "
-                    "block-FP8 quantiser's (2:1) and the INT4 packer's (4:1) read:write mix over contiguous 16-32 KiB pieces",
+                    "block-FP8 quantiser's (2:1) and the INT4 packer's (4:1) read:write mix over contiguous 16-32 KiB pieces, and "
+                    "the FP8 (1:2) and INT4 (1:4) dequantisers' mixes",
             "copy_1_to_1": cal["hbm_frac"], "fold_2_to_1": cal["compute_free_2_to_1"]["hbm_frac"],
-            "fold_4_to_1": cal["compute_free_4_to_1"]["hbm_frac"]}
+            "fold_4_to_1": cal["compute_free_4_to_1"]["hbm_frac"], "expand_1_to_2": cal["compute_free_1_to_2"]["hbm_frac"],
+            "expand_1_to_4": cal["compute_free_1_to_4"]["hbm_frac"]}
         line["other_workloads"] = extras
     # The CPU baseline runs last: its thread pool keeps spinning for a while after each parallel region, which slows
     # the launch-bound legs above (the per-parameter loop) when they run after it.

@@ -47,6 +47,11 @@ int wq_copy_bytes(const void *src, void *dst, int64_t n_bytes, void *stream);
  * memory system gives that mix on the box at hand. */
 int wq_stream_fold_bytes(const void *src, void *dst, int64_t n_out_bytes, int reads_per_write, void *stream);
 
+/* The mirror image for the dequantisers' mixes: `writes_per_read` (2 or 4) bytes written per byte read - FP8 -> bf16 and
+ * INT4 -> bf16.  Output piece w (of writes_per_read) of every 4 KiB input piece is the input with w added to each dword.
+ * n_in_bytes a multiple of 16384; dst holds writes_per_read * n_in_bytes. */
+int wq_stream_expand_bytes(const void *src, void *dst, int64_t n_in_bytes, int writes_per_read, void *stream);
+
 /* An empty kernel over `workgroups` workgroups of `threads` lanes: what a launch costs on the box at hand before any
  * byte moves (dispatch, wave start-up, completion), the floor under every small launch. */
 int wq_empty_launch(int64_t workgroups, int threads, void *stream);

@@ -179,6 +179,26 @@ __global__ __launch_bounds__(256) void fold_kernel(const u32x4* __restrict__ src
     }
 }
 
+// The mirror image for the dequantisers: a compute-free stream with W bytes written per byte read (W = 2: FP8 -> bf16,
+// W = 4: INT4 -> bf16).  An item is STEPS x 4 KiB of input; output piece w of input piece i is the input with w added to
+// every dword, so every output byte depends on the data.
+template <int W, int STEPS>
+__global__ __launch_bounds__(256) void expand_kernel(const u32x4* __restrict__ src, u32x4* __restrict__ dst, int64_t items)
+{
+    const int64_t slot = (int64_t)blockIdx.x + (int64_t)blockIdx.y * gridDim.x;
+    if (slot >= items) return;
+    const int64_t item = xcd_chunked_item(slot, items, kFoldItemsPerXcdRun);
+    const u32x4* in = src + item * (STEPS * 256) + threadIdx.x;
+    u32x4 v[STEPS];
+#pragma unroll
+    for (int i = 0; i < STEPS; ++i) v[i] = __builtin_nontemporal_load(in + i * 256);
+    u32x4* out = dst + item * (W * STEPS * 256) + threadIdx.x;
+#pragma unroll
+    for (int i = 0; i < STEPS; ++i)
+#pragma unroll
+        for (int w = 0; w < W; ++w) __builtin_nontemporal_store(v[i] + (uint32_t)w, out + (i * W + w) * 256);
+}
+
 __global__ void empty_kernel() {}
 
 }  // namespace wq
@@ -292,6 +312,31 @@ WQ_EXPORT int wq_empty_launch(int64_t workgroups, int threads, void* stream)
 {
     if (workgroups <= 0 || workgroups > (1ll << 30) || threads <= 0 || threads > 1024) return WQ_ERR_SHAPE;
     empty_kernel<<<grid_for_items(workgroups), threads, 0, (hipStream_t)stream>>>();
+    WQ_LAUNCH_CHECK();
+    return WQ_OK;
+}
+
+// Launch shapes by measurement (% of the 8 TB/s HBM peak, 2 GiB read; input pieces per lane x workgroups per CU):
+// 1:2 - 2x2 83.6 (used), 1x4 83.1, 2x3 80.5, 1x8 78.9, 1x2 61, 4x2 78.2;  1:4 - 1x3 79.5 (used), 2x2 75.9, 1x4 75.5, 4x3 73.0,
+// 1x8 71.8.  With the dequantiser's own access pattern (8-byte loads, one 16-byte store per load) the 1:2 stream gives the
+// same 82.4-82.6 at two workgroups per CU and 76-78 at five.
+constexpr int kExpandSteps2 = 2, kExpandSteps4 = 1;
+constexpr unsigned kExpandPadBytes2 = 77 * 1024, kExpandPadBytes4 = 50 * 1024;
+WQ_EXPORT int wq_stream_expand_bytes(const void* src, void* dst, int64_t n_in_bytes, int writes_per_read, void* stream)
+{
+    if (n_in_bytes < 0 || (n_in_bytes % 16384)) return WQ_ERR_SHAPE;
+    if (writes_per_read != 2 && writes_per_read != 4) return WQ_ERR_MODE;
+    if (n_in_bytes == 0) return WQ_OK;
+    if (!src || !dst) return WQ_ERR_NULL;
+    if (((uintptr_t)src & 15) || ((uintptr_t)dst & 15)) return WQ_ERR_ALIGN;
+    hipStream_t st = (hipStream_t)stream;
+    if (writes_per_read == 2) {
+        const int64_t items = n_in_bytes / (kExpandSteps2 * 4096);
+        expand_kernel<2, kExpandSteps2><<<grid_for_items(items), 256, kExpandPadBytes2, st>>>((const u32x4*)src, (u32x4*)dst, items);
+    } else {
+        const int64_t items = n_in_bytes / (kExpandSteps4 * 4096);
+        expand_kernel<4, kExpandSteps4><<<grid_for_items(items), 256, kExpandPadBytes4, st>>>((const u32x4*)src, (u32x4*)dst, items);
+    }
     WQ_LAUNCH_CHECK();
     return WQ_OK;
 }

@@ -78,6 +78,23 @@ def test_fold_stream_kernel(cuda, ratio, piece):
     assert lib.wq_stream_fold_bytes(src.data_ptr() + 8, dst.data_ptr(), n_out, ratio, None) == -5   # alignment
 
 
+@pytest.mark.parametrize("writes", [2, 4])
+def test_expand_stream_kernel(cuda, writes):
+    """The compute-free 1:W stream (the dequantisers' mixes): output piece w of every 4 KiB input piece is the input with w added
+    to each dword."""
+    g = torch.Generator().manual_seed(writes)
+    n_in = 16384 * 37
+    src = torch.randint(-2 ** 31, 2 ** 31 - 1, (n_in // 4,), generator=g, dtype=torch.int32).cuda()
+    dst = torch.zeros(writes * n_in // 4, dtype=torch.int32, device="cuda")
+    lib = wq_testlib.load()
+    _lib.check(lib.wq_stream_expand_bytes(src.data_ptr(), dst.data_ptr(), n_in, writes, torch.cuda.current_stream().cuda_stream), "expand")
+    want = src.view(-1, 1, 1024) + torch.arange(writes, dtype=torch.int32, device="cuda").view(1, writes, 1)
+    assert torch.equal(dst, want.reshape(-1))
+    assert lib.wq_stream_expand_bytes(src.data_ptr(), dst.data_ptr(), n_in, 3, None) == -3           # mode
+    assert lib.wq_stream_expand_bytes(src.data_ptr(), dst.data_ptr(), n_in + 4096, writes, None) == -2  # shape
+    assert lib.wq_stream_expand_bytes(src.data_ptr() + 8, dst.data_ptr(), n_in, writes, None) == -5   # alignment
+
+
 def test_empty_launch(cuda):
     lib = wq_testlib.load()
     _lib.check(lib.wq_empty_launch(1024, 256, torch.cuda.current_stream().cuda_stream), "empty launch")

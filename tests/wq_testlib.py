@@ -23,6 +23,7 @@ SIGNATURES = {
     "wq_selftest_decode_fp8": [_vp, _vp],
     "wq_copy_bytes": [_vp, _vp, _i64, _vp],
     "wq_stream_fold_bytes": [_vp, _vp, _i64, _int, _vp],
+    "wq_stream_expand_bytes": [_vp, _vp, _i64, _int, _vp],
     "wq_empty_launch": [_i64, _int, _vp],
 }
 
