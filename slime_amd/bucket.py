@@ -397,16 +397,20 @@ class BucketConverter:
             if plan.fallback:
                 # back-to-back packing puts a tensor at an offset that is not a multiple of its element size:
                 # the per-parameter loop and a plain concatenation, exactly as the reference builds the buffer
-                return flatten_named_tensors(per_param_loop(self.args, params, self.config, self.transform_ue8m0))
+                flat = flatten_named_tensors(per_param_loop(self.args, params, self.config, self.transform_ue8m0))
+                if out is None:
+                    return flat
+                self._check_out(out, plan.total_bytes, plan.device)
+                out[:plan.total_bytes].copy_(flat.get_flattened_tensor())
+                return FlattenedBucket(out[:plan.total_bytes], flat.get_metadata(), flat.launches + 1)
             if not plan.n_items or ptrs == (plan.table or plan.table_off_lines).resolved_for or self._resolve(plan, ptrs):
                 break
             plan = None                                  # an input lost the alignment the cached routing relied on
         device = plan.device
         if out is None:
             out = torch.empty(plan.total_bytes, dtype=torch.uint8, device=device)
-        elif out.dtype != torch.uint8 or out.dim() != 1 or out.numel() < plan.total_bytes or not out.is_contiguous() \
-                or out.device != device or out.data_ptr() % 128:
-            raise ValueError(f"out must be a contiguous 128-byte aligned uint8 vector of at least {plan.total_bytes} bytes on {device}")
+        else:
+            self._check_out(out, plan.total_bytes, device)
         launches = 0
         if plan.n_items:
             lib = _lib.load()
@@ -446,6 +450,12 @@ class BucketConverter:
         if plan.late_copies:
             launches += self._late(plan, params, out)
         return FlattenedBucket(out[:plan.total_bytes], plan.metadata, launches)
+
+    @staticmethod
+    def _check_out(out, total_bytes, device) -> None:
+        if out.dtype != torch.uint8 or out.dim() != 1 or out.numel() < total_bytes or not out.is_contiguous() \
+                or out.device != device or out.data_ptr() % 128:
+            raise ValueError(f"out must be a contiguous 128-byte aligned uint8 vector of at least {total_bytes} bytes on {device}")
 
     def kernel_ms(self) -> float:
         """Sum of the launch times recorded while ``time_kernels`` was set (call after a synchronize); clears the list."""

@@ -347,3 +347,95 @@ def test_resolve_items_through_the_c_abi(cuda, width):
                                        table.template.data_ptr(), None) == -4          # in place: refused
     assert lib.wq_bucket_resolve_items(table.template.data_ptr(), table.owner.data_ptr(), table.bases.data_ptr(), n, 17,
                                        table.items.data_ptr(), None) == -2
+
+
+def _random_bucket(seed, cuda, int4):
+    """A bucket of random composition: expert / dense / attention weights of ragged and aligned shapes (row-chunk views of a
+    fused parameter, now and then a strided or transposed view, a float16 or float32 weight, an empty one), 1-D members of
+    odd lengths between them (they move their successors off the 16-byte and 128-byte grids) and fp32 router weights."""
+    g = torch.Generator().manual_seed(seed)
+    r = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))
+    pick = lambda xs: xs[r(0, len(xs) - 1)]
+    # mostly shapes that keep the bucket on the one-launch kernels (INT4: rows a multiple of 8 for the zero points; FP8: a
+    # multiple of 4 codes so that the fp32 scales behind them can be addressed), now and then one that does not
+    cols = [128, 256, 384, 512, 1024] if int4 else [128, 200, 256, 384, 520, 1000, 2052, 132, 4100] + [7, 2049] * (r(0, 5) == 0)
+    rows = [8, 128, 136, 256, 304, 512, 1000] + ([1, 7, 129, 513] if not int4 or r(0, 7) == 0 else [])
+    params = []
+    for k in range(r(3, 14)):
+        layer, kind = r(0, 3), r(0, 9)
+        hf, mc = f"model.layers.{layer}.", L.format(layer)
+        w = lambda: I.weights(pick(rows), pick(cols), seed=seed * 100 + k).to(cuda)
+        if kind <= 3:                                             # an expert's fused fc1 -> gate, up; or its fc2
+            e = r(0, 7)
+            if r(0, 1):
+                fc1 = I.weights(2 * pick(rows), pick(cols), seed=seed * 100 + k).to(cuda)
+                gate, up = fc1.chunk(2, dim=0)
+                params.append((mc + f"mlp.experts.linear_fc1.weight{e}", [(hf + f"mlp.experts.{e}.gate_proj.weight", gate),
+                                                                         (hf + f"mlp.experts.{e}.up_proj.weight", up)]))
+            else:
+                params.append((mc + f"mlp.experts.linear_fc2.weight{e}", [(hf + f"mlp.experts.{e}.down_proj.weight", w())]))
+        elif kind == 4:
+            params.append((mc + "self_attention.linear_proj.weight", [(hf + "self_attn.o_proj.weight", w())]))
+        elif kind == 5:                                           # a dense MLP weight in another dtype, or a view with strides
+            t = w()
+            how = r(0, 4)
+            if how == 0 and not int4: t = t.float()
+            elif how == 1 and not int4: t = t.half()
+            elif how == 2 and not int4 and t.shape[1] >= 16: t = t[:, 4:t.shape[1] - 4]
+            elif how == 3 and not int4: t = t.t()
+            params.append((mc + "mlp.linear_fc2.weight", [(hf + "mlp.down_proj.weight", t)]))
+        elif kind == 6:
+            params.append((mc + "mlp.router.weight", [(hf + "mlp.gate.weight", I.weights(r(1, 9), pick(cols), seed=k).to(cuda).float())]))
+        elif kind == 7:                                           # a 1-D member of odd length: bf16, fp32 or fp16
+            v = I.weights(1, r(1, 301) * pick([1, 2, 8]), seed=k)[0].to(cuda)
+            params.append((mc + "self_attention.linear_qkv.layer_norm_weight", [(hf + "input_layernorm.weight", pick([v, v.float(), v.half()]))]))
+        elif kind == 8:
+            params.append((f"module.module.x.empty{k}", [(f"empty{k}", torch.empty(0, pick(cols), device=cuda, dtype=torch.bfloat16))]))
+        else:
+            params.append((f"module.module.x.pass{k}", [(f"model.pass{k}.weight", w().t() if r(0, 1) and not int4 else w())]))
+    return params
+
+
+def _same_bytes_as_loop(bucket, want):
+    """Buffer and metadata equal the plain concatenation of the loop's tensors; members read back where torch can view them
+    (an offset that is no multiple of a member's element size cannot be viewed, in the reference's bucket class either)."""
+    ref = B.flatten_named_tensors(want)
+    assert bucket.get_metadata() == ref.get_metadata()
+    assert torch.equal(bucket.get_flattened_tensor(), ref.get_flattened_tensor())
+    if all(m.start_idx % torch.empty(0, dtype=m.dtype).element_size() == 0 for m in ref.get_metadata()):
+        _same_as_loop(bucket, want)
+
+
+RANDOM_CFGS = {"fp8": FP8_CFG, "fp8_64x32": {**FP8_CFG, "weight_block_size": [64, 32]}, "int4": INT4_CFG,
+               "int4_asym": {**INT4_CFG, "config_groups": {"group_0": {"weights": {"group_size": 128, "symmetric": False}}}},
+               "int4_g32": {**INT4_CFG, "config_groups": {"group_0": {"weights": {"group_size": 32, "symmetric": True}}}}}
+
+
+@pytest.mark.parametrize("seed", range(10))
+@pytest.mark.parametrize("cfg", list(RANDOM_CFGS))
+def test_random_buckets_equal_the_per_param_loop(cuda, cfg, seed):
+    """Buckets of random composition: first sync, second sync on the cached layout, third sync with every input at a new
+    address, fourth into the caller's buffer - each identical to the per-parameter loop, also where that loop refuses
+    (a weight whose columns are no multiple of the INT4 group)."""
+    qcfg = RANDOM_CFGS[cfg]
+    params = _random_bucket(seed, cuda, cfg.startswith("int4"))
+    conv = B.BucketConverter(None, qcfg)
+    try:
+        want = B.per_param_loop(None, params, qcfg)
+    except Exception as e:
+        with pytest.raises(type(e)):
+            conv.convert(params, bucket_id=seed)
+        return
+    _same_bytes_as_loop(conv.convert(params, bucket_id=seed), want)
+    _same_bytes_as_loop(conv.convert(params, bucket_id=seed), want)
+    pad = [torch.empty(r, device=cuda) for r in (3, 17, 33)]                # moves the clones off the originals' alignment pattern
+    moved = [(mn, [(n, t.clone(memory_format=torch.preserve_format) if t.is_contiguous() else t) for n, t in cv]) for mn, cv in params]
+    _same_bytes_as_loop(conv.convert(moved, bucket_id=seed), want)
+    del pad
+    if want:
+        total = conv.convert(params, bucket_id=seed).get_flattened_tensor().numel()
+        buf = torch.empty(total + 128, dtype=torch.uint8, device=cuda)
+        buf = buf[(-buf.data_ptr()) % 128:][:total]
+        out = conv.convert(params, out=buf, bucket_id=seed)
+        assert out.get_flattened_tensor().data_ptr() == buf.data_ptr()
+        _same_bytes_as_loop(out, want)
