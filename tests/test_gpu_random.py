@@ -210,11 +210,105 @@ def case_delta(seed, cuda):
     assert torch.equal(old_gpu.cpu(), new if update else old), (n, dtype, update)
 
 
+# ---------------------------------------------------------------------------------- one launch over many tensors
+# The many-tensor forms against the per-tensor functions above (which the first half of this file holds to the oracle):
+# lists short enough for the searched descriptors and long enough for the per-item tables, ragged members, repeats.
+
+
+def _weight_list(d, cuda, cols, rows, lo=1, hi=90):
+    n = d.pick([d.r(lo, 6), d.r(lo, hi)])
+    return [d.values(d.pick(rows), d.pick(cols), torch.bfloat16).nan_to_num(0.0, 1.0, -1.0).to(cuda) for _ in range(n)]
+
+
+def case_fp8_plans(seed, cuda):
+    d = Draw(seed)
+    ws = _weight_list(d, cuda, [128, 256, 384, 200, 520, 7, 1000], [1, 7, 128, 129, 256, 300])
+    if d.r(0, 2) == 0:
+        ws[0] = d.strided(ws[0].cpu(), cuda)[1]
+    block = d.pick([(128, 128), (128, 128), (64, 32), (100, 60)])
+    mode = d.pick([0, 1, 2])
+    outs = slime_amd.Fp8QuantPlan(ws, block, mode).run()
+    for k, (w, (q, s)) in enumerate(zip(ws, outs)):
+        if mode == 1:
+            qo, so = slime_amd.blockwise_cast_to_fp8_triton(w, block)
+        else:
+            with slime_amd.torch_arithmetic({0: "cpu", 2: "device"}[mode]):
+                qo, so = slime_amd.block_fp8(w, block)
+        assert torch.equal(q.view(torch.uint8), qo.view(torch.uint8)) and I.same_bits(s, so), (k, tuple(w.shape), block, mode)
+    if block[0] == block[1]:
+        out_dtype = d.pick([torch.bfloat16, torch.float32])
+        ys = slime_amd.Fp8DequantPlan([q for q, _ in outs], [s for _, s in outs], block[0], 0, out_dtype).run()
+        for k, ((q, s), y) in enumerate(zip(outs, ys)):
+            assert I.same_bits(y, slime_amd.block_quant_dequant(q, s, list(block), out_dtype)), (k, tuple(q.shape), block, out_dtype)
+
+
+def case_int4_plans(seed, cuda):
+    d = Draw(seed)
+    group = d.pick([128, 128, 64, 32])
+    sym = bool(d.r(0, 1))
+    ws = _weight_list(d, cuda, [group * k for k in (1, 2, 3, 8, 11)], [8, 16, 128, 136, 304] + ([1, 7, 129] if sym else []))
+    outs = slime_amd.Int4PackPlan(ws, group, sym).run()
+    for k, (w, got) in enumerate(zip(ws, outs)):
+        want = [v for v in slime_amd.pack_layer(w, group, sym) if v is not None]
+        assert len(got) == len(want) and all(I.same_bits(a, b) for a, b in zip(got, want)), (k, tuple(w.shape), group, sym)
+    if sym:
+        ys = slime_amd.Int4DequantPlan([o[0] for o in outs], [o[1] for o in outs], [w.shape for w in ws], group).run()
+        for k, (w, o, y) in enumerate(zip(ws, outs, ys)):
+            assert I.same_bits(y, slime_amd.dequantize_int4(o[0], o[1], w.shape, group)), (k, tuple(w.shape), group)
+    many = slime_amd.fake_int4_quantization_ste_many(ws, group)
+    plan = slime_amd.Int4StePlan(ws, group).run()
+    for k, (w, a, b) in enumerate(zip(ws, many, plan)):
+        want = slime_amd.fake_int4_quantization_ste(w, group)
+        assert I.same_bits(a, want) and I.same_bits(b, want), (k, tuple(w.shape), group)
+
+
+def case_grouped_weights(seed, cuda):
+    """The stacked form of a grouped linear's experts, twice: the second time every expert lives somewhere else."""
+    d = Draw(seed)
+    M, N = d.pick([128, 256, 384, 200, 7]), d.pick([128, 256, 520, 1000, 132])
+    E = d.r(1, 12)
+    block = d.pick([(128, 128), (128, 128), (64, 32)])
+    ue8m0 = block == (128, 128) and bool(d.r(0, 1))
+    for sync in range(2):
+        ws = [d.values(M, N, torch.bfloat16).nan_to_num(0.0, 1.0, -1.0).to(cuda) for _ in range(E)]
+        if d.r(0, 1):                                   # chunk views of one fused tensor
+            ws = list(torch.cat(ws, dim=0).chunk(E, dim=0))
+        q, s = slime_amd.quantize_grouped_weights(ws, block, ue8m0)
+        for e, w in enumerate(ws):
+            qo, so = slime_amd.quant_weight_ue8m0(w, block) if ue8m0 else slime_amd.blockwise_cast_to_fp8_triton(w, block)
+            assert torch.equal(q[e].view(torch.uint8), qo.view(torch.uint8)) and I.same_bits(s[e], so), (sync, e, M, N, E, block, ue8m0)
+
+
+def case_delta_many(seed, cuda):
+    d = Draw(seed)
+    n = d.pick([d.r(1, 5), d.r(1, 80)])
+    news, olds = [], []
+    for _ in range(n):
+        nbytes = d.pick([d.r(1, 64), d.r(1, 70000), 256 * d.r(1, 300), 16384 * d.r(1, 8)])
+        new = torch.randint(0, 256, (nbytes,), generator=d.g, dtype=torch.int32).to(torch.uint8)
+        old = new.clone()
+        if d.r(0, 2):
+            old[torch.randint(0, nbytes, (max(1, nbytes // d.pick([2, 100, 10000])),), generator=d.g)] ^= 0xA5
+        news.append(new.to(cuda))
+        olds.append(old.to(cuda))
+    want = [slime_amd.delta.xor_diff(a, b.clone()) for a, b in zip(news, olds)]
+    diffs, results = slime_amd.delta.xor_diff_many(news, [o.clone() for o in olds])
+    plan = slime_amd.delta.XorDiffPlan(news, [o.clone() for o in olds], xxh3=True)
+    p_diffs, p_results = plan.run(update_snapshot=True)
+    digests = plan.hexdigests()
+    for k, (dw, rw) in enumerate(want):
+        assert torch.equal(diffs[k], dw) and torch.equal(results[k], rw), (k, n)
+        assert torch.equal(p_diffs[k], dw) and torch.equal(p_results[k], rw) and torch.equal(plan.olds[k], news[k]), (k, n)
+        changed = int(rw[0])
+        assert digests[k] == (slime_amd.delta.xxh3_128(news[k]) if changed else None), (k, n)
+
+
 CASES = {"fp8_block": case_fp8_block, "fp8_row_tensor": case_fp8_row_tensor, "fp8_dequant": case_fp8_dequant, "int4": case_int4,
-         "fake_int4": case_fake_int4, "delta": case_delta}
+         "fake_int4": case_fake_int4, "delta": case_delta, "fp8_plans": case_fp8_plans, "int4_plans": case_int4_plans,
+         "grouped_weights": case_grouped_weights, "delta_many": case_delta_many}
 
 
-@pytest.mark.parametrize("seed", range(24))
+@pytest.mark.parametrize("seed", range(16))
 @pytest.mark.parametrize("kind", list(CASES))
 def test_random_case(cuda, kind, seed):
     CASES[kind](seed, cuda)
