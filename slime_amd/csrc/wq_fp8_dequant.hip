@@ -51,7 +51,7 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float a, float b)
 template <int MODE>
 __device__ __forceinline__ float load_scale(const float* __restrict__ s, int64_t idx)
 {
-    float v = s[idx];
+    float v = ldg<float>(s + idx);      // never a flat access: see the note at the element-wise path below
     if (MODE == WQ_DEQ_MODE_BF16SCALE) v = u2f(f32_to_bf16_bits(v) << 16);
     return v;
 }
@@ -176,7 +176,9 @@ __global__ __launch_bounds__(256) void fp8_block_dequant_kernel(const DeqArgs a,
             }
         }
     } else {
-        // element-wise path: any N, alignment and block size
+        // element-wise path: any N, alignment and block size.  Global-address-space accesses like everywhere else: a flat
+        // (generic-pointer) access anywhere in the kernel makes the compiler drain every outstanding memory operation
+        // (vmcnt(0)) at each wait of the vector path above, which then sends its four stores one round trip at a time.
 #pragma nounroll
         for (int i = 0; i < kSteps; ++i) {
             if (seg0 + 4 * i >= n_segs) break;
@@ -186,11 +188,11 @@ __global__ __launch_bounds__(256) void fp8_block_dequant_kernel(const DeqArgs a,
                 if (cc >= N) break;
                 const float sc = load_scale<MODE>(d.s, (r / block) * kt + cc / block);
                 const uint64_t off = (uint64_t)r * N + cc;
-                const uint32_t code = x[off];
+                const uint32_t code = ldg<uint8_t>(x + off);
                 const f32x2 f = __builtin_amdgcn_cvt_pk_f32_fp8((int)code, false);
-                if (OUT == WQ_DTYPE_BF16) ((uint16_t*)d.y)[off] = (uint16_t)(pack_bf16x2(f.x * sc, 0.0f) & 0xFFFFu);
-                else if (OUT == WQ_DTYPE_F16) ((uint16_t*)d.y)[off] = (uint16_t)(pack_f16x2(f.x * sc, 0.0f) & 0xFFFFu);
-                else ((float*)d.y)[off] = f.x * sc;
+                if (OUT == WQ_DTYPE_BF16) stg<uint16_t>((uint16_t*)d.y + off, (uint16_t)(pack_bf16x2(f.x * sc, 0.0f) & 0xFFFFu));
+                else if (OUT == WQ_DTYPE_F16) stg<uint16_t>((uint16_t*)d.y + off, (uint16_t)(pack_f16x2(f.x * sc, 0.0f) & 0xFFFFu));
+                else stg<float>((float*)d.y + off, f.x * sc);
             }
             c += 4;
             while (c >= spr) { c -= spr; ++r; }

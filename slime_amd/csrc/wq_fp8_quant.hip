@@ -167,6 +167,9 @@ __device__ __forceinline__ void quant_tile_vec128(const wq_fp8_quant_desc& d, in
     }
 }
 
+// Every access goes through the global-address-space helpers, here too: one flat (generic-pointer) access anywhere in a
+// kernel makes the compiler wait for ALL outstanding memory operations (vmcnt(0)) wherever it waits for one, in the vector
+// path as well - its rolling load window then drains after every second load.
 template <int MODE>
 __device__ __forceinline__ void quant_tile_generic(const wq_fp8_quant_desc& d, int64_t tm, int64_t tn, int kt,
                                                    int bm, int bn, uint32_t* lds)
@@ -178,7 +181,7 @@ __device__ __forceinline__ void quant_tile_generic(const wq_fp8_quant_desc& d, i
     uint32_t m = 0;
     for (int e = threadIdx.x; e < n; e += blockDim.x) {
         int i = e / cols, j = e - i * cols;
-        m = max(m, (uint32_t)x[(r0 + i) * d.sx_m + (c0 + j) * d.sx_n] & 0x7FFFu);
+        m = max(m, (uint32_t)ldg<uint16_t>(x + ((r0 + i) * d.sx_m + (c0 + j) * d.sx_n)) & 0x7FFFu);
     }
     m = wave64_max_u32(m);
     if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6] = m;
@@ -186,12 +189,12 @@ __device__ __forceinline__ void quant_tile_generic(const wq_fp8_quant_desc& d, i
     m = 0;
     for (int w = 0; w < kTileWaves; ++w) m = max(m, lds[w]);
     const Fp8BlockParams p = fp8_block_params<MODE>(m);
-    if (threadIdx.x == 0) d.s[tm * kt + tn] = p.scale;
+    if (threadIdx.x == 0) stg<float>(d.s + (tm * kt + tn), p.scale);
     uint8_t* y = (uint8_t*)d.y;
     for (int e = threadIdx.x; e < n; e += blockDim.x) {
         int i = e / cols, j = e - i * cols;
-        float xv = u2f((uint32_t)x[(r0 + i) * d.sx_m + (c0 + j) * d.sx_n] << 16);
-        y[(r0 + i) * d.sy_m + (c0 + j)] = (uint8_t)fp8_quant1_exact<MODE>(xv, p);
+        float xv = u2f((uint32_t)ldg<uint16_t>(x + ((r0 + i) * d.sx_m + (c0 + j) * d.sx_n)) << 16);
+        stg<uint8_t>(y + ((r0 + i) * d.sy_m + (c0 + j)), (uint8_t)fp8_quant1_exact<MODE>(xv, p));
     }
 }
 

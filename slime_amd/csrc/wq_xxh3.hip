@@ -141,15 +141,15 @@ __device__ void xxh3_short(const uint8_t* p, int n, uint64_t& out_low, uint64_t&
         out_low = xxh64_avalanche(secret64(64) ^ secret64(72));
         out_high = xxh64_avalanche(secret64(80) ^ secret64(88));
     } else if (n <= 3) {
-        const uint32_t lo = ((uint32_t)p[0] << 16) | ((uint32_t)p[n >> 1] << 24) | (uint32_t)p[n - 1] | ((uint32_t)n << 8);
+        const uint32_t lo = ((uint32_t)ldg<uint8_t>(p) << 16) | ((uint32_t)ldg<uint8_t>(p + (n >> 1)) << 24) | (uint32_t)ldg<uint8_t>(p + n - 1) | ((uint32_t)n << 8);
         const uint32_t sw = __builtin_bswap32(lo), hi = (sw << 13) | (sw >> 19);
         out_low = xxh64_avalanche((uint64_t)lo ^ (uint64_t)(secret32(0) ^ secret32(4)));
         out_high = xxh64_avalanche((uint64_t)hi ^ (uint64_t)(secret32(8) ^ secret32(12)));
     } else if (n <= 8) {
         uint32_t a = 0, b = 0;
         for (int k = 0; k < 4; ++k) {
-            a |= (uint32_t)p[k] << (8 * k);
-            b |= (uint32_t)p[n - 4 + k] << (8 * k);
+            a |= (uint32_t)ldg<uint8_t>(p + k) << (8 * k);
+            b |= (uint32_t)ldg<uint8_t>(p + n - 4 + k) << (8 * k);
         }
         const uint64_t keyed = ((uint64_t)a + ((uint64_t)b << 32)) ^ (secret64(16) ^ secret64(24));
         const uint64_t mult = kP64_1 + ((uint64_t)n << 2);
@@ -212,7 +212,7 @@ __device__ __forceinline__ wq_xxh3_desc chain_view(const wq_xxh3_desc& d, bool& 
 // after a delta pass: the digest of a tensor that did not change is not wanted (nothing is published for it)
 __device__ __forceinline__ wq_xxh3_desc chain_view(const wq_delta_desc& d, bool& skip)
 {
-    skip = d.result[0] == 0;
+    skip = ldg<uint64_t>(d.result) == 0;
     return wq_xxh3_desc{d.new_bytes, d.n, d.xxh3_sums, d.xxh3_digest};
 }
 
@@ -225,15 +225,15 @@ __global__ __launch_bounds__(64) void xxh3_chain_kernel(const Desc single, const
     const wq_xxh3_desc d = chain_view(descs ? descs[t] : single, skip);
     const int lane = threadIdx.x, i = lane & 7;
     if (skip) {                               // uniform per wavefront
-        if (lane < 2) d.digest[lane] = 0;
+        if (lane < 2) stg<uint64_t>(d.digest + lane, 0);
         return;
     }
     if (d.n <= 240) {                         // uniform per wavefront
         if (lane == 0) {
             uint64_t low, high;
             xxh3_short((const uint8_t*)d.data, (int)d.n, low, high);
-            d.digest[0] = low;
-            d.digest[1] = high;
+            stg<uint64_t>(d.digest, low);
+            stg<uint64_t>(d.digest + 1, high);
         }
         return;
     }
@@ -254,7 +254,7 @@ __global__ __launch_bounds__(64) void xxh3_chain_kernel(const Desc single, const
     if (nb > 0) {
         constexpr int U = 8, DEPTH = 8;
         uint64_t ring[DEPTH][U];
-        acc += s[0];
+        acc += ldg<uint64_t>(s);
         const uint64_t* rest = s + 8;          // sums[1 ..]
         const int64_t m = nb - 1;
         int64_t k = 0;
@@ -262,14 +262,14 @@ __global__ __launch_bounds__(64) void xxh3_chain_kernel(const Desc single, const
 #pragma unroll
             for (int b = 0; b < DEPTH; ++b)
 #pragma unroll
-                for (int u = 0; u < U; ++u) ring[b][u] = rest[(b * U + u) * 8];
+                for (int u = 0; u < U; ++u) ring[b][u] = ldg<uint64_t>(rest + (b * U + u) * 8);
             for (; k + 2 * DEPTH * U <= m; k += DEPTH * U) {
 #pragma unroll
                 for (int b = 0; b < DEPTH; ++b) {
 #pragma unroll
                     for (int u = 0; u < U; ++u) acc = scramble_then_add(acc, scramble_key, ring[b][u]);
 #pragma unroll
-                    for (int u = 0; u < U; ++u) ring[b][u] = rest[(k + (DEPTH + b) * U + u) * 8];
+                    for (int u = 0; u < U; ++u) ring[b][u] = ldg<uint64_t>(rest + (k + (DEPTH + b) * U + u) * 8);
                 }
             }
 #pragma unroll
@@ -278,7 +278,7 @@ __global__ __launch_bounds__(64) void xxh3_chain_kernel(const Desc single, const
                 for (int u = 0; u < U; ++u) acc = scramble_then_add(acc, scramble_key, ring[b][u]);
             k += DEPTH * U;
         }
-        for (; k < m; ++k) acc = scramble_then_add(acc, scramble_key, rest[k * 8]);
+        for (; k < m; ++k) acc = scramble_then_add(acc, scramble_key, ldg<uint64_t>(rest + k * 8));
         acc = scramble_then_add(acc, scramble_key, 0);
     }
 
@@ -309,8 +309,8 @@ __global__ __launch_bounds__(64) void xxh3_chain_kernel(const Desc single, const
             high += mul128_fold64(all[2 * j] ^ secret64(192 - kXxhStripe - 11 + 16 * j),
                                   all[2 * j + 1] ^ secret64(192 - kXxhStripe - 11 + 16 * j + 8));
         }
-        d.digest[0] = avalanche(low);
-        d.digest[1] = avalanche(high);
+        stg<uint64_t>(d.digest, avalanche(low));
+        stg<uint64_t>(d.digest + 1, avalanche(high));
     }
 }
 

@@ -39,7 +39,7 @@ __device__ __forceinline__ uint64_t load64_bytes(const uint8_t* p)
 {
     uint64_t v = 0;
 #pragma unroll
-    for (int b = 0; b < 8; ++b) v |= (uint64_t)p[b] << (8 * b);
+    for (int b = 0; b < 8; ++b) v |= (uint64_t)ldg<uint8_t>(p + b) << (8 * b);
     return v;
 }
 

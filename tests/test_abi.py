@@ -256,6 +256,37 @@ def test_no_mixed_precision_fma_in_the_dequantiser(tmp_path):
     assert "v_cvt_f16_f32" in asm and "fma_mix" not in asm and "mad_mix" not in asm
 
 
+def test_no_flat_memory_instruction_in_any_kernel(tmp_path):
+    """Every device access goes through a global-address-space pointer.  A pointer that a kernel reads from a descriptor
+    table is a generic one to the compiler; one access through it (flat_load / flat_store) is enough for the compiler to
+    stop counting outstanding loads in that kernel and wait for all of them (s_waitcnt vmcnt(0)) wherever it waits for
+    one - rolling load windows drain after every load and stores go out one round trip at a time.  This compiles every
+    kernel source to assembly with the library's own flags and checks that no flat memory instruction is in it."""
+    import concurrent.futures
+    import glob
+    import re
+    import shutil
+    import subprocess
+
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(hipcc):
+        pytest.skip("no hipcc")
+    csrc = os.path.join(ROOT, "slime_amd", "csrc")
+    flags = re.search(r"^HIPFLAGS \?= (.*?)\n(?!\s)", open(os.path.join(csrc, "Makefile")).read(), re.S | re.M).group(1)
+    flags = flags.replace("\\\n", " ").replace("$(ARCH)", "gfx950").split()
+
+    def flat_instructions(src):
+        out = tmp_path / (os.path.basename(src) + ".s")
+        subprocess.check_call([hipcc, *flags, "-S", "--cuda-device-only", "-o", str(out), src], stderr=subprocess.DEVNULL)
+        return src, re.findall(r"^\s*(flat_\w+)", out.read_text(), re.M)
+
+    sources = sorted(glob.glob(os.path.join(csrc, "*.hip")))
+    assert len(sources) >= 9
+    with concurrent.futures.ThreadPoolExecutor(max_workers=4) as pool:
+        for src, found in pool.map(flat_instructions, sources):
+            assert not found, f"{os.path.basename(src)}: {len(found)} flat memory instructions ({sorted(set(found))})"
+
+
 def test_product_never_touches_the_oracle_or_falls_back_to_the_host():
     """The package must not import, load or run anything under oracle/ (test infrastructure), and its entry points must
     refuse to work without the HIP library rather than compute on the host."""
